@@ -1,0 +1,482 @@
+"""HIP code generator: EpilogueIR + tile configuration -> one kernel module.
+
+Replaces the un-vendored CUTLASS Python emitter that the reference drives
+through `plan.compile(...)` / `operation.epilogue_type(visitor_args)`
+(python/gtl/compiler/passes/evt_fuser.py:515-518, :539-546).  The generated
+translation unit instantiates the hand-written main loop
+(csrc/evt_gemm.hpp) with an `Epi` struct whose `tile()` is straight-line code
+over the accumulator registers, and exports the C ABI of include/evt_amd.h.
+"""
+from __future__ import annotations
+
+import json
+from dataclasses import dataclass, asdict
+from typing import Dict, List
+
+from .ir import DTYPE_CTYPES, REDUCE_STATE, EpilogueIR, Node
+
+
+@dataclass(frozen=True)
+class TileConfig:
+    """Workgroup tile of the main loop (the analogue of the reference tuner's
+    (threadblock shape, stages, warp count, swizzle) tuple,
+    python/gtl/compiler/autotuner/gemm_tuner.py:31-44)."""
+    bm: int = 256
+    bn: int = 256
+    bk: int = 64
+    wm: int = 4
+    wn: int = 2
+    stages: int = 2
+    dma: bool = True
+    group_m: int = 4
+
+    def tag(self) -> str:
+        return (f"{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_s{self.stages}"
+                f"_{'dma' if self.dma else 'safe'}_g{self.group_m}")
+
+    def lds_bytes(self) -> int:
+        return self.stages * (self.bm + self.bn) * self.bk * 2
+
+
+@dataclass(frozen=True)
+class KernelSpec:
+    a_kc: bool          # A contiguous along K (row-major [M, K])
+    b_kc: bool          # B contiguous along K (column-major, i.e. stored [N, K])
+    bf16: bool
+    tile: TileConfig
+
+
+_BINARY = {
+    "add": "({a} + {b})", "sub": "({a} - {b})", "mul": "({a} * {b})",
+    "div": "__fdividef({a}, {b})", "max": "fmaxf({a}, {b})", "min": "fminf({a}, {b})",
+    "tanh_backward": "evt::op_tanh_backward({a}, {b})",
+    "gelu_backward_tanh": "evt::op_gelu_backward_tanh({a}, {b})",
+    "gelu_backward_erf": "evt::op_gelu_backward_erf({a}, {b})",
+    "ge": "(({a} >= {b}) ? 1.f : 0.f)", "gt": "(({a} > {b}) ? 1.f : 0.f)",
+    "le": "(({a} <= {b}) ? 1.f : 0.f)", "lt": "(({a} < {b}) ? 1.f : 0.f)",
+    "ne": "(({a} != {b}) ? 1.f : 0.f)", "eq": "(({a} == {b}) ? 1.f : 0.f)",
+}
+_UNARY = {
+    "neg": "(-{a})", "exp": "evt::op_exp({a})", "log": "evt::op_log({a})",
+    "sqrt": "sqrtf({a})", "rsqrt": "rsqrtf({a})", "abs": "fabsf({a})", "rcp": "evt::op_rcp({a})",
+    "gelu_tanh": "evt::op_gelu_tanh({a})", "gelu_erf": "evt::op_gelu_erf({a})",
+    "tanh": "evt::op_tanh({a})", "relu": "evt::op_relu({a})", "sigmoid": "evt::op_sigmoid({a})",
+    "cast_f16": "evt::round_to<evt::f16>({a})", "cast_bf16": "evt::round_to<evt::bf16>({a})",
+    "cast_f32": "({a})", "cast_bool": "(({a} != 0.f) ? 1.f : 0.f)", "cast_int": "truncf({a})",
+}
+
+_IDENTITY = {"sum": "0.f", "max": "-INFINITY"}
+
+
+def _cname(name: str) -> str:
+    return "v_" + "".join(ch if ch.isalnum() else "_" for ch in name)
+
+
+class _Emitter:
+    def __init__(self):
+        self.lines: List[str] = []
+        self.ind = 0
+
+    def __call__(self, text: str = ""):
+        for line in text.split("\n"):
+            self.lines.append(("  " * self.ind + line) if line else "")
+
+    def indent(self):
+        self.ind += 1
+
+    def dedent(self):
+        self.ind -= 1
+
+    def text(self) -> str:
+        return "\n".join(self.lines) + "\n"
+
+
+class Codegen:
+    def __init__(self, ir: EpilogueIR, spec: KernelSpec, module_name: str):
+        self.ir = ir
+        self.spec = spec
+        self.name = module_name
+        # variance of every node: does it vary along m / along n?
+        self.var_m: Dict[str, bool] = {}
+        self.var_n: Dict[str, bool] = {}
+        for n in ir.nodes.values():
+            if n.op in ("accum",):
+                vm, vn = True, True
+            elif n.op == "colidx":
+                vm, vn = False, True
+            elif n.op == "load":
+                st = ir.slots[n.slot].strides
+                vm = st.stride_m != 0 or st.stride_l != 0
+                vn = st.stride_n != 0
+                # a batch-dependent value is re-read per row slot only if it also
+                # depends on m; a pure batch scalar is workgroup-uniform
+                vm = st.stride_m != 0
+            elif n.op in ("imm", "rres"):
+                vm, vn = False, False
+            else:
+                vm = any(self.var_m[i] for i in n.inputs)
+                vn = any(self.var_n[i] for i in n.inputs)
+            self.var_m[n.name], self.var_n[n.name] = vm, vn
+
+    # -- expression helpers ---------------------------------------------------
+    def ref(self, name: str, idx: str = "ni") -> str:
+        return f"{_cname(name)}[{idx}]" if self.var_n[name] else _cname(name)
+
+    def expr(self, n: Node, idx: str = "ni") -> str:
+        a = [self.ref(i, idx) for i in n.inputs]
+        if n.op in _BINARY:
+            return _BINARY[n.op].format(a=a[0], b=a[1])
+        if n.op in _UNARY:
+            return _UNARY[n.op].format(a=a[0])
+        if n.op == "where":
+            return f"(({a[0]} != 0.f) ? {a[1]} : {a[2]})"
+        raise NotImplementedError(n.op)
+
+    def slot_off(self, k: int, batch: str = "t.batch") -> str:
+        return f"(int64_t)({batch} / p.t{k}_ld) * p.t{k}_sl"
+
+    # -- sections ---------------------------------------------------------------
+    def emit_params(self, e: _Emitter):
+        e("struct Params {")
+        e.indent()
+        for k, s in enumerate(self.ir.slots):
+            const = "const " if s.role == "load" else ""
+            e(f"{const}{DTYPE_CTYPES[s.dtype]}* t{k};  // {s.role} {s.kind} '{s.name}'")
+            e(f"int64_t t{k}_sl, t{k}_sm, t{k}_sn; int t{k}_ld; int t{k}_vec;")
+        e(f"float s[{max(1, len(self.ir.scalars))}];")
+        e.dedent()
+        e("};")
+
+    def emit_combine(self, e: _Emitter, axis: str):
+        e(f"static EVT_DEV void {axis}_combine(float* a, const float* b) {{")
+        e.indent()
+        for r in self.ir.reduces.values():
+            if r.axis != axis:
+                continue
+            o = r.state_offset
+            if r.kind == "sum":
+                e(f"a[{o}] += b[{o}];")
+            elif r.kind == "max":
+                e(f"a[{o}] = fmaxf(a[{o}], b[{o}]);")
+            elif r.kind == "maxsumexp":
+                e(f"evt::combine_maxsumexp(a[{o}], a[{o + 1}], b[{o}], b[{o + 1}]);")
+            elif r.kind == "welford":
+                e(f"evt::combine_welford(a[{o}], a[{o + 1}], a[{o + 2}], b[{o}], b[{o + 1}], b[{o + 2}]);")
+        e("(void)a; (void)b;")
+        e.dedent()
+        e("}")
+
+    def emit_finalize(self, e: _Emitter, axis: str):
+        idx = "row" if axis == "row" else "col"
+        stride = "sm" if axis == "row" else "sn"
+        e(f"static EVT_DEV void {axis}_finalize(const Params& p, int batch, int {idx}, const float* st) {{")
+        e.indent()
+        stores = [s for s in self.ir.stores if s.domain == axis]
+        for name in self.ir.closure([s.input for s in stores]):
+            n = self.ir.nodes[name]
+            c = _cname(name)
+            if n.op == "imm":
+                e(f"const float {c} = p.s[{n.slot}];")
+            elif n.op == "rres":
+                r = self.ir.reduces[n.reduce]
+                e(f"const float {c} = st[{r.state_offset + n.comp}];")
+            elif n.op == "load":
+                k = n.slot
+                e(f"const float {c} = evt::ld_f32(p.t{k}, {self.slot_off(k, 'batch')} + (int64_t){idx} * p.t{k}_{stride});")
+            else:
+                a = [_cname(i) for i in n.inputs]
+                if n.op in _BINARY:
+                    ex = _BINARY[n.op].format(a=a[0], b=a[1])
+                elif n.op in _UNARY:
+                    ex = _UNARY[n.op].format(a=a[0])
+                elif n.op == "where":
+                    ex = f"(({a[0]} != 0.f) ? {a[1]} : {a[2]})"
+                else:
+                    raise NotImplementedError(f"{n.op} in a per-{axis} expression")
+                e(f"const float {c} = {ex};")
+        for s in stores:
+            k = s.slot
+            e(f"evt::st_f32(p.t{k}, {self.slot_off(k, 'batch')} + (int64_t){idx} * p.t{k}_{stride}, {_cname(s.input)});")
+        e("(void)p; (void)batch; (void)st;")
+        e.dedent()
+        e("}")
+
+    def emit_tile(self, e: _Emitter):
+        ir = self.ir
+        tile_stores = [s for s in ir.stores if s.domain == "tile"]
+        row_reds = [r for r in ir.reduces.values() if r.axis == "row"]
+        col_reds = [r for r in ir.reduces.values() if r.axis == "col"]
+        roots = [s.input for s in tile_stores] + [r.input for r in ir.reduces.values()]
+        need = ir.closure(roots)
+        hoisted = [n for n in need if not self.var_m[n]]
+        inner = [n for n in need if self.var_m[n]]
+
+        e("template <class Cfg, class Tile>")
+        e("static EVT_DEV void tile(const Params& p, const Tile& t, const evt::f32x16 (&acc)[Cfg::MI][Cfg::NI]) {")
+        e.indent()
+        e("constexpr int MI = Cfg::MI, NI = Cfg::NI;")
+        if row_reds or col_reds:
+            e("__syncthreads();  // all waves are done reading the last operand tile from LDS")
+        # hoisted values
+        for name in hoisted:
+            self.emit_node(e, ir.nodes[name], hoisted=True)
+        if col_reds:
+            e(f"float cst[NI][{ir.col_state}];")
+            e("#pragma unroll")
+            e("for (int ni = 0; ni < NI; ++ni) {")
+            e.indent()
+            for r in col_reds:
+                e(f"cst[ni][{r.state_offset}] = {_IDENTITY[r.kind]};")
+            e.dedent()
+            e("}")
+        e("#pragma unroll")
+        e("for (int mi = 0; mi < MI; ++mi) {")
+        e.indent()
+        e("#pragma unroll")
+        e("for (int v = 0; v < 16; ++v) {")
+        e.indent()
+        e("const int row = t.row(mi, v);")
+        e("const bool rok = row < t.M;")
+        for name in inner:
+            self.emit_node(e, ir.nodes[name], hoisted=False)
+        for s in tile_stores:
+            k = s.slot
+            src = s.input
+            if not self.var_n[src]:
+                e(f"float b_{k}[NI];")
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) b_{k}[ni] = {_cname(src)};")
+                arr = f"b_{k}"
+            else:
+                arr = _cname(src)
+            e(f"evt::aux_store(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
+              f"p.t{k}_sn, p.t{k}_vec != 0, rok, {arr});")
+        if row_reds:
+            e(f"float rst[{ir.row_state}];")
+            for r in row_reds:
+                self.emit_row_reduce(e, r)
+            e(f"evt::row_state_to_lds<Cfg, {ir.row_state}>(t, mi, v, rst);")
+        for r in col_reds:
+            x = lambda: self.ref(r.input)  # noqa: E731
+            o = r.state_offset
+            e("#pragma unroll")
+            e("for (int ni = 0; ni < NI; ++ni) {")
+            e.indent()
+            if r.kind == "sum":
+                e(f"cst[ni][{o}] += (rok && t.col_ok(ni)) ? {x()} : 0.f;")
+            else:
+                e(f"cst[ni][{o}] = (rok && t.col_ok(ni)) ? fmaxf(cst[ni][{o}], {x()}) : cst[ni][{o}];")
+            e.dedent()
+            e("}")
+        e.dedent()
+        e("}")
+        e.dedent()
+        e("}")
+        if row_reds:
+            e("evt::row_reduce_finish<Cfg, Epi>(p, t);")
+        if col_reds:
+            e("evt::col_reduce_finish<Cfg, Epi>(p, t, cst);")
+        e("(void)p; (void)t; (void)acc;")
+        e.dedent()
+        e("}")
+
+    def emit_node(self, e: _Emitter, n: Node, hoisted: bool):
+        c = _cname(n.name)
+        vn = self.var_n[n.name]
+        if n.op == "imm":
+            e(f"const float {c} = p.s[{n.slot}];")
+        elif n.op == "accum":
+            e(f"float {c}[NI];")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = acc[mi][ni][v];")
+        elif n.op == "colidx":
+            e(f"float {c}[NI];")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = (float)t.col(ni);")
+        elif n.op == "load":
+            k = n.slot
+            s = self.ir.slots[k]
+            base = self.slot_off(k)
+            if s.kind == "aux":
+                e(f"float {c}[NI];")
+                e(f"evt::aux_load(t, p.t{k}, {base} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
+                  f"p.t{k}_sn, p.t{k}_vec != 0, rok, {c});")
+            elif s.kind == "row":
+                e(f"float {c}[NI];")
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = t.col_ok(ni) ? "
+                  f"evt::ld_f32(p.t{k}, {base} + (int64_t)t.col(ni) * p.t{k}_sn) : 0.f;")
+            elif s.kind == "col":
+                if hoisted:   # depends on the batch only
+                    e(f"const float {c} = evt::ld_f32(p.t{k}, {base});")
+                else:
+                    e(f"const float {c} = rok ? evt::ld_f32(p.t{k}, {base} + (int64_t)row * p.t{k}_sm) : 0.f;")
+            else:
+                e(f"const float {c} = evt::ld_f32(p.t{k}, 0);")
+        elif n.op == "rres":
+            raise NotImplementedError("reduction result used per element")
+        else:
+            if vn:
+                e(f"float {c}[NI];")
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = {self.expr(n)};")
+            else:
+                e(f"const float {c} = {self.expr(n)};")
+
+    def emit_row_reduce(self, e: _Emitter, r):
+        o = r.state_offset
+        vn = self.var_n[r.input]
+        x = self.ref(r.input)
+        e("{")
+        e.indent()
+        if not vn:
+            # value constant along n: materialise so the generic code applies
+            e(f"float xv[NI];\n#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) xv[ni] = {x};")
+            x = "xv[ni]"
+        if r.kind == "sum":
+            e("float part = 0.f;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) part += t.col_ok(ni) ? {x} : 0.f;")
+            e(f"rst[{o}] = evt::half_wave_sum(part);")
+        elif r.kind == "max":
+            e("float part = -INFINITY;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) part = t.col_ok(ni) ? fmaxf(part, {x}) : part;")
+            e(f"rst[{o}] = evt::half_wave_max(part);")
+        elif r.kind == "maxsumexp":
+            e("float mx = -INFINITY;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) mx = t.col_ok(ni) ? fmaxf(mx, {x}) : mx;")
+            e("mx = evt::half_wave_max(mx);")
+            e("float se = 0.f;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) se += t.col_ok(ni) ? evt::op_exp({x} - mx) : 0.f;")
+            e(f"rst[{o}] = mx; rst[{o + 1}] = evt::half_wave_sum(se);")
+        elif r.kind == "welford":
+            e("const float cnt = (float)t.wave_cols();")
+            e("float sx = 0.f;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) sx += t.col_ok(ni) ? {x} : 0.f;")
+            e("sx = evt::half_wave_sum(sx);")
+            e("const float mean = cnt > 0.f ? sx / cnt : 0.f;")
+            e("float sq = 0.f;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {{ const float d = {x} - mean; sq += t.col_ok(ni) ? d * d : 0.f; }}")
+            e(f"rst[{o}] = cnt; rst[{o + 1}] = mean; rst[{o + 2}] = evt::half_wave_sum(sq);")
+        e.dedent()
+        e("}")
+
+    # -- module -------------------------------------------------------------------
+    def module_spec(self) -> dict:
+        t = self.spec.tile
+        return {
+            "abi": 1,
+            "name": self.name,
+            "tile": asdict(t),
+            "a_k_contiguous": self.spec.a_kc,
+            "b_k_contiguous": self.spec.b_kc,
+            "element": "bf16" if self.spec.bf16 else "f16",
+            "batched": self.ir.batched,
+            "row_state": self.ir.row_state,
+            "col_state": self.ir.col_state,
+            "tensors": [{"name": s.name, "role": s.role, "dtype": s.dtype, "kind": s.kind,
+                         "domain": s.domain} for s in self.ir.slots],
+            "num_scalars": len(self.ir.scalars),
+        }
+
+    def source(self) -> str:
+        ir, sp, t = self.ir, self.spec, self.spec.tile
+        e = _Emitter()
+        e("// Generated by evt_ae_amd.codegen -- do not edit.")
+        e(f"// module {self.name}")
+        e('#include "evt_epilogue.hpp"')
+        e('#include "evt_amd.h"')
+        e("")
+        e("namespace {")
+        e("struct Epi {")
+        e.indent()
+        e(f"static constexpr int ROW_STATE = {ir.row_state};")
+        e(f"static constexpr int COL_STATE = {ir.col_state};")
+        self.emit_params(e)
+        self.emit_combine(e, "row")
+        self.emit_combine(e, "col")
+        self.emit_finalize(e, "row")
+        self.emit_finalize(e, "col")
+        self.emit_tile(e)
+        e.dedent()
+        e("};")
+        b = lambda x: "true" if x else "false"  # noqa: E731
+        e(f"using Cfg = evt::GemmCfg<{t.bm}, {t.bn}, {t.bk}, {t.wm}, {t.wn}, {b(sp.a_kc)}, {b(sp.b_kc)}, "
+          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}>;")
+        e(f"constexpr int kNumTensors = {len(ir.slots)};")
+        e(f"constexpr int kNumScalars = {len(ir.scalars)};")
+        red_lds = 0
+        if ir.row_state:
+            red_lds += t.wn * t.bm * ir.row_state * 4 + 16
+        if ir.col_state:
+            red_lds += t.wm * t.bn * ir.col_state * 4 + 16
+        e(f"static_assert(Cfg::LDS_BYTES >= {red_lds}, \"reduction exchange area exceeds the operand LDS\");")
+        e("")
+        e("int fill(const EvtArgs* a, evt::GemmArgs& g, Epi::Params& p) {")
+        e.indent()
+        e("if (!a || !a->A || !a->B) return EVT_ERR_BAD_ARGS;")
+        e("if (a->num_tensors != kNumTensors || a->num_scalars != kNumScalars) return EVT_ERR_BAD_ARGS;")
+        e("if (a->M <= 0 || a->N <= 0 || a->K <= 0 || a->L <= 0) return EVT_ERR_BAD_ARGS;")
+        e("g.M = a->M; g.N = a->N; g.K = a->K; g.L = a->L;")
+        e("g.A = (const char*)a->A; g.lda = a->lda; g.bsA = a->batch_stride_A;")
+        e("g.B = (const char*)a->B; g.ldb = a->ldb; g.bsB = a->batch_stride_B;")
+        e("g.tiles_m = (a->M + Cfg::BM - 1) / Cfg::BM;")
+        e("g.tiles_n = (a->N + Cfg::BN - 1) / Cfg::BN;")
+        e("g.workspace = nullptr;")
+        e("if ((int64_t)g.tiles_m * g.tiles_n * a->L > 0x7fffffffLL) return EVT_ERR_RANGE;")
+        e("if (a->N > (1 << 24)) return EVT_ERR_RANGE;   // column indices are carried as fp32")
+        if t.dma:
+            e("// fast path: 16-byte global->LDS transfers, buffer range check for the tails")
+            e("if (((uintptr_t)a->A | (uintptr_t)a->B) & 15) return EVT_ERR_ALIGNMENT;")
+            e("if ((a->lda | a->ldb | a->batch_stride_A | a->batch_stride_B) & 7) return EVT_ERR_ALIGNMENT;")
+            if sp.a_kc:
+                e("if (a->K & 7) return EVT_ERR_ALIGNMENT;")
+                e("if ((int64_t)Cfg::BM * a->lda * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
+            else:
+                e("if (a->M & 7) return EVT_ERR_ALIGNMENT;")
+                e("if ((int64_t)Cfg::BK * a->lda * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
+            if sp.b_kc:
+                e("if (a->K & 7) return EVT_ERR_ALIGNMENT;")
+                e("if ((int64_t)Cfg::BN * a->ldb * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
+            else:
+                e("if (a->N & 7) return EVT_ERR_ALIGNMENT;")
+                e("if ((int64_t)Cfg::BK * a->ldb * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
+        for k, s in enumerate(ir.slots):
+            ct = DTYPE_CTYPES[s.dtype]
+            e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
+            e("  if (!x.ptr || x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
+            e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
+            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div;")
+            e(f"  p.t{k}_vec = (x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "
+              f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0) ? 1 : 0; }}")
+        e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
+        e("return EVT_OK;")
+        e.dedent()
+        e("}")
+        e("}  // namespace")
+        e("")
+        e('extern "C" int evt_abi_version(void) { return EVT_ABI_VERSION; }')
+        spec_json = json.dumps(self.module_spec(), sort_keys=True)
+        e(f'extern "C" const char* evt_module_spec(void) {{ return R"evtjson({spec_json})evtjson"; }}')
+        e('extern "C" int64_t evt_workspace_bytes(const EvtArgs* a) {')
+        e("  evt::GemmArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  return evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n).total();")
+        e("}")
+        e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
+        e("  if (bytes <= 0) return EVT_OK;")
+        e("  if (!ws || (bytes & 3)) return EVT_ERR_WORKSPACE;")
+        e("  hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ws, bytes / 4);")
+        e("  return (int)hipGetLastError();")
+        e("}")
+        e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
+        e("  evt::GemmArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  const int64_t need = evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n).total();")
+        e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
+        e("  g.workspace = (char*)ws;")
+        e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L);")
+        e("  hipLaunchKernelGGL((evt::evt_gemm_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  return (int)hipGetLastError();")
+        e("}")
+        return e.text()
+
+
+def generate(ir: EpilogueIR, spec: KernelSpec, module_name: str) -> str:
+    return Codegen(ir, spec, module_name).source()

@@ -1,0 +1,1005 @@
+"""EVT fuser: turns a partition of a torch.fx graph into one fused GEMM/BMM +
+epilogue kernel node.
+
+Host-side mirror of python/gtl/compiler/passes/evt_fuser.py of the reference:
+the same public surface (`EVTFuser.supported_targets`, `EVTFuser.fusible`,
+`EVTFuser(...).trace(gm, partition_names)`, the `visit_*` op vocabulary
+:1308-1485, `FusedOpBase.__call__(*epilogue_inputs, A, B) -> list[Tensor]`
+:190-267, `FusedGEMM` :453-558, `FusedBMM` :561-697), re-homed on this
+package's own IR, code generator and C-ABI kernel modules instead of the
+un-vendored CUTLASS Python package.
+"""
+from __future__ import annotations
+
+import operator
+import os
+from contextlib import nullcontext
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+from torch.fx import Node
+from torch.fx.graph_module import GraphModule
+from torch.fx.passes.tools_common import legalize_graph
+from torch.utils._python_dispatch import _len_torch_dispatch_stack, _pop_mode_temporarily
+
+from . import jit
+from .autotuner.bmm_tuner import BMMTuner
+from .autotuner.gemm_tuner import MMTuner
+from .codegen import KernelSpec, TileConfig
+from .ir import (DTYPE_NAMES, Coord, EpilogueIR, Node as IRNode, Slot, Store, Strides, accum_coord,
+                 fit_strides)
+
+aten = torch.ops.aten
+
+LAYOUT_TARGETS = {"view", "_unsafe_view", "reshape", "unsqueeze", "squeeze", "permute", "clone", "expand",
+                  "detach", "alias", "contiguous"}
+
+
+def packet(target):
+    """aten.add.Tensor -> aten.add (the reference strips overload suffixes in
+    its front end, python/gtl/compiler/passes/pass_frontend.py:131-192)."""
+    return getattr(target, "overloadpacket", target)
+
+
+def target_name(target) -> str:
+    name = getattr(packet(target), "__name__", str(target))
+    return name.split(".")[0]
+
+
+def node_shape_dtype(node: Node) -> Tuple[Tuple[int, ...], torch.dtype]:
+    if "tensor_meta" in node.meta:
+        tm = node.meta["tensor_meta"]
+        if isinstance(tm, (tuple, list)):
+            raise ValueError(f"{node.name} produces several tensors")
+        return tuple(int(s) for s in tm.shape), tm.dtype
+    if "val" in node.meta and isinstance(node.meta["val"], torch.Tensor):
+        v = node.meta["val"]
+        return tuple(int(s) for s in v.shape), v.dtype
+    raise ValueError(f"node {node.name} carries no shape metadata (run ShapeProp first)")
+
+
+def _contig_strides(shape: Sequence[int]) -> Tuple[int, ...]:
+    st, acc = [], 1
+    for s in reversed(shape):
+        st.append(acc)
+        acc *= int(s)
+    return tuple(reversed(st))
+
+
+# ---------------------------------------------------------------------------
+# run-time objects placed in the graph
+# ---------------------------------------------------------------------------
+
+
+class FusedOpBase:
+    """Callable placed in the fx graph.  `fused(*epilogue_inputs, A, B)` returns
+    the list of partition outputs (reference: evt_fuser.py:62-279)."""
+
+    def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
+        self.node = node
+        self.outputs = epilogue_visitor.outputs
+        self.output2store = epilogue_visitor.output2store
+        self.inputs = [i for i in epilogue_visitor.inputs if i is not node]
+        self.input_names = epilogue_visitor.input_names
+        self.post_reshape_permute = epilogue_visitor.post_reshape_permute
+        self.stream = None
+        self.mode = os.environ.get("MODE", "RUN")
+        self.launched = False
+        self.partition_names = epilogue_visitor.partition_names
+        self.rtol = 1e-2
+        self.atol = 1e-3
+        self.ir: EpilogueIR = epilogue_visitor.ir
+        # kernel-tensor bookkeeping filled by the visitor
+        self.slot_sources = epilogue_visitor.slot_sources      # slot -> ('input', idx) | ('output', store name)
+        self.store_meta = epilogue_visitor.store_meta          # store name -> (shape, dtype)
+        self._workspace = {}
+
+    # -- to be provided by subclasses -----------------------------------------
+    module: jit.KernelModule
+    problem: Tuple[int, int, int, int]   # M, N, K, L
+
+    def operands(self, A: torch.Tensor, B: torch.Tensor):
+        """-> (A, lda, batch_stride_A, B, ldb, batch_stride_B) ready for the kernel."""
+        raise NotImplementedError("Should be Overwritten by child class")
+
+    def call(self, visitor_args: Dict[str, torch.Tensor], stream, *args) -> Any:
+        M, N, K, L = self.problem
+        A, lda, bsa, B, ldb, bsb = self.operands(args[-2], args[-1])
+        a = jit.EvtArgs()
+        a.M, a.N, a.K, a.L = M, N, K, L
+        a.A, a.lda, a.batch_stride_A = A.data_ptr(), lda, bsa
+        a.B, a.ldb, a.batch_stride_B = B.data_ptr(), ldb, bsb
+        a.num_tensors = len(self.ir.slots)
+        a.num_scalars = len(self.ir.scalars)
+        keep = [A, B]
+        for k, slot in enumerate(self.ir.slots):
+            kind, ref = self.slot_sources[k]
+            t = args[ref] if kind == "input" else visitor_args[ref]
+            keep.append(t)
+            ta = a.tensors[k]
+            ta.ptr = t.data_ptr()
+            ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
+            ta.l_div = slot.strides.l_div
+        for i, s in enumerate(self.ir.scalars):
+            a.scalars[i] = s
+        ws_bytes = self.module.workspace_bytes(a)
+        ws_ptr = 0
+        if ws_bytes:
+            key = stream.cuda_stream
+            ws = self._workspace.get(key)
+            if ws is None or ws.numel() < ws_bytes:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
+                self.module.workspace_init(ws.data_ptr(), ws_bytes, stream.cuda_stream)
+                self._workspace[key] = ws
+            ws_ptr = ws.data_ptr()
+        self.module.launch(a, ws_ptr, ws_bytes, stream.cuda_stream)
+
+    def get_output_name(self, output: Node) -> str:
+        return "accum" if output is self.node else output.name
+
+    def __call__(self, *args_):
+        if not torch.cuda.is_available():
+            raise RuntimeError("the fused EVT kernels run on a HIP device only; none is available")
+        args = []
+        for arg in args_:
+            if isinstance(arg, torch.Tensor):
+                args.append(arg.contiguous())
+            else:
+                args.append(arg)
+
+        default_stream = torch.cuda.current_stream()
+        if self.stream is not None:
+            self.stream.wait_stream(default_stream)
+            stream = self.stream
+        else:
+            stream = default_stream
+
+        with torch.cuda.stream(stream):
+            device = args[-1].device
+            visitor_args: Dict[str, torch.Tensor] = {}
+            # one buffer per distinct store; reduction outputs need no zero fill
+            for name, (shape, dtype) in self.store_meta.items():
+                visitor_args[name] = torch.empty(shape, dtype=dtype, device=device)
+            for idx, input_name in enumerate(self.input_names):
+                visitor_args.setdefault(input_name, args[idx])
+
+            self.call(visitor_args, stream, *args)
+
+            if self.stream is not None:
+                for arg in args:
+                    if isinstance(arg, torch.Tensor):
+                        arg.record_stream(self.stream)
+
+            results = []
+            for output in self.outputs:
+                name = self.get_output_name(output)
+                out = visitor_args[self.output2store[name]]
+                for op, arg in self.post_reshape_permute.get(name, ()):
+                    out = out.view(arg) if op == "view" else out.permute(arg)
+                results.append(out)
+
+            if self.mode == "DEBUG" and not self.launched:
+                self.launched = True
+                self.reference(args, results)
+            return results
+
+    def reference(self, args, results):
+        """MODE=DEBUG self check against the eager fp32 evaluation of the
+        partition (reference: evt_fuser.py:98-172, rtol 1e-2)."""
+        raise NotImplementedError()
+
+    def get_src(self, node: Node) -> Node:
+        if packet(node.target) in self.mainloop_fusion_targets and node.name in self.partition_names:
+            return node.args[0]
+        return node
+
+    def get_alignment(self, dim: int) -> int:
+        for a in (8, 4, 2):
+            if dim % a == 0:
+                return a
+        return 1
+
+
+def _dma_ok(a_kc: bool, b_kc: bool, M: int, N: int, K: int, lda: int, ldb: int, bsa: int, bsb: int) -> bool:
+    """The fast global->LDS path moves 16-byte chunks: every operand row must
+    start on a 16-byte boundary and the contiguous extent must be a multiple
+    of 8 elements (the same role as the reference's alignment_A/B = 8 case,
+    evt_fuser.py:502-512)."""
+    if (lda | ldb | bsa | bsb) & 7:
+        return False
+    if (a_kc or b_kc) and K % 8:
+        return False
+    if not a_kc and M % 8:
+        return False
+    if not b_kc and N % 8:
+        return False
+    return True
+
+
+class FusedGEMM(FusedOpBase):
+    """epilogue_visitor(A @ B, args) as one kernel (reference: evt_fuser.py:453-558)."""
+    __name__ = "cutlass_gemm_with_visitor"
+    target = aten.mm
+    mainloop_fusion_targets = [aten.permute]
+
+    def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
+        super().__init__(node, epilogue_visitor)
+        lhs_node, rhs_node = node.args[0], node.args[1]
+        self.lhs_layout = self.get_src_layout(lhs_node)
+        self.rhs_layout = self.get_src_layout(rhs_node)
+        self.A = self.get_src(lhs_node)
+        self.B = self.get_src(rhs_node)
+        self.args = [self.A, self.B]
+
+        lhs_shape, dtype = node_shape_dtype(lhs_node)
+        rhs_shape, _ = node_shape_dtype(rhs_node)
+        M, K = lhs_shape[-2:]
+        N = rhs_shape[-1]
+        self.problem = (M, N, K, 1)
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise NotImplementedError(f"GEMM operands of dtype {dtype}")
+        self.a_kc = self.lhs_layout == "RowMajor"
+        self.b_kc = self.rhs_layout == "ColumnMajor"
+        self.lda = K if self.a_kc else M
+        self.ldb = K if self.b_kc else N
+        dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb, 0, 0)
+
+        self.align_A = self.get_alignment(K if self.a_kc else M)
+        self.align_B = self.get_alignment(K if self.b_kc else N)
+        self.align_C = self.get_alignment(N)
+
+        with (_pop_mode_temporarily() if _len_torch_dispatch_stack() > 0 else nullcontext()):
+            tuner = MMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
+            tile = tuner.get_best_config()
+            self.tile = tile
+            self.spec = KernelSpec(self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
+            self.module = jit.load_module(self.ir, self.spec)
+
+    def operands(self, A, B):
+        A = A.contiguous()
+        B = B.contiguous()
+        return A, self.lda, 0, B, self.ldb, 0
+
+    def get_src_layout(self, node: Node) -> str:
+        if packet(node.target) == aten.permute and node.name in self.partition_names:
+            indices = [int(i) for i in node.args[1]]
+            if indices == [0, 1]:
+                return "RowMajor"
+            if indices == [1, 0]:
+                return "ColumnMajor"
+            raise ValueError(f"Invalid permutation: {indices}")
+        return "RowMajor"
+
+
+class FusedBMM(FusedOpBase):
+    """Batched variant; A/B may be 3-D permutations of their source tensors
+    (reference: evt_fuser.py:561-697, python/gtl/ops/bmm.py:23-64)."""
+    __name__ = "cutlass_bmm_with_visitor"
+    target = aten.bmm
+    mainloop_fusion_targets = [aten.permute]
+
+    def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
+        super().__init__(node, epilogue_visitor)
+        lhs_node, rhs_node = node.args[0], node.args[1]
+        self.A = self.get_src(lhs_node)
+        self.B = self.get_src(rhs_node)
+        self.args = [self.A, self.B]
+        self.permute_A = self.get_permutation(lhs_node)
+        self.permute_B = self.get_permutation(rhs_node)
+
+        lhs_shape, dtype = node_shape_dtype(lhs_node)
+        rhs_shape, _ = node_shape_dtype(rhs_node)
+        L, M, K = lhs_shape
+        N = rhs_shape[-1]
+        self.problem = (M, N, K, L)
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise NotImplementedError(f"BMM operands of dtype {dtype}")
+
+        # strides of the logical [L, M, K] / [L, K, N] operands inside their
+        # (contiguous) source tensors
+        sa = self._logical_strides(self.A, self.permute_A)
+        sb = self._logical_strides(self.B, self.permute_B)
+        self.copy_A = self.copy_B = False
+        if sa[2] == 1:
+            self.a_kc, self.lda, self.bsa = True, sa[1], sa[0]
+        elif sa[1] == 1:
+            self.a_kc, self.lda, self.bsa = False, sa[2], sa[0]
+        else:   # batch-last source: make the permuted operand contiguous first (evt_fuser.py:663-672)
+            self.copy_A, self.a_kc, self.lda, self.bsa = True, True, K, M * K
+        if sb[1] == 1:
+            self.b_kc, self.ldb, self.bsb = True, sb[2], sb[0]
+        elif sb[2] == 1:
+            self.b_kc, self.ldb, self.bsb = False, sb[1], sb[0]
+        else:
+            self.copy_B, self.b_kc, self.ldb, self.bsb = True, False, N, K * N
+        if M == 1 and self.a_kc is False:
+            pass
+        self.lhs_layout = "RowMajor" if self.a_kc else "ColumnMajor"
+        self.rhs_layout = "ColumnMajor" if self.b_kc else "RowMajor"
+        dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb, self.bsa, self.bsb)
+
+        with (_pop_mode_temporarily() if _len_torch_dispatch_stack() > 0 else nullcontext()):
+            tuner = BMMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
+            tile = tuner.get_best_config()
+            self.tile = tile
+            self.spec = KernelSpec(self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
+            self.module = jit.load_module(self.ir, self.spec)
+
+    def get_permutation(self, node: Node) -> List[int]:
+        if packet(node.target) == aten.permute and node.name in self.partition_names:
+            return [int(i) for i in node.args[1]]
+        return [0, 1, 2]
+
+    @staticmethod
+    def _logical_strides(src: Node, perm: List[int]) -> Tuple[int, int, int]:
+        shape, _ = node_shape_dtype(src)
+        st = _contig_strides(shape)
+        return tuple(st[p] for p in perm)
+
+    def operands(self, A, B):
+        if self.copy_A:
+            A = aten.permute(A, self.permute_A).contiguous()
+        if self.copy_B:
+            B = aten.permute(B, self.permute_B).contiguous()
+        return A, self.lda, self.bsa, B, self.ldb, self.bsb
+
+
+def _unsupported_anchor(name: str, where: str):
+    class _Stub(FusedOpBase):
+        __doc__ = (f"{name}: anchor outside this backend's scope (the fused GEMM/BMM path); "
+                   f"reference: evt_fuser.py:{where}.")
+
+        def __init__(self, *a, **k) -> None:
+            raise NotImplementedError(f"{name} is not provided by the MI355X GEMM/BMM backend")
+    _Stub.__name__ = name
+    _Stub.__qualname__ = name
+    return _Stub
+
+
+FusedConvFprop = _unsupported_anchor("FusedConvFprop", "282-365")
+FusedConvDgrad = _unsupported_anchor("FusedConvDgrad", "368-450")
+FusedSoftmax = _unsupported_anchor("FusedSoftmax", "700-762")
+FusedSoftmaxBackward = _unsupported_anchor("FusedSoftmaxBackward", "765-826")
+FusedLayerNorm = _unsupported_anchor("FusedLayerNorm", "829-902")
+FusedLayerNormBackward = _unsupported_anchor("FusedLayerNormBackward", "905-970")
+FusedSpmm = _unsupported_anchor("FusedSpmm", "973-1035")
+
+
+# ---------------------------------------------------------------------------
+# the fuser
+# ---------------------------------------------------------------------------
+
+
+class EVTFuser:
+    """Entry point: `EVTFuser.fusible(partition, gm)` and
+    `EVTFuser().trace(gm, partition)` (reference: evt_fuser.py:1038-1235)."""
+
+    supported_targets = [aten.mm, aten.bmm]
+
+    def __init__(self, element_compute=torch.float32, **kwargs):
+        self.element_compute = element_compute
+        self.mode = os.environ.get("MODE", "RUN")
+
+    @staticmethod
+    def get_node_with_name(name: str, graph_module: GraphModule) -> Node:
+        for node in graph_module.graph.nodes:
+            if node.name == name:
+                return node
+        raise ValueError(f"{name} is not in the graph.")
+
+    @staticmethod
+    def fusible(partition: Sequence[str], graph_module: GraphModule) -> bool:
+        for node_name in partition:
+            node = EVTFuser.get_node_with_name(node_name, graph_module)
+            if node.op == "call_function" and packet(node.target) in EVTFuser.supported_targets:
+                return True
+        return False
+
+    # -- tracing ------------------------------------------------------------------
+    def trace(self, graph_module: GraphModule, partition_: Sequence[str]):
+        self.partition_names = list(partition_)
+        try:
+            graph_module.graph.lint()
+        except Exception:
+            legalize_graph(graph_module)
+        in_partition = set(self.partition_names)
+        partition = [n for n in graph_module.graph.nodes if n.name in in_partition]
+
+        # Step 1: anchor = the heavy op; producers of the anchor inside the
+        # partition are main-loop fusions (operand permutes), not epilogue
+        anchor = None
+        for node in partition:
+            if node.op == "call_function" and packet(node.target) in self.supported_targets:
+                anchor = node
+        if anchor is None:
+            raise ValueError("partition holds no supported anchor")
+        self.anchor = anchor
+        epilogue_partition = [n for n in partition if n is not anchor and anchor not in n.users]
+        epi_set = set(epilogue_partition)
+
+        # Step 2: inputs and outputs of the epilogue, in graph order
+        inputs: List[Node] = []
+        for node in epilogue_partition:
+            for inp in node.all_input_nodes:
+                if inp not in epi_set and inp not in inputs:
+                    inputs.append(inp)
+        outputs: List[Node] = []
+        for node in epilogue_partition:
+            if any(user not in epi_set for user in node.users):
+                outputs.append(node)
+        store_anchor = any(user not in epi_set for user in anchor.users) or not epilogue_partition
+        if store_anchor:
+            outputs.insert(0, anchor)
+        self.inputs = inputs
+        self.outputs = outputs
+        self.outputs_subgraph = set(outputs)
+
+        # Step 3: build the IR
+        (ashape, adtype) = node_shape_dtype(anchor)
+        batched = packet(anchor.target) == aten.bmm
+        if batched:
+            L, M, N = ashape
+        else:
+            L, (M, N) = 1, ashape
+        self.L, self.M, self.N = L, M, N
+        self.ir = EpilogueIR(L, M, N, batched)
+        self.ir.add_node(IRNode("accum", "accum", domain="tile"))
+        self.coords: Dict[Node, Coord] = {anchor: accum_coord(L, M, N, batched)}
+        self.ir_name: Dict[Node, str] = {anchor: "accum"}
+        self.full = self._accum_dependents(anchor, epi_set)
+        self.load_cache: Dict[Tuple[str, Tuple[int, ...]], str] = {}
+        self.input_index = {n: i for i, n in enumerate(x for x in inputs if x is not anchor)}
+        self.input_names = [n.name for n in inputs if n is not anchor]
+        self.input_nodes = [n for n in inputs if n is not anchor]
+        self.slot_sources: Dict[int, Tuple[str, Any]] = {}
+        self.pending_multi: Dict[Node, Dict[int, str]] = {}
+
+        for node in epilogue_partition:
+            if node in self.full:
+                self.visit(node)
+
+        # Step 4: stores
+        self.output2store: Dict[str, str] = {}
+        self.post_reshape_permute: Dict[str, List[Tuple[str, Any]]] = {}
+        self.store_meta: Dict[str, Tuple[Tuple[int, ...], torch.dtype]] = {}
+        store_key: Dict[Tuple, str] = {}
+        for out in outputs:
+            self._insert_store(out, store_key)
+        self.ir.finalize()
+        # slot indices may have been compacted by finalize(): rebuild the map
+        self._rebuild_slot_sources()
+        self.return_names = [o.name for o in outputs]
+        self.reduction_names = [s.name for s in self.ir.slots if s.role == "store" and s.domain != "tile"]
+        self.transposed = False
+
+        # Step 5: compose the fused kernel and rewire the graph
+        fused_kernel = self.get_fused_node(anchor)
+        args = [i for i in inputs if i is not anchor] + fused_kernel.args
+        graph_module.graph.inserting_after(anchor)
+        fused_node = graph_module.graph.call_function(fused_kernel, args=tuple(args))
+        fused_node.meta = {"evt": True}
+        graph_module.graph.inserting_after(fused_node)
+        for idx, output_node in enumerate(outputs):
+            get_item_node = graph_module.graph.call_function(operator.getitem, args=(fused_node, idx))
+            graph_module.graph.inserting_after(get_item_node)
+            shape, _ = node_shape_dtype(output_node)
+            view_node = graph_module.graph.call_function(aten.view, args=(get_item_node, list(shape)))
+            view_node.meta = {k: v for k, v in output_node.meta.items() if k in ("tensor_meta", "val")}
+            if output_node is anchor:
+                for user in list(anchor.users):
+                    if user not in epi_set and user is not fused_node:
+                        user.replace_input_with(anchor, view_node)
+            else:
+                output_node.replace_all_uses_with(view_node)
+            graph_module.graph.inserting_after(view_node)
+        self.fused_kernel = fused_kernel
+        return fused_kernel
+
+    def _accum_dependents(self, anchor: Node, epi_set) -> set:
+        full = {anchor}
+        changed = True
+        order = [n for n in anchor.graph.nodes if n in epi_set]
+        while changed:
+            changed = False
+            for n in order:
+                if n not in full and any(i in full for i in n.all_input_nodes):
+                    full.add(n)
+                    changed = True
+        return full
+
+    def _rebuild_slot_sources(self):
+        self.slot_sources = {}
+        for k, slot in enumerate(self.ir.slots):
+            if slot.role == "load":
+                node = next(n for n in self.input_nodes if n.name == slot.name)
+                self.slot_sources[k] = ("input", self.input_index[node])
+            else:
+                self.slot_sources[k] = ("output", slot.name)
+
+    # -- stores ---------------------------------------------------------------------
+    def _insert_store(self, out: Node, store_key: Dict[Tuple, str]):
+        name = "accum" if out is self.anchor else out.name
+        shape, dtype = node_shape_dtype(out)
+        if dtype not in DTYPE_NAMES:
+            raise NotImplementedError(f"output dtype {dtype}")
+        value = self.ir_name[out]
+        domain = self.ir.nodes[value].domain
+        if domain not in ("tile", "row", "col"):
+            raise NotImplementedError(
+                f"output {out.name} does not depend on the accumulator; keep it outside the partition")
+        # find the tensor to materialise: the output itself, or (if its layout
+        # is not strided in (l, m, n)) the node before trailing view/permute
+        # ops, which are then applied as free views on the stored tensor
+        # (the reference's post_reshape_permute, evt_fuser.py:247-255)
+        node, post = out, []
+        while True:
+            st = fit_strides(self.coords[node], self.L, self.M, self.N)
+            if st is not None:
+                break
+            tname = target_name(node.target) if node.op == "call_function" else ""
+            src = node.args[0] if node.args and isinstance(node.args[0], Node) else None
+            if tname not in LAYOUT_TARGETS or src is None or src not in self.coords:
+                raise NotImplementedError(f"output {out.name}: layout is not expressible with (l, m, n) strides")
+            nshape, _ = node_shape_dtype(node)
+            if tname == "permute":
+                post.insert(0, ("permute", [int(i) for i in node.args[1]]))
+            elif tname in ("clone", "contiguous"):
+                raise NotImplementedError(f"output {out.name}: materialised permutation is not strided in (l, m, n)")
+            else:
+                post.insert(0, ("view", list(nshape)))
+            node = src
+        sshape, _ = node_shape_dtype(node)
+        key = (value, st.stride_l, st.stride_m, st.stride_n, st.l_div, dtype, domain)
+        if key in store_key:
+            self.output2store[name] = store_key[key]
+            stored_shape = self.store_meta[store_key[key]][0]
+            if tuple(stored_shape) != tuple(sshape):
+                post.insert(0, ("view", list(sshape)))
+        else:
+            store_key[key] = name
+            self.output2store[name] = name
+            self.store_meta[name] = (tuple(sshape), dtype)
+            kind = {"tile": "aux", "row": "col", "col": "row"}[domain]
+            k = self.ir.add_slot(Slot(name, "store", DTYPE_NAMES[dtype], domain, kind, st, tuple(sshape)))
+            self.ir.stores.append(Store(k, value, domain))
+        if post:
+            self.post_reshape_permute[name] = post
+
+    # -- operand materialisation (top-down) -----------------------------------------
+    def _operand(self, arg, consumer_coord: Coord) -> str:
+        """IR value name for operand `arg` of a node indexed by `consumer_coord`."""
+        if isinstance(arg, (int, float, bool)):
+            return self.ir.add_imm(float(arg))
+        if not isinstance(arg, Node):
+            raise NotImplementedError(f"operand {arg!r}")
+        if arg in self.ir_name and arg in self.coords:
+            return self.ir_name[arg]
+        shape, dtype = node_shape_dtype(arg)
+        return self._materialize(arg, consumer_coord.restrict(shape))
+
+    def _materialize(self, node: Node, coord: Coord) -> str:
+        """Value of a tensor that does not depend on the accumulator, indexed
+        through `coord` (derived from its consumer)."""
+        shape, dtype = node_shape_dtype(node)
+        in_epilogue = node.name in self.partition_names and node.op == "call_function" and node is not self.anchor
+        if not in_epilogue or node in self.inputs:
+            # a kernel input: classify by how its offset varies with (l, m, n)
+            st = fit_strides(coord, self.L, self.M, self.N)
+            if st is None:
+                raise NotImplementedError(f"input {node.name}: broadcast pattern is not strided in (l, m, n)")
+            key = (node.name, (st.stride_l, st.stride_m, st.stride_n, st.l_div))
+            if key in self.load_cache:
+                return self.load_cache[key]
+            if dtype not in DTYPE_NAMES:
+                raise NotImplementedError(f"input dtype {dtype}")
+            if node not in self.input_index:
+                raise NotImplementedError(f"{node.name} is used by the epilogue but is not a partition input")
+            k = self.ir.add_slot(Slot(node.name, "load", DTYPE_NAMES[dtype], "tile", st.kind, st, shape))
+            name = node.name if node.name not in self.ir.nodes else f"{node.name}_ld{k}"
+            self.ir.add_node(IRNode(name, "load", domain="flex", slot=k))
+            self.load_cache[key] = name
+            return name
+        tname = target_name(node.target)
+        src = node.args[0] if node.args and isinstance(node.args[0], Node) else None
+        if tname in ("view", "_unsafe_view", "reshape", "unsqueeze", "squeeze", "clone", "detach", "alias",
+                     "contiguous", "expand"):
+            sshape, _ = node_shape_dtype(src)
+            if tname == "expand":
+                return self._materialize(src, coord.restrict(sshape))
+            return self._materialize(src, coord.reshape(sshape))
+        if tname == "permute":
+            sshape, _ = node_shape_dtype(src)
+            return self._materialize(src, coord.inverse_permute([int(i) for i in node.args[1]], sshape))
+        # elementwise on small tensors: evaluate per element from its operands
+        saved = (self.coords.get(node), )
+        self.coords[node] = coord
+        try:
+            self.visit(node)
+        finally:
+            pass
+        return self.ir_name[node]
+
+    # -- node visitors (reference vocabulary: evt_fuser.py:1308-1485) ----------------
+    def visit(self, node: Node):
+        if node.op in ("placeholder", "get_attr"):
+            return
+        if node.op == "call_function":
+            name = target_name(node.target)
+            fn = getattr(self, f"visit_{name}", None)
+            if fn is None:
+                raise NotImplementedError(f"Doesn't support target {node.target}")
+            return fn(node)
+
+    def _coord_for(self, node: Node) -> Coord:
+        """Coordinate function of an elementwise node: inherited from its
+        accumulator-dependent operand (shapes equal up to broadcasting)."""
+        if node in self.coords:
+            return self.coords[node]
+        shape, _ = node_shape_dtype(node)
+        numel = 1
+        for s in shape:
+            numel *= s
+        for arg in node.all_input_nodes:
+            if arg in self.coords and arg in self.full:
+                c = self.coords[arg]
+                if c.numel() == numel:
+                    return Coord(shape, c.fn)
+        raise NotImplementedError(f"{node.name}: result is larger than its accumulator-dependent operand")
+
+    def _visit_compute(self, node: Node, op: str, args: Optional[Sequence] = None):
+        coord = self._coord_for(node)
+        self.coords[node] = coord
+        operands = [self._operand(a, coord) for a in (node.args if args is None else args)]
+        name = node.name
+        self.ir.add_compute(name, op, operands)
+        self.ir_name[node] = name
+        return name
+
+    def _visit_layout(self, node: Node, fn):
+        src = node.args[0]
+        self.coords[node] = fn(self.coords[src])
+        self.ir_name[node] = self.ir_name[src]
+        return self.ir_name[node]
+
+    def visit_add(self, node: Node):
+        args = list(node.args)
+        alpha = node.kwargs.get("alpha", 1)
+        if alpha != 1:
+            raise NotImplementedError("add with alpha")
+        return self._visit_compute(node, "add", args)
+
+    def visit_sub(self, node: Node):
+        if node.kwargs.get("alpha", 1) != 1:
+            raise NotImplementedError("sub with alpha")
+        return self._visit_compute(node, "sub")
+
+    def visit_rsub(self, node: Node):
+        return self._visit_compute(node, "sub", [node.args[1], node.args[0]])
+
+    def visit_mul(self, node: Node):
+        return self._visit_compute(node, "mul")
+
+    def visit_div(self, node: Node):
+        return self._visit_compute(node, "div")
+
+    def visit_neg(self, node: Node):
+        return self._visit_compute(node, "neg")
+
+    def visit_maximum(self, node: Node):
+        return self._visit_compute(node, "max")
+
+    def visit_minimum(self, node: Node):
+        return self._visit_compute(node, "min")
+
+    def visit_exp(self, node: Node):
+        return self._visit_compute(node, "exp")
+
+    def visit_log(self, node: Node):
+        return self._visit_compute(node, "log")
+
+    def visit_sqrt(self, node: Node):
+        return self._visit_compute(node, "sqrt")
+
+    def visit_rsqrt(self, node: Node):
+        return self._visit_compute(node, "rsqrt")
+
+    def visit_abs(self, node: Node):
+        return self._visit_compute(node, "abs")
+
+    def visit_reciprocal(self, node: Node):
+        return self._visit_compute(node, "rcp")
+
+    def visit_gelu(self, node: Node):
+        # the reference drops the `approximate` keyword (evt_fuser.py:1377-1378);
+        # here it selects the functor, as PyTorch defines it
+        approx = node.kwargs.get("approximate", "none")
+        return self._visit_compute(node, "gelu_tanh" if approx == "tanh" else "gelu_erf", node.args[:1])
+
+    def visit_tanh(self, node: Node):
+        return self._visit_compute(node, "tanh")
+
+    def visit_relu(self, node: Node):
+        return self._visit_compute(node, "relu")
+
+    def visit_sigmoid(self, node: Node):
+        return self._visit_compute(node, "sigmoid")
+
+    def visit_tanh_backward(self, node: Node):
+        return self._visit_compute(node, "tanh_backward")
+
+    def visit_gelu_backward(self, node: Node):
+        approx = node.kwargs.get("approximate", "none")
+        return self._visit_compute(node, "gelu_backward_tanh" if approx == "tanh" else "gelu_backward_erf",
+                                   node.args[:2])
+
+    def visit_ge(self, node: Node):
+        return self._visit_compute(node, "ge")
+
+    def visit_gt(self, node: Node):
+        return self._visit_compute(node, "gt")
+
+    def visit_le(self, node: Node):
+        return self._visit_compute(node, "le")
+
+    def visit_lt(self, node: Node):
+        return self._visit_compute(node, "lt")
+
+    def visit_ne(self, node: Node):
+        return self._visit_compute(node, "ne")
+
+    def visit_eq(self, node: Node):
+        return self._visit_compute(node, "eq")
+
+    def visit_where(self, node: Node):
+        return self._visit_compute(node, "where")
+
+    def visit_rand_like(self, node: Node):
+        raise NotImplementedError("fused dropout (rand_like) is not provided yet")
+
+    def visit__to_copy(self, node: Node):
+        dtype = node.kwargs.get("dtype", None)
+        return self._visit_cast(node, dtype)
+
+    def visit_to(self, node: Node):
+        dtype = node.args[1] if len(node.args) > 1 and isinstance(node.args[1], torch.dtype) else node.kwargs.get("dtype")
+        return self._visit_cast(node, dtype)
+
+    def _visit_cast(self, node: Node, dtype):
+        op = {torch.float16: "cast_f16", torch.bfloat16: "cast_bf16", torch.float32: "cast_f32",
+              torch.bool: "cast_bool", torch.int32: "cast_int", torch.int64: "cast_int", None: "cast_f32"}.get(dtype)
+        if op is None:
+            raise NotImplementedError(f"cast to {dtype}")
+        src = node.args[0]
+        _, sdtype = node_shape_dtype(src)
+        if op == "cast_f32" or (sdtype == dtype):
+            # widening (or no-op) casts do not change the fp32 value
+            if src in self.coords and src in self.ir_name:
+                self.coords[node] = Coord(node_shape_dtype(node)[0], self.coords[src].fn)
+                self.ir_name[node] = self.ir_name[src]
+                return self.ir_name[node]
+        return self._visit_compute(node, op, node.args[:1])
+
+    def visit_one_hot(self, node: Node):
+        """one_hot(label, num_classes)[..., n] == (label == n); the class axis is
+        the GEMM N axis (reference: VisitorComputeOneHot,
+        src/cuda/epilogue/threadblock/visitor_compute.hpp:98-145)."""
+        num_classes = node.kwargs.get("num_classes", node.args[1] if len(node.args) > 1 else -1)
+        shape, _ = node_shape_dtype(node)
+        if int(num_classes) != self.N or shape[-1] != self.N:
+            raise NotImplementedError("one_hot whose class axis is not the GEMM N axis")
+        coord = self._coord_for(node) if node in self.coords else None
+        if coord is None:
+            raise NotImplementedError("one_hot must be consumed by an accumulator-dependent node")
+        labels = node.args[0]
+        lshape, _ = node_shape_dtype(labels)
+        label_val = self._materialize(labels, coord.restrict(tuple(lshape) + (1,)))
+        if "colidx" not in self.ir.nodes:
+            self.ir.add_node(IRNode("colidx", "colidx", domain="tile"))
+        self.ir.add_compute(node.name, "eq", [label_val, "colidx"])
+        self.ir_name[node] = node.name
+        return node.name
+
+    def visit_gather(self, node: Node):
+        """gather(x, -1, index[..., 1]) of an accumulator-dependent x along the N
+        axis: sum_n x[n] * (index == n), a per-row reduction."""
+        x, dim, index = node.args[0], node.args[1], node.args[2]
+        xshape, _ = node_shape_dtype(x)
+        ishape, _ = node_shape_dtype(index)
+        if dim % len(xshape) != len(xshape) - 1 or ishape[-1] != 1 or xshape[-1] != self.N:
+            raise NotImplementedError("gather other than one index per row along N")
+        cx = self.coords[x]
+        label_val = self._materialize(index, cx.restrict(ishape))
+        if "colidx" not in self.ir.nodes:
+            self.ir.add_node(IRNode("colidx", "colidx", domain="tile"))
+        hit = f"{node.name}_hit"
+        self.ir.add_compute(hit, "eq", [label_val, "colidx"])
+        sel = f"{node.name}_sel"
+        zero = self.ir.add_imm(0.0)
+        self.ir.add_compute(sel, "where", [hit, self.ir_name[x], zero])
+        return self._reduce(node, sel, cx, [len(xshape) - 1], True, "sum")
+
+    # -- reductions ------------------------------------------------------------------
+    def _reduce(self, node: Node, value: str, coord: Coord, dims, keepdim: bool, kind: str,
+                comps: Sequence[int] = (0,)):
+        rc = coord.reduce(dims, keepdim)
+        st = fit_strides(rc, self.L, self.M, self.N)
+        if st is None:
+            raise NotImplementedError(f"{node.name}: reduction result is not strided in (l, m, n)")
+        numel = rc.numel()
+        if st.stride_n == 0 and numel == self.L * self.M:
+            axis = "row"
+        elif st.stride_m == 0 and numel == self.L * self.N and (self.L == 1 or st.stride_l != 0):
+            axis = "col"
+        else:
+            raise NotImplementedError(
+                f"{node.name}: reduces over something other than exactly the N axis or exactly the M axis")
+        rname = f"{node.name}_red"
+        self.ir.add_reduce(rname, kind, axis, value)
+        names = []
+        for c in comps:
+            n = f"{node.name}_r{c}"
+            self.ir.add_node(IRNode(n, "rres", domain=axis, reduce=rname, comp=c))
+            names.append(n)
+        self.coords[node] = rc
+        return names
+
+    @staticmethod
+    def _dims(arg, rank):
+        if arg is None or arg == []:
+            return list(range(rank))
+        if isinstance(arg, int):
+            return [arg]
+        return [int(a) for a in arg]
+
+    def visit_sum(self, node: Node):
+        x = node.args[0]
+        shape, _ = node_shape_dtype(x)
+        dims = self._dims(node.args[1] if len(node.args) > 1 else None, len(shape))
+        keepdim = bool(node.args[2]) if len(node.args) > 2 else bool(node.kwargs.get("keepdim", False))
+        value = self.ir_name[x]
+        fused = self._match_softmax_stats(x, dims)
+        if fused is not None:
+            base, amax_node = fused
+            rname = self.ir.nodes[self.ir_name[amax_node]].reduce
+            # upgrade the row max to the (max, sum-exp) pair; this sum is its
+            # second component
+            self.ir.reduces[rname].kind = "maxsumexp"
+            n = f"{node.name}_r1"
+            self.ir.add_node(IRNode(n, "rres", domain="row", reduce=rname, comp=1))
+            self.coords[node] = self.coords[x].reduce(dims, keepdim)
+            self.ir_name[node] = n
+            return n
+        (n,) = self._reduce(node, value, self.coords[x], dims, keepdim, "sum")
+        self.ir_name[node] = n
+        return n
+
+    def _match_softmax_stats(self, x: Node, dims) -> Optional[Tuple[Node, Node]]:
+        """x == exp(sub(s, amax(s, dims, keepdim=True))) with the amax already a
+        per-row max reduction of the same s -> (s, amax node)."""
+        if x.op != "call_function" or target_name(x.target) != "exp":
+            return None
+        sub = x.args[0]
+        if not isinstance(sub, Node) or sub.op != "call_function" or target_name(sub.target) != "sub":
+            return None
+        s, m = sub.args[0], sub.args[1]
+        if not isinstance(m, Node) or not isinstance(s, Node) or m not in self.ir_name:
+            return None
+        mval = self.ir.nodes.get(self.ir_name[m])
+        if mval is None or mval.op != "rres" or mval.comp != 0:
+            return None
+        red = self.ir.reduces[mval.reduce]
+        if red.kind not in ("max", "maxsumexp") or red.axis != "row" or red.input != self.ir_name.get(s):
+            return None
+        shape, _ = node_shape_dtype(x)
+        if sorted(d % len(shape) for d in dims) != [len(shape) - 1]:
+            return None
+        return s, m
+
+    def visit_amax(self, node: Node):
+        x = node.args[0]
+        shape, _ = node_shape_dtype(x)
+        dims = self._dims(node.args[1] if len(node.args) > 1 else None, len(shape))
+        keepdim = bool(node.args[2]) if len(node.args) > 2 else bool(node.kwargs.get("keepdim", False))
+        (n,) = self._reduce(node, self.ir_name[x], self.coords[x], dims, keepdim, "max")
+        self.ir_name[node] = n
+        return n
+
+    def visit_mean(self, node: Node):
+        x = node.args[0]
+        shape, _ = node_shape_dtype(x)
+        dims = self._dims(node.args[1] if len(node.args) > 1 else None, len(shape))
+        keepdim = bool(node.args[2]) if len(node.args) > 2 else bool(node.kwargs.get("keepdim", False))
+        (s,) = self._reduce(node, self.ir_name[x], self.coords[x], dims, keepdim, "sum")
+        count = 1
+        for d in dims:
+            count *= shape[d]
+        inv = self.ir.add_imm(1.0 / count)
+        self.ir.add_compute(node.name, "mul", [s, inv])
+        self.ir_name[node] = node.name
+        return node.name
+
+    def visit_logsumexp(self, node: Node):
+        x = node.args[0]
+        shape, _ = node_shape_dtype(x)
+        dims = self._dims(node.args[1], len(shape))
+        keepdim = bool(node.args[2]) if len(node.args) > 2 else bool(node.kwargs.get("keepdim", False))
+        m, l = self._reduce(node, self.ir_name[x], self.coords[x], dims, keepdim, "maxsumexp", (0, 1))
+        if self.ir.reduces[f"{node.name}_red"].axis != "row":
+            raise NotImplementedError("logsumexp over the M axis")
+        self.ir.add_compute(f"{node.name}_log", "log", [l])
+        self.ir.add_compute(node.name, "add", [m, f"{node.name}_log"])
+        self.ir_name[node] = node.name
+        return node.name
+
+    def visit_var_mean(self, node: Node):
+        """var_mean(x, dims, correction=c, keepdim=k) -> (var, mean); consumed
+        through getitem."""
+        x = node.args[0]
+        shape, _ = node_shape_dtype(x)
+        dims = self._dims(node.args[1] if len(node.args) > 1 else node.kwargs.get("dim"), len(shape))
+        keepdim = bool(node.kwargs.get("keepdim", False))
+        correction = node.kwargs.get("correction", 1)
+        if "unbiased" in node.kwargs:
+            correction = 1 if node.kwargs["unbiased"] else 0
+        n, mean, m2 = self._reduce(node, self.ir_name[x], self.coords[x], dims, keepdim, "welford", (0, 1, 2))
+        if self.ir.reduces[f"{node.name}_red"].axis != "row":
+            raise NotImplementedError("var_mean over the M axis")
+        denom = n
+        if correction:
+            c = self.ir.add_imm(float(correction))
+            denom = f"{node.name}_dof"
+            self.ir.add_compute(denom, "sub", [n, c])
+        var = f"{node.name}_var"
+        self.ir.add_compute(var, "div", [m2, denom])
+        self.pending_multi[node] = {0: var, 1: mean}
+        return var
+
+    def visit_getitem(self, node: Node):
+        src, idx = node.args
+        if src not in self.pending_multi:
+            raise NotImplementedError(f"getitem of {src.name}")
+        self.ir_name[node] = self.pending_multi[src][int(idx)]
+        self.coords[node] = Coord(node_shape_dtype(node)[0], self.coords[src].fn)
+        return self.ir_name[node]
+
+    # -- layout ops: no data movement, only index bookkeeping -----------------------
+    def visit_view(self, node: Node):
+        shape, _ = node_shape_dtype(node)
+        return self._visit_layout(node, lambda c: c.reshape(shape))
+
+    visit__unsafe_view = visit_view
+    visit_reshape = visit_view
+    visit_unsqueeze = visit_view
+    visit_squeeze = visit_view
+
+    def visit_permute(self, node: Node):
+        dims = [int(i) for i in node.args[1]]
+        return self._visit_layout(node, lambda c: c.permute(dims))
+
+    def visit_clone(self, node: Node):
+        return self._visit_layout(node, lambda c: c)
+
+    visit_detach = visit_clone
+    visit_alias = visit_clone
+    visit_contiguous = visit_clone
+
+    def visit_expand(self, node: Node):
+        shape, _ = node_shape_dtype(node)
+        src_shape, _ = node_shape_dtype(node.args[0])
+        n1 = n2 = 1
+        for s in shape:
+            n1 *= s
+        for s in src_shape:
+            n2 *= s
+        if n1 != n2:
+            raise NotImplementedError("expand that enlarges an accumulator-dependent tensor")
+        return self._visit_layout(node, lambda c: c.reshape(shape))
+
+    # -- main-loop op ------------------------------------------------------------------
+    def get_fused_node(self, node: Node):
+        tgt = packet(node.target)
+        if tgt == aten.mm:
+            return FusedGEMM(node, self)
+        if tgt == aten.bmm:
+            return FusedBMM(node, self)
+        raise NotImplementedError()

@@ -1,0 +1,170 @@
+"""Compile, cache and load generated kernel modules.
+
+Replaces the un-vendored `cutlass.backend.compiler` (nvcc/nvrtc JIT with a
+sqlite `compiled_cache.db`; call sites python/gtl/compiler/passes/
+evt_fuser.py:515-518, :738-746).  A module is identified by the SHA-256 of its
+generated source and compile flags; the shared object is kept in-tree under
+`evt_ae_amd/_kernels/` so that modules built ahead of time travel with the
+source tree, and an sqlite index (`compiled_cache.db`) records what each file
+is.  Loading goes through ctypes against the C ABI of include/evt_amd.h.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import json
+import os
+import sqlite3
+import subprocess
+import threading
+from pathlib import Path
+from typing import Dict, Optional
+
+from .codegen import KernelSpec, generate
+from .ir import EpilogueIR
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC_DIR = PKG_DIR / "csrc"
+INCLUDE_DIR = PKG_DIR.parent / "include"
+KERNEL_DIR = Path(os.environ.get("EVT_KERNEL_DIR", PKG_DIR / "_kernels"))
+CACHE_FILE = KERNEL_DIR / "compiled_cache.db"
+
+EVT_MAX_TENSORS = 16
+EVT_MAX_SCALARS = 16
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-shared", "-fPIC",
+    # packed-fp32 VALU forms are kept off on this hardware pool
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-value", "-Wno-unknown-attributes",
+]
+
+
+class EvtTensorArg(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("stride_l", ctypes.c_int64), ("stride_m", ctypes.c_int64),
+                ("stride_n", ctypes.c_int64), ("l_div", ctypes.c_int64)]
+
+
+class EvtArgs(ctypes.Structure):
+    _fields_ = [("M", ctypes.c_int32), ("N", ctypes.c_int32), ("K", ctypes.c_int32), ("L", ctypes.c_int32),
+                ("A", ctypes.c_void_p), ("lda", ctypes.c_int64), ("batch_stride_A", ctypes.c_int64),
+                ("B", ctypes.c_void_p), ("ldb", ctypes.c_int64), ("batch_stride_B", ctypes.c_int64),
+                ("num_tensors", ctypes.c_int32), ("num_scalars", ctypes.c_int32),
+                ("tensors", EvtTensorArg * EVT_MAX_TENSORS), ("scalars", ctypes.c_float * EVT_MAX_SCALARS)]
+
+
+ERROR_NAMES = {-1: "EVT_ERR_BAD_ARGS", -2: "EVT_ERR_ALIGNMENT", -3: "EVT_ERR_WORKSPACE", -4: "EVT_ERR_RANGE"}
+
+
+class KernelModule:
+    """A loaded fused-kernel shared object."""
+
+    def __init__(self, path: Path):
+        self.path = Path(path)
+        self.lib = ctypes.CDLL(str(path), mode=ctypes.RTLD_LOCAL)
+        self.lib.evt_abi_version.restype = ctypes.c_int
+        self.lib.evt_module_spec.restype = ctypes.c_char_p
+        self.lib.evt_workspace_bytes.restype = ctypes.c_int64
+        self.lib.evt_workspace_bytes.argtypes = [ctypes.POINTER(EvtArgs)]
+        self.lib.evt_workspace_init.restype = ctypes.c_int
+        self.lib.evt_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        self.lib.evt_launch.restype = ctypes.c_int
+        self.lib.evt_launch.argtypes = [ctypes.POINTER(EvtArgs), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        if self.lib.evt_abi_version() != 1:
+            raise RuntimeError(f"{path}: ABI version mismatch")
+        self.spec = json.loads(self.lib.evt_module_spec().decode())
+
+    def workspace_bytes(self, args: EvtArgs) -> int:
+        n = self.lib.evt_workspace_bytes(ctypes.byref(args))
+        if n < 0:
+            raise RuntimeError(f"evt_workspace_bytes: {ERROR_NAMES.get(n, n)}")
+        return n
+
+    def workspace_init(self, ptr: int, nbytes: int, stream: int) -> None:
+        rc = self.lib.evt_workspace_init(ctypes.c_void_p(ptr), nbytes, ctypes.c_void_p(stream))
+        if rc != 0:
+            raise RuntimeError(f"HIP Error {rc} in evt_workspace_init")
+
+    def launch(self, args: EvtArgs, ws_ptr: int, ws_bytes: int, stream: int) -> None:
+        rc = self.lib.evt_launch(ctypes.byref(args), ctypes.c_void_p(ws_ptr), ws_bytes, ctypes.c_void_p(stream))
+        if rc < 0:
+            raise RuntimeError(f"evt_launch rejected the arguments: {ERROR_NAMES.get(rc, rc)} ({self.path.name})")
+        if rc > 0:
+            # same error class as the reference raises on a failed launch
+            # (python/gtl/ops/reduce_apply_operation.py:157-158)
+            raise RuntimeError(f"HIP Error {rc} launching {self.path.name}")
+
+
+_loaded: Dict[str, KernelModule] = {}
+_lock = threading.Lock()
+
+
+def _db() -> sqlite3.Connection:
+    KERNEL_DIR.mkdir(parents=True, exist_ok=True)
+    con = sqlite3.connect(str(CACHE_FILE), timeout=60)
+    con.execute("CREATE TABLE IF NOT EXISTS compiled_modules("
+                "hash TEXT PRIMARY KEY, name TEXT, file TEXT, spec TEXT)")
+    return con
+
+
+def module_hash(source: str) -> str:
+    h = hashlib.sha256()
+    h.update(source.encode())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    for hdr in sorted(CSRC_DIR.glob("*.hpp")) + [INCLUDE_DIR / "evt_amd.h"]:
+        h.update(hdr.read_bytes())
+    return h.hexdigest()[:20]
+
+
+def compile_source(source: str, out: Path, keep_source: bool = True, extra_flags=()) -> None:
+    out.parent.mkdir(parents=True, exist_ok=True)
+    src = out.with_suffix(".hip")
+    src.write_text(source)
+    tmp = out.with_suffix(f".tmp{os.getpid()}.so")
+    cmd = [HIPCC, *HIPCC_FLAGS, *extra_flags, f"-I{CSRC_DIR}", f"-I{INCLUDE_DIR}", str(src), "-o", str(tmp)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{proc.stderr[-4000:]}")
+    os.replace(tmp, out)
+    if not keep_source:
+        src.unlink()
+
+
+def module_path(ir: EpilogueIR, spec: KernelSpec) -> tuple:
+    name = f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}"
+    source = generate(ir, spec, name)
+    h = module_hash(source)
+    return name, source, h, KERNEL_DIR / f"evt_{h}.so"
+
+
+def build_module(ir: EpilogueIR, spec: KernelSpec, force: bool = False) -> Path:
+    """Generate + compile (if not already built); returns the .so path."""
+    name, source, h, path = module_path(ir, spec)
+    if path.exists() and not force:
+        return path
+    compile_source(source, path)
+    try:
+        con = _db()
+        with con:
+            con.execute("INSERT OR REPLACE INTO compiled_modules VALUES (?,?,?,?)",
+                        (h, name, path.name, json.dumps(Codegen_spec(ir, spec, name))))
+        con.close()
+    except sqlite3.Error:
+        pass   # the index is informational; the file name carries the hash
+    return path
+
+
+def Codegen_spec(ir, spec, name):
+    from .codegen import Codegen
+    return Codegen(ir, spec, name).module_spec()
+
+
+def load_module(ir: EpilogueIR, spec: KernelSpec) -> KernelModule:
+    path = build_module(ir, spec)
+    with _lock:
+        mod = _loaded.get(str(path))
+        if mod is None:
+            mod = KernelModule(path)
+            _loaded[str(path)] = mod
+        return mod

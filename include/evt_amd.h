@@ -1,0 +1,107 @@
+/*
+ * C ABI of one fused GEMM/BMM + epilogue-visitor-tree kernel module for MI355X
+ * (gfx950).
+ *
+ * Every fused kernel the code generator emits is compiled into its own shared
+ * object that exports exactly the symbols declared here (fixed names, loaded
+ * with RTLD_LOCAL so many modules can coexist in one process).  The caller owns
+ * every buffer: inputs, outputs and the workspace; a module never allocates
+ * device memory, never synchronises the device and never reads device memory
+ * from the host, so `evt_launch` can be recorded into a HIP graph.
+ *
+ * What each entry point replaces in the reference (apuaaChen/EVT_AE):
+ *   - the per-kernel `extern "C"` trio `${op}_get_param_size`,
+ *     `${op}_shared_memory_size`, `${op}_get_params` plus the
+ *     `extern "C" __global__ ${op}(Params)` entry that the Python side launches
+ *     (python/gtl/ops/reduce_apply_operation.py:44-86), and
+ *   - for the GEMM/BMM anchors, `GemmArguments(...)` / `BmmArguments2x(...)` +
+ *     `operation.run(arguments, stream)` of the un-vendored CUTLASS Python
+ *     package (python/gtl/compiler/passes/evt_fuser.py:539-546, :674-680,
+ *     python/gtl/ops/bmm.py:23-64).
+ */
+#ifndef EVT_AMD_H_
+#define EVT_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EVT_ABI_VERSION 1
+#define EVT_MAX_TENSORS 16
+#define EVT_MAX_SCALARS 16
+
+/* Error codes returned by evt_launch / evt_workspace_bytes (negative); a
+ * positive value is a hipError_t reported by the runtime at launch. */
+#define EVT_OK 0
+#define EVT_ERR_BAD_ARGS (-1)      /* null pointer, wrong tensor/scalar count   */
+#define EVT_ERR_ALIGNMENT (-2)     /* operand not aligned for this module       */
+#define EVT_ERR_WORKSPACE (-3)     /* workspace missing or too small            */
+#define EVT_ERR_RANGE (-4)         /* a dimension exceeds what the kernel holds */
+
+/* One epilogue tensor (load or store).  Element (l, m, n) of the logical
+ * [L, M, N] iteration space lives at
+ *     ptr + (l / l_div) * stride_l + m * stride_m + n * stride_n   (elements).
+ * A broadcast dimension has stride 0.  Replaces the (M, N, L)-strided
+ * tensor arguments of VisitorAuxLoad / VisitorRowBroadcast / VisitorRowStore
+ * (src/cuda/epilogue/threadblock/visitor_load.hpp:364-571,
+ *  visitor_store.hpp:46-145). */
+typedef struct EvtTensorArg {
+  void* ptr;
+  int64_t stride_l;
+  int64_t stride_m;
+  int64_t stride_n;
+  int64_t l_div;
+} EvtTensorArg;
+
+/* Launch arguments.  A is [L, M, K], B is [L, K, N]; which of the two
+ * dimensions of each operand is contiguous is a compile-time property of the
+ * module (see evt_module_spec).  `lda`/`ldb` are the strides, in elements, of
+ * the non-contiguous dimension; batch strides are in elements and may be 0.
+ * Replaces GemmArguments / BmmArguments2x (evt_fuser.py:539-544, bmm.py:23-64).
+ */
+typedef struct EvtArgs {
+  int32_t M, N, K, L;
+  const void* A;
+  int64_t lda;
+  int64_t batch_stride_A;
+  const void* B;
+  int64_t ldb;
+  int64_t batch_stride_B;
+  int32_t num_tensors;
+  int32_t num_scalars;
+  EvtTensorArg tensors[EVT_MAX_TENSORS];
+  float scalars[EVT_MAX_SCALARS];
+} EvtArgs;
+
+/* ABI version the module was built against (== EVT_ABI_VERSION). */
+int evt_abi_version(void);
+
+/* Static JSON text describing the module: kernel name, tile shape, operand
+ * layouts, alignment requirements, and the name / dtype / role of every tensor
+ * and scalar slot.  Replaces the reference's emitted-source introspection
+ * (`${op}_get_param_size`, reduce_apply_operation.py:44-58). */
+const char* evt_module_spec(void);
+
+/* Bytes of device workspace `evt_launch` needs for these arguments (0 when the
+ * epilogue has no cross-workgroup reduction).  The workspace must be
+ * zero-filled once before its first use (see evt_workspace_init); launches
+ * leave it ready for the next launch.  Replaces the host-side pre-zeroing of
+ * reduction outputs (evt_fuser.py:217-225). */
+int64_t evt_workspace_bytes(const EvtArgs* args);
+
+/* Zero-fill a fresh workspace on `stream` with a fill kernel (graph-safe). */
+int evt_workspace_init(void* workspace, int64_t bytes, void* stream);
+
+/* Enqueue the fused kernel on `stream` (a hipStream_t).  Asynchronous; returns
+ * EVT_OK, a negative EVT_ERR_* code, or a positive hipError_t.  Replaces
+ * `operation.run(arguments, stream=stream.cuda_stream)` (evt_fuser.py:546). */
+int evt_launch(const EvtArgs* args, void* workspace, int64_t workspace_bytes,
+               void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* EVT_AMD_H_ */
