@@ -1,0 +1,192 @@
+"""Tile autotuner base: candidate enumeration, sqlite result cache, timing.
+
+Mirror of python/gtl/compiler/autotuner/tuner_base.py:28-289 of the reference
+(`AutoTunerBase`: sqlite `tuner_cache.db`, key = problem + dtypes + layouts + the
+seven epilogue-node counts :107-152, `get_best_config` :263-270).  The search
+space is this backend's (workgroup tile, wave grid, LDS stages, k-depth,
+raster group) instead of CUTLASS tile descriptions x swizzling functors, and
+timing uses HIP events on the current stream instead of a torch.profiler sum.
+
+Tuning runs only when EVT_AUTOTUNE=1 and a GPU is present; otherwise a cached
+row or the analytic heuristic is used, so tracing never needs a device.
+"""
+from __future__ import annotations
+
+import os
+import sqlite3
+from pathlib import Path
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from ..codegen import KernelSpec, TileConfig
+from ..ir import EpilogueIR
+
+NUM_CUS = 256
+LDS_LIMIT = 160 * 1024
+
+DTYPE_BY_NAME = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32, "bool": torch.bool,
+                 "i32": torch.int32, "i64": torch.int64, "u8": torch.uint8}
+
+
+def default_cache_file() -> Path:
+    return Path(os.environ.get("EVT_TUNER_CACHE", Path(__file__).resolve().parent / "tuner_cache.db"))
+
+
+class AutoTunerBase:
+    table = "best_config"
+    warmup_iterations = 10
+    profile_iterations = 50
+
+    def __init__(self, problem: Tuple[int, int, int, int], a_kc: bool, b_kc: bool, bf16: bool, dma: bool,
+                 ir: EpilogueIR) -> None:
+        self.M, self.N, self.K, self.L = problem
+        self.a_kc, self.b_kc, self.bf16, self.dma, self.ir = a_kc, b_kc, bf16, dma, ir
+        self.cache_file = default_cache_file()
+
+    # -- key (reference: tuner_base.py:107-152, gemm_tuner.py:95-100) -----------
+    def epilogue_key(self) -> str:
+        return "_".join(str(c) for c in self.ir.epilogue_counts())
+
+    def key(self) -> str:
+        e = "bf16" if self.bf16 else "f16"
+        la = "R" if self.a_kc else "C"
+        lb = "C" if self.b_kc else "R"
+        align = "a8" if self.dma else "a1"
+        return f"{self.M}_{self.N}_{self.K}_{e}_{e}_{la}_{lb}_{align}_{self.epilogue_key()}"
+
+    # -- cache -------------------------------------------------------------------
+    def _connect(self) -> sqlite3.Connection:
+        con = sqlite3.connect(str(self.cache_file), timeout=30)
+        con.execute(f"CREATE TABLE IF NOT EXISTS {self.table}(key TEXT PRIMARY KEY, bm INTEGER, bn INTEGER, "
+                    "bk INTEGER, wm INTEGER, wn INTEGER, stages INTEGER, dma INTEGER, group_m INTEGER, us REAL)")
+        return con
+
+    def fetch_cached(self) -> Optional[TileConfig]:
+        if not self.cache_file.exists():
+            return None
+        try:
+            con = self._connect()
+            row = con.execute(f"SELECT bm,bn,bk,wm,wn,stages,dma,group_m FROM {self.table} WHERE key=?",
+                              (self.key(),)).fetchone()
+            con.close()
+        except sqlite3.Error:
+            return None
+        if row is None:
+            return None
+        return TileConfig(row[0], row[1], row[2], row[3], row[4], row[5], bool(row[6]), row[7])
+
+    def store(self, tile: TileConfig, us: float) -> None:
+        con = self._connect()
+        with con:
+            con.execute(f"INSERT OR REPLACE INTO {self.table} VALUES (?,?,?,?,?,?,?,?,?,?)",
+                        (self.key(), tile.bm, tile.bn, tile.bk, tile.wm, tile.wn, tile.stages, int(tile.dma),
+                         tile.group_m, us))
+        con.close()
+
+    # -- search space --------------------------------------------------------------
+    def candidates(self) -> List[TileConfig]:
+        red_lds = lambda t: ((t.wn * t.bm * self.ir.row_state * 4 + 16 if self.ir.row_state else 0) +   # noqa: E731
+                             (t.wm * t.bn * self.ir.col_state * 4 + 16 if self.ir.col_state else 0))
+        out = []
+        if self.dma:
+            shapes = [(256, 256, 64, 4, 2, 2), (256, 256, 32, 4, 2, 3), (256, 256, 32, 4, 2, 4),
+                      (256, 128, 64, 4, 2, 2), (256, 128, 64, 4, 2, 3), (128, 256, 64, 2, 4, 2),
+                      (128, 256, 64, 2, 4, 3), (128, 128, 64, 2, 2, 2), (128, 128, 64, 2, 2, 3),
+                      (128, 128, 32, 2, 2, 4), (64, 64, 64, 2, 2, 2), (64, 64, 32, 2, 2, 2)]
+        else:
+            shapes = [(128, 128, 32, 2, 2, 2), (64, 64, 32, 2, 2, 2)]
+        for bm, bn, bk, wm, wn, st in shapes:
+            for g in ((4, 8) if self.dma else (4,)):
+                t = TileConfig(bm, bn, bk, wm, wn, st, self.dma, g)
+                if t.lds_bytes() <= LDS_LIMIT and t.lds_bytes() >= red_lds(t):
+                    out.append(t)
+        return out
+
+    def heuristic(self) -> TileConfig:
+        """Pick the candidate with the lowest modelled time: number of
+        workgroup rounds on 256 CUs x work per tile / efficiency of the tile."""
+        eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3}
+        best, best_cost = None, None
+        for t in self.candidates():
+            if t.group_m != 4:
+                continue
+            tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
+            wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 else 1
+            rounds = -(-tiles // (NUM_CUS * wg_per_cu))
+            cost = rounds * wg_per_cu * t.bm * t.bn / eff[(t.bm, t.bn)]
+            # deeper k-tiles and fewer stages first on ties
+            cost *= 1.0 + 0.01 * (64 // t.bk - 1) + 0.005 * (t.stages - 2)
+            if best_cost is None or cost < best_cost:
+                best, best_cost = t, cost
+        return best
+
+    # -- timing ----------------------------------------------------------------------
+    def make_arguments(self, module):
+        """Synthetic operands and epilogue tensors for profiling."""
+        from .. import jit
+        dev = "cuda"
+        dt = torch.bfloat16 if self.bf16 else torch.float16
+        M, N, K, L = self.M, self.N, self.K, self.L
+        A = torch.randn(L, M, K, device=dev, dtype=dt) if self.a_kc else torch.randn(L, K, M, device=dev, dtype=dt)
+        B = torch.randn(L, N, K, device=dev, dtype=dt) if self.b_kc else torch.randn(L, K, N, device=dev, dtype=dt)
+        a = jit.EvtArgs()
+        a.M, a.N, a.K, a.L = M, N, K, L
+        a.A, a.lda, a.batch_stride_A = A.data_ptr(), (K if self.a_kc else M), M * K
+        a.B, a.ldb, a.batch_stride_B = B.data_ptr(), (K if self.b_kc else N), N * K
+        a.num_tensors, a.num_scalars = len(self.ir.slots), len(self.ir.scalars)
+        keep = [A, B]
+        for k, s in enumerate(self.ir.slots):
+            st = s.strides
+            span = ((L - 1) // st.l_div) * st.stride_l + (M - 1) * st.stride_m + (N - 1) * st.stride_n + 1
+            dtype = DTYPE_BY_NAME[s.dtype]
+            if dtype.is_floating_point:
+                t = torch.randn(span, device=dev, dtype=torch.float32).to(dtype)
+            else:
+                t = torch.zeros(span, device=dev, dtype=dtype)
+            keep.append(t)
+            ta = a.tensors[k]
+            ta.ptr, ta.stride_l, ta.stride_m, ta.stride_n, ta.l_div = t.data_ptr(), st.stride_l, st.stride_m, st.stride_n, st.l_div
+        for i, v in enumerate(self.ir.scalars):
+            a.scalars[i] = v
+        return a, keep
+
+    def profile(self, tile: TileConfig) -> float:
+        from .. import jit
+        module = jit.load_module(self.ir, KernelSpec(self.a_kc, self.b_kc, self.bf16, tile))
+        args, keep = self.make_arguments(module)
+        stream = torch.cuda.current_stream().cuda_stream
+        nbytes = module.workspace_bytes(args)
+        ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device="cuda")
+        module.workspace_init(ws.data_ptr(), nbytes, stream)
+        for _ in range(self.warmup_iterations):
+            module.launch(args, ws.data_ptr(), nbytes, stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(self.profile_iterations):
+            module.launch(args, ws.data_ptr(), nbytes, stream)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / self.profile_iterations
+
+    def tune(self) -> TileConfig:
+        best, best_us = None, None
+        for tile in self.candidates():
+            try:
+                us = self.profile(tile)
+            except RuntimeError:
+                continue
+            if best_us is None or us < best_us:
+                best, best_us = tile, us
+        if best is None:
+            return self.heuristic()
+        self.store(best, best_us)
+        return best
+
+    def get_best_config(self) -> TileConfig:
+        cached = self.fetch_cached()
+        if cached is not None:
+            return cached
+        if os.environ.get("EVT_AUTOTUNE", "0") == "1" and torch.cuda.is_available():
+            return self.tune()
+        return self.heuristic()

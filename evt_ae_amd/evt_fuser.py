@@ -49,7 +49,7 @@ def target_name(target) -> str:
 def node_shape_dtype(node: Node) -> Tuple[Tuple[int, ...], torch.dtype]:
     if "tensor_meta" in node.meta:
         tm = node.meta["tensor_meta"]
-        if isinstance(tm, (tuple, list)):
+        if not hasattr(tm, "shape"):
             raise ValueError(f"{node.name} produces several tensors")
         return tuple(int(s) for s in tm.shape), tm.dtype
     if "val" in node.meta and isinstance(node.meta["val"], torch.Tensor):
@@ -102,7 +102,11 @@ class FusedOpBase:
         """-> (A, lda, batch_stride_A, B, ldb, batch_stride_B) ready for the kernel."""
         raise NotImplementedError("Should be Overwritten by child class")
 
-    def call(self, visitor_args: Dict[str, torch.Tensor], stream, *args) -> Any:
+    def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args) -> Tuple[jit.EvtArgs, list]:
+        """Marshal operands and epilogue tensors into the C-ABI argument block
+        (the counterpart of GemmArguments / BmmArguments2x +
+        operation.epilogue_type(visitor_args), evt_fuser.py:539-544, :674-678).
+        Returns the block and the tensors it points into (keep them alive)."""
         M, N, K, L = self.problem
         A, lda, bsa, B, ldb, bsb = self.operands(args[-2], args[-1])
         a = jit.EvtArgs()
@@ -122,16 +126,31 @@ class FusedOpBase:
             ta.l_div = slot.strides.l_div
         for i, s in enumerate(self.ir.scalars):
             a.scalars[i] = s
+        return a, keep
+
+    def workspace_for(self, a: jit.EvtArgs, stream, device) -> Tuple[int, int]:
+        """Device workspace for cross-workgroup reductions, one per stream,
+        zero-filled once (launches leave it clean)."""
         ws_bytes = self.module.workspace_bytes(a)
-        ws_ptr = 0
-        if ws_bytes:
-            key = stream.cuda_stream
-            ws = self._workspace.get(key)
-            if ws is None or ws.numel() < ws_bytes:
-                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=A.device)
-                self.module.workspace_init(ws.data_ptr(), ws_bytes, stream.cuda_stream)
-                self._workspace[key] = ws
-            ws_ptr = ws.data_ptr()
+        if not ws_bytes:
+            return 0, 0
+        key = stream.cuda_stream
+        ws = self._workspace.get(key)
+        if ws is None or ws.numel() < ws_bytes:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
+            self.module.workspace_init(ws.data_ptr(), ws_bytes, stream.cuda_stream)
+            self._workspace[key] = ws
+        return ws.data_ptr(), ws_bytes
+
+    def allocate_outputs(self, device) -> Dict[str, torch.Tensor]:
+        # one buffer per distinct store; reduction outputs need no zero fill
+        # (the reference zero-fills them for its atomics, evt_fuser.py:217-225)
+        return {name: torch.empty(shape, dtype=dtype, device=device)
+                for name, (shape, dtype) in self.store_meta.items()}
+
+    def call(self, visitor_args: Dict[str, torch.Tensor], stream, *args) -> Any:
+        a, keep = self.build_arguments(visitor_args, *args)
+        ws_ptr, ws_bytes = self.workspace_for(a, stream, keep[0].device)
         self.module.launch(a, ws_ptr, ws_bytes, stream.cuda_stream)
 
     def get_output_name(self, output: Node) -> str:
@@ -156,10 +175,7 @@ class FusedOpBase:
 
         with torch.cuda.stream(stream):
             device = args[-1].device
-            visitor_args: Dict[str, torch.Tensor] = {}
-            # one buffer per distinct store; reduction outputs need no zero fill
-            for name, (shape, dtype) in self.store_meta.items():
-                visitor_args[name] = torch.empty(shape, dtype=dtype, device=device)
+            visitor_args = self.allocate_outputs(device)
             for idx, input_name in enumerate(self.input_names):
                 visitor_args.setdefault(input_name, args[idx])
 
@@ -816,7 +832,9 @@ class EVTFuser:
         sel = f"{node.name}_sel"
         zero = self.ir.add_imm(0.0)
         self.ir.add_compute(sel, "where", [hit, self.ir_name[x], zero])
-        return self._reduce(node, sel, cx, [len(xshape) - 1], True, "sum")
+        (n,) = self._reduce(node, sel, cx, [len(xshape) - 1], True, "sum")
+        self.ir_name[node] = n
+        return n
 
     # -- reductions ------------------------------------------------------------------
     def _reduce(self, node: Node, value: str, coord: Coord, dims, keepdim: bool, kind: str,

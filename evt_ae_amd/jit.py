@@ -117,7 +117,7 @@ def module_hash(source: str) -> str:
     return h.hexdigest()[:20]
 
 
-def compile_source(source: str, out: Path, keep_source: bool = True, extra_flags=()) -> None:
+def compile_source(source: str, out: Path, extra_flags=()) -> None:
     out.parent.mkdir(parents=True, exist_ok=True)
     src = out.with_suffix(".hip")
     src.write_text(source)
@@ -127,44 +127,78 @@ def compile_source(source: str, out: Path, keep_source: bool = True, extra_flags
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{proc.stderr[-4000:]}")
     os.replace(tmp, out)
-    if not keep_source:
-        src.unlink()
 
 
-def module_path(ir: EpilogueIR, spec: KernelSpec) -> tuple:
-    name = f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}"
-    source = generate(ir, spec, name)
-    h = module_hash(source)
-    return name, source, h, KERNEL_DIR / f"evt_{h}.so"
-
-
-def build_module(ir: EpilogueIR, spec: KernelSpec, force: bool = False) -> Path:
-    """Generate + compile (if not already built); returns the .so path."""
-    name, source, h, path = module_path(ir, spec)
-    if path.exists() and not force:
-        return path
-    compile_source(source, path)
+def _record(h: str, name: str, path: Path, spec_json: str) -> None:
     try:
         con = _db()
         with con:
-            con.execute("INSERT OR REPLACE INTO compiled_modules VALUES (?,?,?,?)",
-                        (h, name, path.name, json.dumps(Codegen_spec(ir, spec, name))))
+            con.execute("INSERT OR REPLACE INTO compiled_modules VALUES (?,?,?,?)", (h, name, path.name, spec_json))
         con.close()
     except sqlite3.Error:
         pass   # the index is informational; the file name carries the hash
-    return path
 
 
-def Codegen_spec(ir, spec, name):
-    from .codegen import Codegen
-    return Codegen(ir, spec, name).module_spec()
+class LazyModule:
+    """A kernel module identified at trace time and compiled / loaded on first
+    use, so that tracing a graph never needs hipcc or a GPU.  Modules built
+    ahead of time (evt_ae_amd.prebuild) are found by their hash."""
+
+    def __init__(self, ir: EpilogueIR, spec: KernelSpec):
+        from .codegen import Codegen
+        self.ir, self.kernel_spec = ir, spec
+        self.name = f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}"
+        cg = Codegen(ir, spec, self.name)
+        self.source = cg.source()
+        self.spec_json = json.dumps(cg.module_spec(), sort_keys=True)
+        self.hash = module_hash(self.source)
+        self.path = KERNEL_DIR / f"evt_{self.hash}.so"
+        self._mod: Optional[KernelModule] = None
+
+    def build(self, force: bool = False) -> Path:
+        if force or not self.path.exists():
+            compile_source(self.source, self.path)
+            _record(self.hash, self.name, self.path, self.spec_json)
+        return self.path
+
+    def ensure(self) -> KernelModule:
+        if self._mod is None:
+            self.build()
+            with _lock:
+                mod = _loaded.get(str(self.path))
+                if mod is None:
+                    mod = KernelModule(self.path)
+                    _loaded[str(self.path)] = mod
+                self._mod = mod
+        return self._mod
+
+    @property
+    def spec(self) -> dict:
+        return json.loads(self.spec_json)
+
+    def workspace_bytes(self, args: EvtArgs) -> int:
+        return self.ensure().workspace_bytes(args)
+
+    def workspace_init(self, ptr: int, nbytes: int, stream: int) -> None:
+        self.ensure().workspace_init(ptr, nbytes, stream)
+
+    def launch(self, args: EvtArgs, ws_ptr: int, ws_bytes: int, stream: int) -> None:
+        self.ensure().launch(args, ws_ptr, ws_bytes, stream)
 
 
-def load_module(ir: EpilogueIR, spec: KernelSpec) -> KernelModule:
-    path = build_module(ir, spec)
+_registry: Dict[str, LazyModule] = {}
+
+
+def load_module(ir: EpilogueIR, spec: KernelSpec) -> LazyModule:
+    mod = LazyModule(ir, spec)
     with _lock:
-        mod = _loaded.get(str(path))
-        if mod is None:
-            mod = KernelModule(path)
-            _loaded[str(path)] = mod
-        return mod
+        return _registry.setdefault(str(mod.path), mod)
+
+
+def registered_modules():
+    with _lock:
+        return list(_registry.values())
+
+
+def build_module(ir: EpilogueIR, spec: KernelSpec, force: bool = False) -> Path:
+    return load_module(ir, spec).build(force)

@@ -1,0 +1,81 @@
+"""Ahead-of-time build of every kernel module the tests, the smoke check and the
+benchmark use, so that nothing has to be compiled on the GPU box.
+
+Each workload is traced on meta tensors (no data, no GPU) exactly as it will be
+at run time, which registers its kernel module; the modules are then compiled
+in parallel with hipcc for gfx950.  The reference has no counterpart: it JITs
+through nvcc on first use and keeps cubins in compiled_cache.db.
+"""
+from __future__ import annotations
+
+import sys
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import List
+
+import torch
+
+from . import jit, workloads as W
+
+
+def _meta(inputs):
+    return [torch.empty(t.shape, dtype=t.dtype, device="meta") for t in inputs]
+
+
+def _shapes_of(cfg: int, shapes: dict):
+    """Input shapes/dtypes without materialising full-size random data."""
+    import inspect
+    fn = W.CONFIGS[cfg].make_inputs
+    sig = inspect.signature(fn)
+    kw = {k: v.default for k, v in list(sig.parameters.items())[1:]}
+    kw.update(shapes or {})
+
+    class _G:   # shape-only stand-in for torch.Generator
+        pass
+    shapes_only = {
+        1: lambda M, N, K: [((M, K), torch.half), ((K, N), torch.half), ((N,), torch.half)],
+        2: lambda L, S, D: [((L, S, D), torch.half), ((L, S, D), torch.half)],
+        3: lambda M, N, K: [((M, K), torch.half), ((K, N), torch.half), ((N,), torch.half), ((M, N), torch.half)],
+        4: lambda M, N, K: [((M, K), torch.half), ((N, K), torch.half), ((M, N), torch.half)],
+        5: lambda M, N, K: [((M, K), torch.half), ((K, N), torch.half), ((M,), torch.int32)],
+    }[cfg](**kw)
+    return [torch.empty(s, dtype=d, device="meta") for s, d in shapes_only]
+
+
+def register_all() -> List[jit.LazyModule]:
+    for cfg in W.CONFIGS:
+        for shapes in (None, W.SMALL_SHAPES[cfg], W.RAGGED_SHAPES[cfg], W.UNALIGNED_SHAPES[cfg], W.GOLDEN_SHAPES[cfg]):
+            W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
+    for name, (cls, _) in W.REFERENCE_PATTERNS.items():
+        g = torch.Generator(device="cpu").manual_seed(0)
+        # shapes only: generate on CPU lazily is costly for the big patterns, so
+        # take shapes from a meta run of the generator functions
+        with torch.device("meta"):
+            pass
+        ins = W.pattern_inputs(name) if name not in ("mm10", "mm11") else None
+        if ins is None:
+            shapes = {"mm10": [(16384, 1024), (1024, 4096)], "mm11": [(33792, 768), (33792, 768)]}[name]
+            metas = [torch.empty(s, dtype=torch.half, device="meta") for s in shapes]
+        else:
+            metas = _meta(ins)
+        W.fuse(cls(), metas)
+    return jit.registered_modules()
+
+
+def build_all(jobs: int = 8, force: bool = False, verbose: bool = True) -> List[jit.LazyModule]:
+    mods = register_all()
+    todo = [m for m in mods if force or not m.path.exists()]
+    t0 = time.time()
+    if verbose:
+        print(f"[prebuild] {len(mods)} modules registered, {len(todo)} to compile", flush=True)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        for m, _ in zip(todo, pool.map(lambda mod: mod.build(force=force), todo)):
+            if verbose:
+                print(f"[prebuild] built {m.name} -> {m.path.name}", flush=True)
+    if verbose:
+        print(f"[prebuild] done in {time.time() - t0:.1f}s", flush=True)
+    return mods
+
+
+if __name__ == "__main__":
+    build_all(force="--force" in sys.argv)

@@ -1,0 +1,392 @@
+"""The fused-subgraph workloads this backend is measured and tested on.
+
+`CONFIGS` holds the five headline subgraphs (FFN up-projection + GELU,
+attention scores + softmax statistics, output projection + residual +
+LayerNorm statistics, FFN backward + bias gradient, classifier + cross
+entropy), written as ATen-level modules the way the reference's own fuser
+tests are (unittest/evt_fuser/mm.py:30-236, bmm.py:29-94), each with its seeded
+input generator, algorithmic flop / byte counts and output roles.
+`REFERENCE_PATTERNS` restates the graph patterns of those reference tests.
+"""
+from __future__ import annotations
+
+import operator
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Sequence, Tuple
+
+import torch
+from torch.fx import GraphModule, symbolic_trace
+from torch.fx.passes.shape_prop import ShapeProp
+
+aten = torch.ops.aten
+
+
+# ---------------------------------------------------------------------------
+# the five headline configurations
+# ---------------------------------------------------------------------------
+
+class FFNUpGelu(torch.nn.Module):
+    """Y = GELU_tanh(X W + b)"""
+    def forward(self, x, w, b):
+        mm = aten.mm(x, w)
+        add = aten.add(mm, b)
+        gelu = aten.gelu(add, approximate="tanh")
+        return gelu
+
+
+class AttnScoreSoftmaxStats(torch.nn.Module):
+    """S = (Q K^T) / 8 ; per-row max and sum-exp of S"""
+    def forward(self, q, k):
+        kt = aten.permute(k, [0, 2, 1])
+        bmm = aten.bmm(q, kt)
+        s = aten.mul(bmm, 0.125)
+        sf = aten._to_copy(s, dtype=torch.float32)
+        m = aten.amax(sf, [-1], True)
+        sub = aten.sub(sf, m)
+        e = aten.exp(sub)
+        l = aten.sum(e, [-1], True)
+        return s, m, l
+
+
+class OutProjResidualLNStats(torch.nn.Module):
+    """O = X W + b + R ; per-row mean and (biased) variance of O"""
+    def forward(self, x, w, b, r):
+        mm = aten.mm(x, w)
+        add = aten.add(mm, b)
+        o = aten.add(add, r)
+        of = aten._to_copy(o, dtype=torch.float32)
+        vm = aten.var_mean(of, [1], correction=0, keepdim=False)
+        var = operator.getitem(vm, 0)
+        mean = operator.getitem(vm, 1)
+        return o, mean, var
+
+
+class FFNBackwardDBias(torch.nn.Module):
+    """dP = (dY W^T) * GELU_tanh'(P) ; dbias = sum_m dP"""
+    def forward(self, dy, w, p):
+        wt = aten.permute(w, [1, 0])
+        mm = aten.mm(dy, wt)
+        dp = aten.gelu_backward(mm, p, approximate="tanh")
+        dpf = aten._to_copy(dp, dtype=torch.float32)
+        db = aten.sum(dpf, [0])
+        return dp, db
+
+
+class ClassifierCrossEntropy(torch.nn.Module):
+    """loss_m = logsumexp_n(H W) - (H W)[m, label_m]   (logits never stored)"""
+    def forward(self, h, w, labels):
+        mm = aten.mm(h, w)
+        lf = aten._to_copy(mm, dtype=torch.float32)
+        lse = aten.logsumexp(lf, [1])
+        idx64 = aten._to_copy(labels, dtype=torch.int64)
+        idx = aten.unsqueeze(idx64, 1)
+        z = aten.gather(lf, 1, idx)
+        zs = aten.squeeze(z, 1)
+        loss = aten.sub(lse, zs)
+        return loss
+
+
+def _randn(g, shape, scale=1.0):
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * scale).half()
+
+
+@dataclass
+class Workload:
+    name: str
+    module: Callable[[], torch.nn.Module]
+    make_inputs: Callable[[torch.Generator, float], List[torch.Tensor]]   # (generator, size scale) -> CPU tensors
+    dims: Tuple[int, int, int, int]          # M, N, K, L at full size
+    flops: int
+    bytes: int
+    reduction_outputs: Tuple[int, ...] = ()  # indices of fp32 reduction outputs (tolerance 1e-3)
+    description: str = ""
+
+    def seed(self, cfg_index: int) -> int:
+        return 0xE7A0 + cfg_index
+
+
+def _cfg1(g, M=4096, N=4096, K=1024):
+    return [_randn(g, (M, K)), _randn(g, (K, N), 0.02), _randn(g, (N,), 0.02)]
+
+
+def _cfg2(g, L=64, S=512, D=64):
+    return [_randn(g, (L, S, D)), _randn(g, (L, S, D))]
+
+
+def _cfg3(g, M=8192, N=1024, K=4096):
+    return [_randn(g, (M, K)), _randn(g, (K, N), 0.02), _randn(g, (N,), 0.02), _randn(g, (M, N))]
+
+
+def _cfg4(g, M=8192, N=1024, K=4096):
+    return [_randn(g, (M, K), 0.01), _randn(g, (N, K), 0.02), _randn(g, (M, N))]
+
+
+def _cfg5(g, M=1024, N=131072, K=512):
+    h = _randn(g, (M, K))
+    w = _randn(g, (K, N), 0.02)
+    labels = torch.randint(0, N, (M,), generator=g, dtype=torch.int64).to(torch.int32)
+    return [h, w, labels]
+
+
+CONFIGS: Dict[int, Workload] = {
+    1: Workload("ffn_up_gelu", FFNUpGelu, _cfg1, (4096, 4096, 1024, 1), 34_359_738_368, 50_339_840, (),
+                "BERT-large FFN up-projection: GELU_tanh(XW+b)"),
+    2: Workload("attn_score_softmax_stats", AttnScoreSoftmaxStats, _cfg2, (512, 512, 64, 64), 2_147_483_648,
+                42_205_184, (1, 2), "QK^T/8 + per-row max and sum-exp"),
+    3: Workload("out_proj_residual_ln_stats", OutProjResidualLNStats, _cfg3, (8192, 1024, 4096, 1),
+                68_719_476_736, 109_119_488, (1, 2), "XW+b+R + per-row mean/var"),
+    4: Workload("ffn_backward_dbias", FFNBackwardDBias, _cfg4, (8192, 1024, 4096, 1), 68_719_476_736,
+                109_056_000, (1,), "(dY W^T) * GELU'(P) + column sum"),
+    5: Workload("classifier_cross_entropy", ClassifierCrossEntropy, _cfg5, (1024, 131072, 512, 1),
+                137_438_953_472, 135_274_496, (0,), "HW -> per-row CE loss"),
+}
+
+# small instances of the same graphs (shape arguments for make_inputs) used by
+# parity tests where the CPU oracle must finish in seconds
+SMALL_SHAPES = {
+    1: dict(M=256, N=384, K=128),
+    2: dict(L=3, S=192, D=64),
+    3: dict(M=320, N=640, K=256),
+    4: dict(M=512, N=320, K=192),
+    5: dict(M=128, N=4096, K=128),
+}
+RAGGED_SHAPES = {
+    1: dict(M=100, N=72, K=40),
+    2: dict(L=2, S=77, D=24),
+    3: dict(M=33, N=136, K=72),
+    4: dict(M=130, N=56, K=88),
+    5: dict(M=37, N=1000, K=64),
+}
+# shapes of the committed golden fixtures (tests/golden)
+GOLDEN_SHAPES = {
+    1: dict(M=64, N=96, K=64),
+    2: dict(L=2, S=64, D=32),
+    3: dict(M=64, N=128, K=64),
+    4: dict(M=96, N=64, K=64),
+    5: dict(M=32, N=512, K=64),
+}
+# no dimension a multiple of 8: operands are not 16-byte aligned row by row, so
+# these run the element-wise (safe) operand path
+UNALIGNED_SHAPES = {
+    1: dict(M=33, N=17, K=41),
+    2: dict(L=2, S=45, D=19),
+    3: dict(M=70, N=129, K=33),
+    4: dict(M=65, N=31, K=50),
+    5: dict(M=19, N=333, K=27),
+}
+
+
+def make_inputs(cfg: int, shapes: dict = None, seed: int = None) -> List[torch.Tensor]:
+    g = torch.Generator(device="cpu").manual_seed(CONFIGS[cfg].seed(cfg) if seed is None else seed)
+    fn = CONFIGS[cfg].make_inputs
+    return fn(g, **(shapes or {}))
+
+
+def unfused_eager(cfg: int) -> Callable:
+    """The literal unfused GPU sequence (rocBLAS/hipBLASLt GEMM + one eager
+    kernel per epilogue op) the fused kernel is compared with."""
+    F = torch.nn.functional
+    if cfg == 1:
+        return lambda x, w, b: F.gelu(torch.mm(x, w) + b, approximate="tanh")
+    if cfg == 2:
+        def f(q, k):
+            s = torch.bmm(q, k.transpose(1, 2)) * 0.125
+            sf = s.float()
+            m = sf.amax(-1, keepdim=True)
+            return s, m, (sf - m).exp().sum(-1, keepdim=True)
+        return f
+    if cfg == 3:
+        def f(x, w, b, r):
+            o = torch.mm(x, w) + b + r
+            var, mean = torch.var_mean(o.float(), dim=1, correction=0)
+            return o, mean, var
+        return f
+    if cfg == 4:
+        def f(dy, w, p):
+            dp = aten.gelu_backward(torch.mm(dy, w.t()), p, approximate="tanh")
+            return dp, dp.float().sum(0)
+        return f
+    if cfg == 5:
+        def f(h, w, labels):
+            lf = torch.mm(h, w).float()
+            return torch.logsumexp(lf, 1) - lf.gather(1, labels.long().unsqueeze(1)).squeeze(1)
+        return f
+    raise KeyError(cfg)
+
+
+# ---------------------------------------------------------------------------
+# tracing helper (symbolic_trace + ShapeProp on meta tensors: no data needed)
+# ---------------------------------------------------------------------------
+
+def trace_module(module: torch.nn.Module, example_inputs: Sequence[torch.Tensor]) -> GraphModule:
+    gm = symbolic_trace(module)
+    metas = [t.to("meta") if isinstance(t, torch.Tensor) else t for t in example_inputs]
+    ShapeProp(gm).propagate(*metas)
+    return gm
+
+
+def fused_nodes(gm: GraphModule):
+    """The fused-kernel call nodes `EVTFuser.trace` placed in `gm` (meta["evt"])."""
+    return [n for n in gm.graph.nodes if n.op == "call_function" and n.meta.get("evt")]
+
+
+def fuse(module: torch.nn.Module, example_inputs: Sequence[torch.Tensor], passes=None) -> GraphModule:
+    """symbolic_trace -> ShapeProp -> pass_fusion -> recompile, as the
+    reference's UnitTestBase.util_test does (python/gtl/helper/test_helper.py:78-96)."""
+    from .passes import pass_fusion
+    gm = trace_module(module, example_inputs)
+    for p in (passes or [pass_fusion]):
+        p(gm, gm.graph)
+    gm.recompile()
+    return gm
+
+
+# ---------------------------------------------------------------------------
+# graph patterns of the reference's fuser tests
+# ---------------------------------------------------------------------------
+
+class MMPartition1(torch.nn.Module):   # mm.py:30-50  bias + GELU, two stores through views
+    def forward(self, primals_1, view_11, primals_2):
+        permute_24 = aten.permute(primals_1, [1, 0])
+        mm_37 = aten.mm(view_11, permute_24)
+        add_21 = aten.add(mm_37, primals_2)
+        view_12 = aten.view(add_21, [512, 2, 4096])
+        gelu = aten.gelu(view_12, approximate="tanh")
+        view_13 = aten.view(gelu, [1024, 4096])
+        return view_13, view_12
+
+
+class MMPartition2(torch.nn.Module):   # mm.py:52-70  tiny M, bias + tanh
+    def forward(self, select, primals_5, primals_6):
+        permute_32 = aten.permute(primals_5, [1, 0])
+        mm_45 = aten.mm(select, permute_32)
+        add_29 = aten.add(mm_45, primals_6)
+        tanh = aten.tanh(add_29)
+        return tanh
+
+
+class MMPartition3(torch.nn.Module):   # mm.py:72-91  view before the bias add
+    def forward(self, view_93, primals_10, primals_11):
+        permute_112 = aten.permute(primals_10, [1, 0])
+        mm = aten.mm(view_93, permute_112)
+        view = aten.view(mm, [512, 2, 1024])
+        add = aten.add(view, primals_11)
+        view_3 = aten.view(add, [512, 32, 64])
+        return view_3
+
+
+class MMPartition4(torch.nn.Module):   # mm.py:93-111  N = 2
+    def forward(self, tanh, primals_41, primals_42):
+        permute_123 = aten.permute(primals_41, [1, 0])
+        mm_47 = aten.mm(tanh, permute_123)
+        add = aten.add(mm_47, primals_42)
+        view_39 = aten.view(add, [2, 2])
+        return view_39
+
+
+class MMPartition5(torch.nn.Module):   # mm.py:113-127  tanh_backward + column sum, K = 2
+    def forward(self, A, B, tanh):
+        mm = aten.mm(A, B)
+        out = aten.tanh_backward(mm, tanh)
+        sum = aten.sum(out, [0], True)
+        return out, sum
+
+
+class MMPartition6(torch.nn.Module):   # mm.py:129-146  residual adds, permuted output
+    def forward(self, view_295, primals_12, add_17, view_299):
+        mm_33 = aten.mm(view_295, primals_12)
+        view_298 = aten.view(mm_33, [512, 4, 1024])
+        add_18 = aten.add(view_298, add_17)
+        add_19 = aten.add(add_18, view_299)
+        permute_183 = aten.permute(add_19, [1, 0, 2])
+        return permute_183
+
+
+class MMPartition7(torch.nn.Module):   # mm.py:148-165  four outputs
+    def forward(self, view_295, primals_12, add_17, view_299):
+        mm_33 = aten.mm(view_295, primals_12)
+        view_298 = aten.view(mm_33, [512, 4, 1024])
+        add_18 = aten.add(view_298, add_17)
+        add_19 = aten.add(add_18, view_299)
+        view_183 = aten.view(add_19, [2048, 1024])
+        return view_298, add_18, add_19, view_183
+
+
+class MMPartition9(torch.nn.Module):   # mm.py:167-186  bias used twice
+    def forward(self, select, primals_5, primals_6):
+        permute_32 = aten.permute(primals_5, [1, 0])
+        mm_45 = aten.mm(select, permute_32)
+        add_29 = aten.add(mm_45, primals_6)
+        tanh = aten.tanh(add_29)
+        add_30 = aten.add(tanh, primals_6)
+        return add_30
+
+
+class MMPartition10(torch.nn.Module):  # mm.py:188-200  store + column sum, large M
+    def forward(self, view_237, primals_34):
+        mm_12 = aten.mm(view_237, primals_34)
+        sum_6 = aten.sum(mm_12, [0], True)
+        return mm_12, sum_6
+
+
+class MMPartition11(torch.nn.Module):  # mm.py:202-214  weight gradient A^T B
+    def forward(self, view_206, view_160):
+        permute_142 = aten.permute(view_206, [1, 0])
+        mm_9 = aten.mm(permute_142, view_160)
+        return mm_9
+
+
+class BMMPartition1(torch.nn.Module):  # bmm.py:29-46  permuted B, permuted + reshaped store
+    def forward(self, view_5, view_7):
+        permute_127 = aten.permute(view_5, [1, 0, 2])
+        bmm_1 = aten.bmm(view_7, permute_127)
+        permute_132 = aten.permute(bmm_1, [1, 0, 2])
+        clone_3 = aten.clone(permute_132, memory_format=torch.contiguous_format)
+        view_8 = aten.view(clone_3, [512, 2, 1024])
+        view_9 = aten.view(view_8, [1024, 1024])
+        return view_9
+
+
+class BMMPartition3(torch.nn.Module):  # bmm.py:69-94  QK^T * scale + additive mask (mask output kept outside)
+    def forward(self, view_3, view_4, primals_44, const_scalar0, const_scalar1, inv_const_scalar2):
+        unsqueeze = aten.unsqueeze(primals_44, 1)
+        unsqueeze_1 = aten.unsqueeze(unsqueeze, 2)
+        mul_40 = aten.mul(unsqueeze_1, -1.0)
+        add_37 = aten.add(mul_40, const_scalar0)
+        mul_1 = aten.mul(add_37, const_scalar1)
+        permute_125 = aten.permute(view_3, [1, 0, 2])
+        permute_126 = aten.permute(view_4, [1, 2, 0])
+        bmm = aten.bmm(permute_125, permute_126)
+        view_6 = aten.view(bmm, [2, 16, 512, 512])
+        mul = aten.mul(view_6, inv_const_scalar2)
+        add_3 = aten.add(mul, mul_1)
+        return add_3, mul_1
+
+
+def _h(g, shape, scale=1.0):
+    return _randn(g, shape, scale)
+
+
+# name -> (module class, input generator(generator) -> CPU tensors, allclose criteria of the reference test)
+REFERENCE_PATTERNS = {
+    "mm1": (MMPartition1, lambda g: [_h(g, (4096, 1024), 0.03), _h(g, (1024, 1024)), _h(g, (4096,))]),
+    "mm2": (MMPartition2, lambda g: [_h(g, (4, 1024)), _h(g, (1024, 1024), 0.018), _h(g, (1024,), 0.018)]),
+    "mm3": (MMPartition3, lambda g: [_h(g, (1024, 1024)), _h(g, (1024, 1024), 0.03), _h(g, (1024,))]),
+    "mm4": (MMPartition4, lambda g: [_h(g, (2, 1024)), _h(g, (2, 1024), 0.03), _h(g, (2,))]),
+    "mm5": (MMPartition5, lambda g: [_h(g, (4, 2)), _h(g, (2, 1024)), torch.tanh(_h(g, (4, 1024)).float()).half()]),
+    "mm6": (MMPartition6, lambda g: [_h(g, (2048, 1024)), _h(g, (1024, 1024), 0.03), _h(g, (512, 4, 1024)),
+                                     _h(g, (512, 4, 1024))]),
+    "mm7": (MMPartition7, lambda g: [_h(g, (2048, 1024)), _h(g, (1024, 1024), 0.03), _h(g, (512, 4, 1024)),
+                                     _h(g, (512, 4, 1024))]),
+    "mm9": (MMPartition9, lambda g: [_h(g, (4, 1024)), _h(g, (1024, 1024), 0.018), _h(g, (1024,), 0.018)]),
+    "mm10": (MMPartition10, lambda g: [_h(g, (16384, 1024), 0.05), _h(g, (1024, 4096), 0.05)]),
+    "mm11": (MMPartition11, lambda g: [_h(g, (33792, 768), 0.01), _h(g, (33792, 768))]),
+    "bmm1": (BMMPartition1, lambda g: [_h(g, (512, 32, 64)), _h(g, (32, 512, 512), 0.05)]),
+    "bmm3": (BMMPartition3, lambda g: [_h(g, (512, 32, 64)), _h(g, (512, 32, 64), 0.2), _h(g, (2, 512)),
+                                       _h(g, (1,)), _h(g, (1,)), _h(g, (1,))]),
+}
+
+
+def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
+    g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
+    return REFERENCE_PATTERNS[name][1](g)

@@ -1,0 +1,137 @@
+"""The C-ABI boundary without a GPU: every built kernel module loads, exports
+exactly the symbols include/evt_amd.h declares, describes itself, and rejects
+malformed arguments with the documented error codes before any launch."""
+import ctypes
+import json
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from evt_ae_amd import jit, workloads as W
+from tests.util import fused_nodes
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "evt_amd.h"
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(evt_[a-z_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def module():
+    inputs = W.make_inputs(3, W.SMALL_SHAPES[3])
+    gm = W.fuse(W.CONFIGS[3].module(), [t.to("meta") for t in inputs])
+    (n,) = fused_nodes(gm)
+    return n.target, n.target.module.ensure()
+
+
+def test_header_declares_the_expected_entry_points():
+    assert declared_symbols() == ["evt_abi_version", "evt_launch", "evt_module_spec", "evt_workspace_bytes",
+                                  "evt_workspace_init"]
+
+
+def test_every_built_module_exports_the_abi():
+    paths = sorted(jit.KERNEL_DIR.glob("evt_*.so"))
+    if not paths:
+        pytest.skip("no kernel modules built yet")
+    for p in paths:
+        lib = ctypes.CDLL(str(p), mode=ctypes.RTLD_LOCAL)
+        for sym in declared_symbols():
+            assert hasattr(lib, sym), f"{p.name} lacks {sym}"
+        lib.evt_abi_version.restype = ctypes.c_int
+        assert lib.evt_abi_version() == 1
+        lib.evt_module_spec.restype = ctypes.c_char_p
+        spec = json.loads(lib.evt_module_spec().decode())
+        assert spec["abi"] == 1 and spec["element"] in ("f16", "bf16") and "tile" in spec
+
+
+def test_struct_layout_matches_header():
+    # EvtTensorArg: pointer + 4 x int64 ; EvtArgs: 4 x int32, 2 x (ptr, int64, int64), 2 x int32, arrays
+    assert ctypes.sizeof(jit.EvtTensorArg) == 40
+    assert ctypes.sizeof(jit.EvtArgs) == 16 + 48 + 8 + 16 * 40 + 16 * 4
+    assert jit.EvtArgs.tensors.offset == 72 and jit.EvtArgs.scalars.offset == 72 + 640
+
+
+def test_module_spec_describes_slots(module):
+    op, km = module
+    spec = km.spec
+    assert spec["row_state"] == 3 and spec["col_state"] == 0 and not spec["batched"]
+    assert [t["role"] for t in spec["tensors"]] == ["load", "load", "store", "store", "store"]
+    assert [t["kind"] for t in spec["tensors"]] == ["row", "aux", "aux", "col", "col"]
+
+
+def _args(op, km):
+    M, N, K, L = op.problem
+    a = jit.EvtArgs()
+    a.M, a.N, a.K, a.L = M, N, K, L
+    a.A, a.lda, a.B, a.ldb = 0x10000, K, 0x20000, N
+    a.num_tensors, a.num_scalars = len(op.ir.slots), len(op.ir.scalars)
+    for k in range(a.num_tensors):
+        a.tensors[k].ptr = 0x30000 + 0x1000 * k
+        a.tensors[k].l_div = 1
+    return a
+
+
+def test_argument_validation_happens_before_launch(module):
+    op, km = module
+    a = _args(op, km)
+    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) >= 0
+    bad = _args(op, km); bad.num_tensors -= 1
+    assert km.lib.evt_workspace_bytes(ctypes.byref(bad)) == -1          # EVT_ERR_BAD_ARGS
+    bad = _args(op, km); bad.A = 0
+    assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -1
+    bad = _args(op, km); bad.A = 0x10002
+    assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -2    # EVT_ERR_ALIGNMENT
+    bad = _args(op, km); bad.lda += 1
+    assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -2
+    bad = _args(op, km); bad.tensors[0].l_div = 0
+    assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -1
+    # a reduction module needs its workspace
+    big = _args(op, km); big.N = 4096; big.ldb = 4096
+    need = km.lib.evt_workspace_bytes(ctypes.byref(big))
+    assert need > 0
+    assert km.lib.evt_launch(ctypes.byref(big), None, 0, None) == -3    # EVT_ERR_WORKSPACE
+    with pytest.raises(RuntimeError, match="EVT_ERR_WORKSPACE"):
+        km.launch(big, 0, 0, 0)
+
+
+def test_workspace_size_formula(module):
+    op, km = module
+    tile = op.tile
+    a = _args(op, km); a.M, a.N = 1000, 5 * tile.bn; a.ldb = a.N
+    tiles_m, tiles_n = -(-a.M // tile.bm), 5
+    counters = (tiles_m * 4 + 255) // 256 * 256
+    rows = (tiles_n * a.M * 3 * 4 + 255) // 256 * 256
+    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) == counters + rows
+    a.N = tile.bn; a.ldb = a.N
+    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) == 0    # one tile along N: finalised in-kernel
+
+
+def test_fused_op_refuses_to_run_without_a_device():
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    inputs = W.make_inputs(1, W.GOLDEN_SHAPES[1])
+    gm = W.fuse(W.CONFIGS[1].module(), inputs)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        gm(*inputs)
+
+
+def test_tuner_cache_round_trip(tmp_path, monkeypatch):
+    from evt_ae_amd.autotuner.gemm_tuner import MMTuner
+    from evt_ae_amd.codegen import TileConfig
+    monkeypatch.setenv("EVT_TUNER_CACHE", str(tmp_path / "tuner_cache.db"))
+    inputs = W.make_inputs(1, W.GOLDEN_SHAPES[1])
+    gm = W.fuse(W.CONFIGS[1].module(), [t.to("meta") for t in inputs])
+    (n,) = fused_nodes(gm)
+    tuner = MMTuner((4096, 4096, 1024, 1), True, False, False, True, n.target.ir)
+    assert tuner.key() == "4096_4096_1024_f16_f16_R_R_a8_0_1_0_1_0_0_0"
+    assert tuner.fetch_cached() is None
+    h = tuner.get_best_config()
+    assert (h.bm, h.bn) == (256, 256)
+    t = TileConfig(128, 256, 64, 2, 4, 2, True, 8)
+    tuner.store(t, 12.5)
+    assert tuner.get_best_config() == t

@@ -1,0 +1,121 @@
+"""Host logic without a GPU: EVTFuser.trace / pass_fusion lower the headline
+subgraphs and the reference's fuser-test patterns (unittest/evt_fuser/mm.py,
+bmm.py) to an IR whose CPU interpretation equals PyTorch's fp32 eager
+evaluation of the original module."""
+import pytest
+import torch
+
+from evt_ae_amd import workloads as W
+from evt_ae_amd.evt_fuser import EVTFuser, FusedBMM, FusedGEMM
+from oracle import evt_oracle
+from tests.util import fused_nodes, run_emulated
+
+
+def _check(module_cls, inputs, n_fused=1, tol=2e-5):
+    gm = W.fuse(module_cls(), inputs)
+    fused = fused_nodes(gm)
+    assert len(fused) == n_fused
+    for n in fused:
+        assert n.meta.get("evt") is True
+        assert n.target.__name__ in ("cutlass_gemm_with_visitor", "cutlass_bmm_with_visitor")
+    got = run_emulated(gm, inputs)
+    ref = evt_oracle.eval_fp32(module_cls(), inputs)
+    assert len(got) == len(ref)
+    for g, r in zip(got, ref):
+        assert tuple(g.shape) == tuple(r.shape)
+        if r.dtype == torch.bool:
+            assert torch.equal(g.bool(), r)
+            continue
+        # the emulation rounds each store to the output dtype once
+        err = evt_oracle.max_rel_err(g.float(), r)
+        lim = 5e-3 if g.dtype in (torch.float16, torch.bfloat16) else tol
+        assert err <= lim, err
+    return gm
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("shapes", ["small", "ragged"])
+def test_headline_configs_lower_correctly(cfg, shapes):
+    sh = W.SMALL_SHAPES[cfg] if shapes == "small" else W.RAGGED_SHAPES[cfg]
+    inputs = W.make_inputs(cfg, sh)
+    _check(W.CONFIGS[cfg].module, inputs)
+
+
+def test_config_classification():
+    """Loads and stores are classified as the reference's pass manager names them
+    (tuner_base.py:120-152): bias -> RowBroadcast, residual -> AuxLoad,
+    labels -> ColumnBroadcast, dbias -> RowReduction ([N]), stats -> ColumnReduction ([M])."""
+    kinds = {}
+    for cfg in (1, 3, 4, 5):
+        inputs = W.make_inputs(cfg, W.SMALL_SHAPES[cfg])
+        gm = W.fuse(W.CONFIGS[cfg].module(), [t.to("meta") for t in inputs])
+        (n,) = fused_nodes(gm)
+        kinds[cfg] = {s.name: (s.role, s.kind, s.domain) for s in n.target.ir.slots}
+        assert n.target.ir.epilogue_counts() == {
+            1: (0, 1, 0, 1, 0, 0, 0), 3: (1, 1, 0, 1, 0, 2, 0), 4: (1, 0, 0, 1, 1, 0, 0), 5: (0, 0, 1, 0, 0, 1, 0)}[cfg]
+    assert kinds[1]["b"] == ("load", "row", "tile")
+    assert kinds[3]["r"] == ("load", "aux", "tile")
+    assert kinds[5]["labels"] == ("load", "col", "tile")
+    assert kinds[4]["sum_1"] == ("store", "row", "col")
+
+
+def test_operand_layouts_follow_permutes():
+    """permute [1, 0] in front of mm selects the column-major operand without a
+    copy (evt_fuser.py:548-558); 3-D permutes give BMM strides (bmm.py:36-56)."""
+    i4 = W.make_inputs(4, W.SMALL_SHAPES[4])
+    (n4,) = fused_nodes(W.fuse(W.CONFIGS[4].module(), i4))
+    assert isinstance(n4.target, FusedGEMM) and n4.target.rhs_layout == "ColumnMajor" and n4.target.b_kc
+    i2 = W.make_inputs(2, W.SMALL_SHAPES[2])
+    (n2,) = fused_nodes(W.fuse(W.CONFIGS[2].module(), i2))
+    assert isinstance(n2.target, FusedBMM) and n2.target.b_kc and n2.target.a_kc
+    i1 = W.pattern_inputs("bmm1")
+    (b1,) = fused_nodes(W.fuse(W.BMMPartition1(), [t.to("meta") for t in i1]))
+    assert (b1.target.b_kc, b1.target.ldb, b1.target.bsb) == (False, 2048, 64)
+
+
+SMALL_PATTERNS = ["mm2", "mm3", "mm4", "mm5", "mm9", "bmm1", "bmm3"]
+
+
+@pytest.mark.parametrize("name", SMALL_PATTERNS)
+def test_reference_patterns_lower_correctly(name):
+    cls, _ = W.REFERENCE_PATTERNS[name]
+    inputs = W.pattern_inputs(name)
+    _check(cls, inputs)
+
+
+def test_reference_patterns_shrunk():
+    """mm1/mm6/mm7 at reduced sizes (same graphs; the view shapes are fixed by
+    the reference so M = 1024 / 2048 stays, K is what the CPU pays for)."""
+    g = torch.Generator().manual_seed(3)
+    h = lambda *s: (torch.randn(*s, generator=g) * 0.5).half()   # noqa: E731
+    _check(W.MMPartition1, [h(4096, 64), h(1024, 64), h(4096)])
+    gm = _check(W.MMPartition6, [h(2048, 32), h(32, 1024), h(512, 4, 1024), h(512, 4, 1024)])
+    (n,) = fused_nodes(gm)
+    assert n.target.post_reshape_permute   # stored un-permuted, returned as a view
+    gm = _check(W.MMPartition7, [h(2048, 32), h(32, 1024), h(512, 4, 1024), h(512, 4, 1024)])
+    (n,) = fused_nodes(gm)
+    # add_19 and its view share one store (the reference's output2store aliasing)
+    assert len({v for v in n.target.output2store.values()}) == 3
+
+
+def test_unsupported_ops_raise():
+    class Bad(torch.nn.Module):
+        def forward(self, a, b):
+            mm = torch.ops.aten.mm(a, b)
+            return torch.ops.aten.erf(mm)
+    a, b = torch.randn(64, 32).half(), torch.randn(32, 64).half()
+    gm = W.trace_module(Bad(), [a, b])
+    names = [n.name for n in gm.graph.nodes if n.op == "call_function"]
+    assert EVTFuser.fusible(names, gm)
+    with pytest.raises(NotImplementedError):
+        EVTFuser().trace(gm, names)
+    # pass_fusion falls back to fusing the anchor alone
+    gm2 = W.fuse(Bad(), [a, b])
+    assert len(fused_nodes(gm2)) == 1
+
+
+def test_stubbed_anchors():
+    from evt_ae_amd import evt_fuser
+    for name in ("FusedSoftmax", "FusedLayerNorm", "FusedConvFprop", "FusedSpmm"):
+        with pytest.raises(NotImplementedError):
+            getattr(evt_fuser, name)(None, None)

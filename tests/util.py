@@ -1,0 +1,68 @@
+"""Shared helpers for the tests."""
+from __future__ import annotations
+
+import torch
+
+from evt_ae_amd.evt_fuser import FusedBMM, FusedGEMM, FusedOpBase
+from oracle import ir_interp
+
+aten = torch.ops.aten
+
+
+from evt_ae_amd.workloads import fused_nodes  # noqa: E402,F401
+
+
+def emulate_fused(op: FusedOpBase, *args):
+    """What `FusedOpBase.__call__` returns, computed on CPU from the op's IR
+    with the IR interpreter instead of the HIP kernel."""
+    args = [a.contiguous() if isinstance(a, torch.Tensor) else a for a in args]
+    A, B = args[-2].float(), args[-1].float()
+    if isinstance(op, FusedGEMM):
+        Al = A if op.a_kc else A.t()
+        Bl = B.t() if op.b_kc else B
+        acc = Al @ Bl
+    else:
+        acc = torch.bmm(aten.permute(A, op.permute_A), aten.permute(B, op.permute_B))
+    loads = {}
+    for k, slot in enumerate(op.ir.slots):
+        kind, ref = op.slot_sources[k]
+        if kind == "input":
+            loads[k] = args[ref]
+    stored = ir_interp.interpret(op.ir, acc, loads)
+    visitor = {}
+    for k, slot in enumerate(op.ir.slots):
+        if slot.role == "store":
+            shape, dtype = op.store_meta[slot.name]
+            numel = 1
+            for s in shape:
+                numel *= s
+            flat = stored[k]
+            assert flat.numel() == numel, (slot.name, flat.numel(), shape)
+            visitor[slot.name] = flat.view(shape)
+    results = []
+    for out in op.outputs:
+        name = op.get_output_name(out)
+        t = visitor[op.output2store[name]]
+        for kind, arg in op.post_reshape_permute.get(name, ()):
+            t = t.view(arg) if kind == "view" else t.permute(arg)
+        results.append(t)
+    return results
+
+
+def run_emulated(gm, inputs):
+    """Run a fused GraphModule on CPU with every fused node emulated."""
+    import types
+    patched = []
+    for n in fused_nodes(gm):
+        op = n.target
+        patched.append((op, op.__class__.__call__))
+    # FusedOpBase.__call__ is looked up on the class: patch per instance via a subclass
+    for op, _ in patched:
+        op.__class__ = type("Emulated" + op.__class__.__name__, (op.__class__,),
+                            {"__call__": lambda self, *a: emulate_fused(self, *a)})
+    try:
+        out = gm(*inputs)
+    finally:
+        for op, _ in patched:
+            op.__class__ = op.__class__.__mro__[1]
+    return list(out) if isinstance(out, (tuple, list)) else [out]
