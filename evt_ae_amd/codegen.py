@@ -29,10 +29,11 @@ class TileConfig:
     stages: int = 2
     dma: bool = True
     group_m: int = 4
+    pipe: int = 0       # 0: plain ring; 1: look-ahead ring with pinned instruction order (stages >= 3)
 
     def tag(self) -> str:
         return (f"{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_s{self.stages}"
-                f"_{'dma' if self.dma else 'safe'}_g{self.group_m}")
+                f"_{'dma' if self.dma else 'safe'}_g{self.group_m}" + (f"_p{self.pipe}" if self.pipe else ""))
 
     def lds_bytes(self) -> int:
         return self.stages * (self.bm + self.bn) * self.bk * 2
@@ -166,6 +167,25 @@ class Codegen:
         e.dedent()
         e("}")
 
+    def emit_identity(self, e: _Emitter, axis: str):
+        e(f"static EVT_DEV void {axis}_identity(float* a) {{")
+        e.indent()
+        for r in self.ir.reduces.values():
+            if r.axis != axis:
+                continue
+            o = r.state_offset
+            if r.kind == "sum":
+                e(f"a[{o}] = 0.f;")
+            elif r.kind == "max":
+                e(f"a[{o}] = -INFINITY;")
+            elif r.kind == "maxsumexp":
+                e(f"a[{o}] = -INFINITY; a[{o + 1}] = 0.f;")
+            elif r.kind == "welford":
+                e(f"a[{o}] = 0.f; a[{o + 1}] = 0.f; a[{o + 2}] = 0.f;")
+        e("(void)a;")
+        e.dedent()
+        e("}")
+
     def emit_finalize(self, e: _Emitter, axis: str):
         idx = "row" if axis == "row" else "col"
         stride = "sm" if axis == "row" else "sn"
@@ -236,7 +256,7 @@ class Codegen:
         e("for (int v = 0; v < 16; ++v) {")
         e.indent()
         e("const int row = t.row(mi, v);")
-        e("const bool rok = row < t.M;")
+        e("const bool rok = t.row_ok(row);")
         for name in inner:
             self.emit_node(e, ir.nodes[name], hoisted=False)
         for s in tile_stores:
@@ -249,7 +269,7 @@ class Codegen:
             else:
                 arr = _cname(src)
             e(f"evt::aux_store(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
-              f"p.t{k}_sn, p.t{k}_vec != 0, rok, {arr});")
+              f"p.t{k}_sn, p.t{k}_vec, rok, {arr});")
         if row_reds:
             e(f"float rst[{ir.row_state}];")
             for r in row_reds:
@@ -297,7 +317,7 @@ class Codegen:
             if s.kind == "aux":
                 e(f"float {c}[NI];")
                 e(f"evt::aux_load(t, p.t{k}, {base} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
-                  f"p.t{k}_sn, p.t{k}_vec != 0, rok, {c});")
+                  f"p.t{k}_sn, p.t{k}_vec, rok, {c});")
             elif s.kind == "row":
                 e(f"float {c}[NI];")
                 e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = t.col_ok(ni) ? "
@@ -389,6 +409,8 @@ class Codegen:
         self.emit_params(e)
         self.emit_combine(e, "row")
         self.emit_combine(e, "col")
+        self.emit_identity(e, "row")
+        self.emit_identity(e, "col")
         self.emit_finalize(e, "row")
         self.emit_finalize(e, "col")
         self.emit_tile(e)
@@ -396,14 +418,14 @@ class Codegen:
         e("};")
         b = lambda x: "true" if x else "false"  # noqa: E731
         e(f"using Cfg = evt::GemmCfg<{t.bm}, {t.bn}, {t.bk}, {t.wm}, {t.wn}, {b(sp.a_kc)}, {b(sp.b_kc)}, "
-          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}>;")
+          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}, {t.pipe}>;")
         e(f"constexpr int kNumTensors = {len(ir.slots)};")
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
         red_lds = 0
         if ir.row_state:
-            red_lds += t.wn * t.bm * ir.row_state * 4 + 16
+            red_lds += t.wn * t.bm * ir.row_state * 4
         if ir.col_state:
-            red_lds += t.wm * t.bn * ir.col_state * 4 + 16
+            red_lds += t.wm * t.bn * ir.col_state * 4
         e(f"static_assert(Cfg::LDS_BYTES >= {red_lds}, \"reduction exchange area exceeds the operand LDS\");")
         e("")
         e("int fill(const EvtArgs* a, evt::GemmArgs& g, Epi::Params& p) {")
@@ -441,8 +463,8 @@ class Codegen:
             e("  if (!x.ptr || x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
             e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
             e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div;")
-            e(f"  p.t{k}_vec = (x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "
-              f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0) ? 1 : 0; }}")
+            e(f"  p.t{k}_vec = (x.stride_n == 1 ? 1 : 0) | ((x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "
+              f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0) ? 2 : 0); }}")
         e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
         e("return EVT_OK;")
         e.dedent()
@@ -459,10 +481,10 @@ class Codegen:
         e("  return evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n).total();")
         e("}")
         e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
-        e("  if (bytes <= 0) return EVT_OK;")
-        e("  if (!ws || (bytes & 3)) return EVT_ERR_WORKSPACE;")
-        e("  hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ws, bytes / 4);")
-        e("  return (int)hipGetLastError();")
+        e("  // partials are fully written by every launch before they are read: nothing to clear")
+        e("  (void)stream;")
+        e("  if (bytes > 0 && !ws) return EVT_ERR_WORKSPACE;")
+        e("  return EVT_OK;")
         e("}")
         e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
         e("  evt::GemmArgs g; Epi::Params p;")
@@ -473,7 +495,9 @@ class Codegen:
         e("  g.workspace = (char*)ws;")
         e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L);")
         e("  hipLaunchKernelGGL((evt::evt_gemm_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
-        e("  return (int)hipGetLastError();")
+        e("  const int err = (int)hipGetLastError();")
+        e("  if (err != 0) return err;")
+        e("  return evt::launch_finalize<Epi>(p, g, (hipStream_t)stream);")
         e("}")
         return e.text()
 

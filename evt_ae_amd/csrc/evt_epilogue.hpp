@@ -10,11 +10,12 @@
 // rounded once (visitor.hpp:221-226, visitor_store.hpp:99-112).
 //
 // Differences by design: reductions do not use atomics into pre-zeroed
-// outputs (visitor_store.hpp:293-301, :544-553).  Each workgroup reduces its
-// tile with wave64 cross-lane operations and LDS, writes one partial per
-// (tile, row) or (tile, column) to a workspace, and the last workgroup to
-// arrive for a row block / column block combines the partials in tile order
-// and finalises the outputs, so results are deterministic.
+// outputs (visitor_store.hpp:293-301, :544-553).  Phase 1: each workgroup
+// reduces its tile with wave64 cross-lane operations and LDS and writes one
+// partial per (tile, row) or (tile, column) to a workspace.  Phase 2: a small
+// finalize kernel combines the partials in a fixed order and evaluates the
+// per-row / per-column output expressions, so results are deterministic and
+// no output needs pre-zeroing.
 #pragma once
 
 #include "evt_gemm.hpp"
@@ -24,33 +25,37 @@ namespace evt {
 // ---------------------------------------------------------------------------
 // elementwise functions (fp32)
 // ---------------------------------------------------------------------------
-EVT_DEV float op_exp(float x) { return __expf(x); }
-EVT_DEV float op_log(float x) { return __logf(x); }
-EVT_DEV float op_rcp(float x) { return __frcp_rn(x); }
-EVT_DEV float op_tanh(float x) {
-  // tanh(x) = 1 - 2 / (1 + exp(2x)); saturates correctly for |x| large
-  const float e = __expf(2.f * x);
-  return 1.f - 2.f * __frcp_rn(1.f + e);
-}
-EVT_DEV float op_sigmoid(float x) { return __frcp_rn(1.f + __expf(-x)); }
+// v_exp_f32 / v_log_f32 / v_rcp_f32 are base-2 / 1-ulp hardware functions; the
+// constants fold the base change.  Errors are ~1e-7 relative, far inside the
+// 2e-2 / 1e-3 parity contract.
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+EVT_DEV float op_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+EVT_DEV float op_log(float x) { return __builtin_amdgcn_logf(x) * kLn2; }
+EVT_DEV float op_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// sigmoid(x) = 1 / (1 + 2^(-x log2 e)); saturates to 0 / 1 for |x| large
+EVT_DEV float op_sigmoid(float x) { return op_rcp(1.f + __builtin_amdgcn_exp2f(-kLog2e * x)); }
+EVT_DEV float op_tanh(float x) { return 2.f * op_sigmoid(2.f * x) - 1.f; }
 EVT_DEV float op_relu(float x) { return x > 0.f ? x : 0.f; }
-EVT_DEV float op_gelu_tanh(float x) {
-  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-  const float u = k0 * (x + k1 * x * x * x);
-  return 0.5f * x * (1.f + op_tanh(u));
+// gelu_tanh(x) = 0.5 x (1 + tanh(u)) = x sigmoid(2u),  u = sqrt(2/pi) (x + 0.044715 x^3)
+constexpr float kGeluA = -2.f * 0.7978845608028654f * kLog2e;   // -2 sqrt(2/pi) log2(e)
+constexpr float kGeluB = kGeluA * 0.044715f;
+EVT_DEV float gelu_sig(float x, float x2) {   // sigmoid(2u)
+  return op_rcp(1.f + __builtin_amdgcn_exp2f(x * (kGeluA + kGeluB * x2)));
 }
+EVT_DEV float op_gelu_tanh(float x) { return x * gelu_sig(x, x * x); }
 EVT_DEV float op_gelu_erf(float x) { return 0.5f * x * (1.f + erff(x * 0.7071067811865476f)); }
 EVT_DEV float op_tanh_backward(float gy, float y) { return gy * (1.f - y * y); }
+// d/dx gelu_tanh = s + 2 sqrt(2/pi) x s (1 - s) (1 + 3*0.044715 x^2),  s = sigmoid(2u)
 EVT_DEV float op_gelu_backward_tanh(float gy, float x) {
-  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
   const float x2 = x * x;
-  const float t = op_tanh(k0 * (x + k1 * x * x2));
-  const float dt = (1.f - t * t) * k0 * (1.f + 3.f * k1 * x2);
-  return gy * (0.5f * (1.f + t) + 0.5f * x * dt);
+  const float s = gelu_sig(x, x2);
+  const float a = (2.f * 0.7978845608028654f) * x * (1.f + (3.f * 0.044715f) * x2);
+  return gy * (s + s * (a - a * s));
 }
 EVT_DEV float op_gelu_backward_erf(float gy, float x) {
   const float cdf = 0.5f * (1.f + erff(x * 0.7071067811865476f));
-  const float pdf = 0.3989422804014327f * __expf(-0.5f * x * x);
+  const float pdf = 0.3989422804014327f * op_exp(-0.5f * x * x);
   return gy * (cdf + x * pdf);
 }
 
@@ -75,8 +80,10 @@ EVT_DEV void st_f32<bool>(bool* p, int64_t off, float v) { p[off] = (v != 0.f); 
 // Where this lane's accumulator elements live in the output.
 // acc[mi][ni][v] is element (row(mi, v), col(ni)).
 // ---------------------------------------------------------------------------
-template <class Cfg>
+// FULL: the whole workgroup tile lies inside the matrix, so no bound checks.
+template <class Cfg, bool FULL_>
 struct TileCtx {
+  static constexpr bool FULL = FULL_;
   static constexpr int MI = Cfg::MI, NI = Cfg::NI;
   static constexpr bool INTERLEAVE = Cfg::INTERLEAVE;
   static constexpr int COL_STEP = INTERLEAVE ? 1 : 32;
@@ -101,7 +108,8 @@ struct TileCtx {
   }
   EVT_DEV int row(int mi, int v) const { return row0 + mi * 32 + 8 * (v >> 2) + (v & 3); }
   EVT_DEV int col(int ni) const { return col0 + ni * COL_STEP; }
-  EVT_DEV bool col_ok(int ni) const { return col(ni) < N; }
+  EVT_DEV bool col_ok(int ni) const { return FULL || col(ni) < N; }
+  EVT_DEV bool row_ok(int r) const { return FULL || r < M; }
   // row / column index local to the workgroup tile
   EVT_DEV int lrow(int mi, int v) const { return row(mi, v) - m0; }
   EVT_DEV int lcol(int ni) const { return col(ni) - n0; }
@@ -113,52 +121,66 @@ struct TileCtx {
 };
 
 // Load NI values of one accumulator row from an (l, m, n)-strided tensor.
-// `off` is the element offset of (batch, row, col(0)); `vec` says the tensor
-// is unit-stride along n and aligned so NI adjacent elements can move at once.
+// `off` is the element offset of (batch, row, col(0)).  `flags` bit 0: the
+// tensor has unit stride along n; bit 1: it is also aligned so the NI adjacent
+// elements of an interleaved lane can move as one 4- or 8-byte access.
 template <class T, class Tile>
-EVT_DEV void aux_load(const Tile& t, const T* p, int64_t off, int64_t sn, bool vec, bool rok,
+EVT_DEV void aux_load(const Tile& t, const T* p, int64_t off, int64_t sn, int flags, bool rok,
                       float (&out)[Tile::NI]) {
   constexpr int NI = Tile::NI;
+  const T* rp = p + off;
   if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4)) {
-    if (vec && rok && t.col0 + NI <= t.N) {
+    if ((flags & 2) && rok && (Tile::FULL || t.col0 + NI <= t.N)) {
       if constexpr (NI == 4) {
-        const u32x2 raw = *(const u32x2*)(p + off);
+        const u32x2 raw = *(const u32x2*)rp;
         const T* e = (const T*)&raw;
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni) out[ni] = (float)e[ni];
       } else {
-        const uint32_t raw = *(const uint32_t*)(p + off);
+        const uint32_t raw = *(const uint32_t*)rp;
         const T* e = (const T*)&raw;
         out[0] = (float)e[0]; out[1] = (float)e[1];
       }
       return;
     }
   }
+  if (flags & 1) {
 #pragma unroll
-  for (int ni = 0; ni < NI; ++ni)
-    out[ni] = (rok && t.col_ok(ni)) ? ld_f32<T>(p, off + (int64_t)ni * Tile::COL_STEP * sn) : 0.f;
+    for (int ni = 0; ni < NI; ++ni) out[ni] = (rok && t.col_ok(ni)) ? ld_f32<T>(rp, ni * Tile::COL_STEP) : 0.f;
+  } else {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+      out[ni] = (rok && t.col_ok(ni)) ? ld_f32<T>(rp, (int64_t)ni * Tile::COL_STEP * sn) : 0.f;
+  }
 }
 
 template <class T, class Tile>
-EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, bool vec, bool rok,
+EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, bool rok,
                        const float (&val)[Tile::NI]) {
   constexpr int NI = Tile::NI;
+  T* rp = p + off;
   if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4)) {
-    if (vec && rok && t.col0 + NI <= t.N) {
+    if ((flags & 2) && rok && (Tile::FULL || t.col0 + NI <= t.N)) {
       T e[NI];
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) e[ni] = (T)val[ni];
       if constexpr (NI == 4) {
-        *(u32x2*)(p + off) = *(const u32x2*)e;
+        *(u32x2*)rp = *(const u32x2*)e;
       } else {
-        *(uint32_t*)(p + off) = *(const uint32_t*)e;
+        *(uint32_t*)rp = *(const uint32_t*)e;
       }
       return;
     }
   }
+  if (flags & 1) {
 #pragma unroll
-  for (int ni = 0; ni < NI; ++ni)
-    if (rok && t.col_ok(ni)) st_f32<T>(p, off + (int64_t)ni * Tile::COL_STEP * sn, val[ni]);
+    for (int ni = 0; ni < NI; ++ni)
+      if (rok && t.col_ok(ni)) st_f32<T>(rp, ni * Tile::COL_STEP, val[ni]);
+  } else {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+      if (rok && t.col_ok(ni)) st_f32<T>(rp, (int64_t)ni * Tile::COL_STEP * sn, val[ni]);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -179,6 +201,9 @@ EVT_DEV float half_wave_xchg(float x) {
 }
 
 EVT_DEV float half_wave_sum(float x) {
+#ifdef EVT_ABLATE_ROWRED
+  return x;
+#endif
   x += half_wave_xchg<0>(x);
   x += half_wave_xchg<1>(x);
   x += half_wave_xchg<2>(x);
@@ -187,6 +212,9 @@ EVT_DEV float half_wave_sum(float x) {
   return x;
 }
 EVT_DEV float half_wave_max(float x) {
+#ifdef EVT_ABLATE_ROWRED
+  return x;
+#endif
   x = fmaxf(x, half_wave_xchg<0>(x));
   x = fmaxf(x, half_wave_xchg<1>(x));
   x = fmaxf(x, half_wave_xchg<2>(x));
@@ -196,11 +224,15 @@ EVT_DEV float half_wave_max(float x) {
 }
 
 // ---------------------------------------------------------------------------
-// workspace layout (bytes): [counters | row partials | column partials]
+// workspace layout (bytes): [row partials | column partials]
+//   row partials    [L][tiles_n][M][ROW_STATE] floats (only if tiles_n > 1)
+//   column partials [L][tiles_m][N][COL_STATE] floats (only if tiles_m > 1)
+// Every element a finalize kernel reads is written by the GEMM kernel of the
+// same launch, so the workspace needs no initialisation.
 // ---------------------------------------------------------------------------
 struct WsLayout {
-  int64_t counters_bytes, row_bytes, col_bytes;
-  EVT_DEV __host__ int64_t total() const { return counters_bytes + row_bytes + col_bytes; }
+  int64_t row_bytes, col_bytes;
+  __host__ __device__ int64_t total() const { return row_bytes + col_bytes; }
 };
 
 template <int ROW_STATE, int COL_STATE>
@@ -208,88 +240,50 @@ __host__ __device__ inline WsLayout ws_layout(int M, int N, int L, int tiles_m, 
   WsLayout w;
   const bool row = ROW_STATE > 0 && tiles_n > 1;
   const bool col = COL_STATE > 0 && tiles_m > 1;
-  int64_t ncnt = 0;
-  if (row) ncnt += (int64_t)L * tiles_m;
-  if (col) ncnt += (int64_t)L * tiles_n;
-  w.counters_bytes = (ncnt * 4 + 255) / 256 * 256;
   w.row_bytes = row ? ((int64_t)L * tiles_n * M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
   w.col_bytes = col ? ((int64_t)L * tiles_m * N * COL_STATE * 4 + 255) / 256 * 256 : 0;
   return w;
 }
 
-// Arrive at `counter`; returns true in every thread of the workgroup that
-// arrives last of `expected`.  Partials written before the call are visible
-// to the last arriver after it.
-EVT_DEV bool arrive_last(int* counter, int expected, int* smem_flag) {
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    *smem_flag = ticket;
-  }
-  __syncthreads();
-  const bool last = (*smem_flag == expected - 1);
-  if (last) __threadfence();
-  return last;
-}
-
-// Per-row reductions: combine the per-wave states left in LDS by the tile
-// visitor across the WN waves, then across workgroups.
+// Per-row reductions, phase 1: combine the per-wave states left in LDS by the
+// tile visitor across the WN waves.  With one tile along N the result is
+// final; otherwise it is this tile's partial for phase 2.
 //   LDS layout: state[wn][local_row][ROW_STATE] floats at smem.
 template <class Cfg, class Epi, class Tile>
 EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t) {
   constexpr int RS = Epi::ROW_STATE;
   if constexpr (RS > 0) {
-    float* lds = (float*)t.smem;
-    int* flag = (int*)(t.smem + Cfg::WN * Cfg::BM * RS * 4);
+    const float* lds = (const float*)t.smem;
     __syncthreads();
-    const int row = t.m0 + t.tid;
-    const bool mine = t.tid < Cfg::BM && row < t.M;
-    float st[RS];
-    if (mine) {
+    for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
+      const int row = t.m0 + lr;
+      if (row >= t.M) continue;
+      float st[RS];
 #pragma unroll
-      for (int c = 0; c < RS; ++c) st[c] = lds[t.tid * RS + c];
+      for (int c = 0; c < RS; ++c) st[c] = lds[lr * RS + c];
 #pragma unroll
-      for (int w = 1; w < Cfg::WN; ++w) Epi::row_combine(st, lds + (w * Cfg::BM + t.tid) * RS);
-    }
-    if (t.tiles_n == 1) {
-      if (mine) Epi::row_finalize(p, t.batch, row, st);
-      return;
-    }
-    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
-    float* part = (float*)(t.workspace + wl.counters_bytes);
-    int* counters = (int*)t.workspace;
-    const int64_t brow = (int64_t)t.batch * t.tiles_n;
-    if (mine) {
-      float* dst = part + ((brow + t.tile_n) * t.M + row) * RS;
-#pragma unroll
-      for (int c = 0; c < RS; ++c) dst[c] = st[c];
-    }
-    int* counter = counters + t.batch * t.tiles_m + t.tile_m;
-    if (arrive_last(counter, t.tiles_n, flag)) {
-      if (mine) {
-        const float* src = part + (brow * t.M + row) * RS;
-#pragma unroll
-        for (int c = 0; c < RS; ++c) st[c] = src[c];
-        for (int j = 1; j < t.tiles_n; ++j) Epi::row_combine(st, src + (int64_t)j * t.M * RS);
+      for (int w = 1; w < Cfg::WN; ++w) Epi::row_combine(st, lds + (w * Cfg::BM + lr) * RS);
+      if (t.tiles_n == 1) {
         Epi::row_finalize(p, t.batch, row, st);
+      } else {
+        float* dst = (float*)t.workspace + (((int64_t)t.batch * t.tiles_n + t.tile_n) * t.M + row) * RS;
+#pragma unroll
+        for (int c = 0; c < RS; ++c) dst[c] = st[c];
       }
-      if (t.tid == 0) *counter = 0;
     }
   }
 }
 
-// Per-column reductions.  `cs[ni][c]` holds this lane's state for column
-// col(ni) over all its rows.  LDS layout: state[wm][local_col][COL_STATE] floats
-// placed after the row-reduction area.
+// Per-column reductions, phase 1.  `cs[ni][c]` holds this lane's state for
+// column col(ni) over all its rows.  LDS layout: state[wm][local_col][COL_STATE]
+// floats placed after the row-reduction area.
 template <class Cfg, class Epi, class Tile>
 EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t,
                                float (&cs)[Tile::NI][Epi::COL_STATE > 0 ? Epi::COL_STATE : 1]) {
   constexpr int CS = Epi::COL_STATE;
   if constexpr (CS > 0) {
-    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
+    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4) : 0;
     float* lds = (float*)(t.smem + ROW_AREA);
-    int* flag = (int*)(t.smem + ROW_AREA + Cfg::WM * Cfg::BN * CS * 4);
     // the two halves of a wave hold different rows of the same columns
 #pragma unroll
     for (int ni = 0; ni < Tile::NI; ++ni) {
@@ -305,6 +299,8 @@ EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t,
         for (int c = 0; c < CS; ++c) lds[(t.wm * Cfg::BN + t.lcol(ni)) * CS + c] = cs[ni][c];
     }
     __syncthreads();
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    float* part = (float*)(t.workspace + wl.row_bytes);
     for (int lc = t.tid; lc < Cfg::BN; lc += Cfg::THREADS) {
       const int col = t.n0 + lc;
       if (col >= t.N) continue;
@@ -316,33 +312,89 @@ EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t,
       if (t.tiles_m == 1) {
         Epi::col_finalize(p, t.batch, col, st);
       } else {
-        const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
-        float* part = (float*)(t.workspace + wl.counters_bytes + wl.row_bytes);
         float* dst = part + (((int64_t)t.batch * t.tiles_m + t.tile_m) * t.N + col) * CS;
 #pragma unroll
         for (int c = 0; c < CS; ++c) dst[c] = st[c];
       }
     }
-    if (t.tiles_m == 1) return;
-    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
-    float* part = (float*)(t.workspace + wl.counters_bytes + wl.row_bytes);
-    int* counters = (int*)t.workspace;
-    const int row_counters = (Epi::ROW_STATE > 0 && t.tiles_n > 1) ? t.L * t.tiles_m : 0;
-    int* counter = counters + row_counters + t.batch * t.tiles_n + t.tile_n;
-    if (arrive_last(counter, t.tiles_m, flag)) {
-      for (int lc = t.tid; lc < Cfg::BN; lc += Cfg::THREADS) {
-        const int col = t.n0 + lc;
-        if (col >= t.N) continue;
-        const float* src = part + ((int64_t)t.batch * t.tiles_m * t.N + col) * CS;
-        float st[CS];
+  }
+}
+
+// Phase 2 of per-row reductions: 2^LG lanes share one row; each folds every
+// 2^LG-th tile partial (in tile order), then the lanes combine pairwise.  The
+// combination tree is fixed by (tiles_n, LG), so results are reproducible.
+template <class Epi, int LG>
+__global__ void __launch_bounds__(256) evt_row_finalize_kernel(typename Epi::Params p, const float* part,
+                                                               int M, int L, int tiles_n) {
+  constexpr int RS = Epi::ROW_STATE > 0 ? Epi::ROW_STATE : 1;
+  constexpr int G = 1 << LG;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t rowid = gid >> LG;
+  const int sub = (int)(gid & (G - 1));
+  const bool live = rowid < (int64_t)L * M;
+  const int batch = live ? (int)(rowid / M) : 0;
+  const int row = live ? (int)(rowid % M) : 0;
+  float st[RS];
+  Epi::row_identity(st);
+  if (live) {
+    const float* src = part + ((int64_t)batch * tiles_n * M + row) * RS;
+    for (int j = sub; j < tiles_n; j += G) Epi::row_combine(st, src + (int64_t)j * M * RS);
+  }
 #pragma unroll
-        for (int c = 0; c < CS; ++c) st[c] = src[c];
-        for (int j = 1; j < t.tiles_m; ++j) Epi::col_combine(st, src + (int64_t)j * t.N * CS);
-        Epi::col_finalize(p, t.batch, col, st);
-      }
-      if (t.tid == 0) *counter = 0;
+  for (int o = G >> 1; o > 0; o >>= 1) {
+    float other[RS];
+#pragma unroll
+    for (int c = 0; c < RS; ++c) other[c] = __shfl_xor(st[c], o);
+    Epi::row_combine(st, other);
+  }
+  if (live && sub == 0) Epi::row_finalize(p, batch, row, st);
+}
+
+// Phase 2 of per-column reductions: one thread per column folds the tile
+// partials in tile order (adjacent threads read adjacent addresses).
+template <class Epi>
+__global__ void __launch_bounds__(256) evt_col_finalize_kernel(typename Epi::Params p, const float* part,
+                                                               int N, int L, int tiles_m) {
+  constexpr int CS = Epi::COL_STATE > 0 ? Epi::COL_STATE : 1;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (int64_t)L * N) return;
+  const int batch = (int)(gid / N), col = (int)(gid % N);
+  const float* src = part + ((int64_t)batch * tiles_m * N + col) * CS;
+  float st[CS];
+#pragma unroll
+  for (int c = 0; c < CS; ++c) st[c] = src[c];
+#pragma unroll 8
+  for (int j = 1; j < tiles_m; ++j) Epi::col_combine(st, src + (int64_t)j * N * CS);
+  Epi::col_finalize(p, batch, col, st);
+}
+
+// Host side: enqueue the phase-2 kernels a launch needs (none when a single
+// tile spans the reduced axis).
+template <class Epi>
+inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hipStream_t stream) {
+  const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n);
+  if (Epi::ROW_STATE > 0 && g.tiles_n > 1) {
+    const float* part = (const float*)g.workspace;
+    int lg = 0;
+    while ((1 << lg) < g.tiles_n && lg < 6) ++lg;
+    const int64_t threads = ((int64_t)g.L * g.M) << lg;
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    switch (lg) {
+      case 1: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 1>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
+      case 2: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 2>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
+      case 3: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 3>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
+      case 4: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 4>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
+      case 5: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 5>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
+      default: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 6>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
     }
   }
+  if (Epi::COL_STATE > 0 && g.tiles_m > 1) {
+    const float* part = (const float*)(g.workspace + wl.row_bytes);
+    const int64_t threads = (int64_t)g.L * g.N;
+    hipLaunchKernelGGL((evt_col_finalize_kernel<Epi>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                       p, part, g.N, g.L, g.tiles_m);
+  }
+  return (int)hipGetLastError();
 }
 
 // Write one per-wave row state into the LDS exchange area (lane 0 of each half).
@@ -387,13 +439,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, type
   tile_coords<Cfg::GROUP_M>(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
   f32x16 acc[Cfg::MI][Cfg::NI];
   Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, smem, acc);
-  TileCtx<Cfg> t;
-  t.init(g, batch, tm, tn, smem);
-  Epi::template tile<Cfg>(p, t, acc);
-}
-
-__global__ void evt_fill_zero_kernel(uint32_t* p, int64_t n) {
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
+  if ((tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
+    TileCtx<Cfg, true> t;
+    t.init(g, batch, tm, tn, smem);
+    Epi::template tile<Cfg>(p, t, acc);
+  } else {
+    TileCtx<Cfg, false> t;
+    t.init(g, batch, tm, tn, smem);
+    Epi::template tile<Cfg>(p, t, acc);
+  }
 }
 
 }  // namespace evt

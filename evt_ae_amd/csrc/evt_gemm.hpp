@@ -57,8 +57,14 @@ struct GemmArgs {
 
 // Compile-time description of one kernel variant.
 template <int BM_, int BN_, int BK_, int WM_, int WN_, bool A_KC_, bool B_KC_,
-          bool DMA_, int STAGES_, bool BF16_, int GROUP_M_>
+          bool DMA_, int STAGES_, bool BF16_, int GROUP_M_, int PIPE_ = 0>
 struct GemmCfg {
+  // PIPE 0: ring of STAGES tiles, fragments fetched inside each k-tile.
+  // PIPE 1: look-ahead ring (STAGES >= 3): tile kt+1 is made visible one
+  //         iteration early so the first fragments of the next k-tile are
+  //         fetched under the MFMAs of the current one, and the instruction
+  //         order (MFMA / LDS read / DMA issue) is pinned.
+  static constexpr int PIPE = PIPE_;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DMA = DMA_, BF16 = BF16_;
   static constexpr int STAGES = STAGES_, GROUP_M = GROUP_M_;
@@ -79,7 +85,8 @@ struct GemmCfg {
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be 32-aligned");
-  static_assert(STAGES >= 2 && STAGES <= 4, "2..4 stages");
+  static_assert(STAGES >= 2 && STAGES <= 8, "2..8 stages");
+  static_assert(PIPE == 0 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
 };
 
 // ---------------------------------------------------------------------------
@@ -317,23 +324,161 @@ struct Mainloop {
   using RdB = FragReader<Cfg::BN, Cfg::BK, Cfg::B_LDS_KC, Cfg::NI>;
   static constexpr int LPS = OpA::NLOAD + OpB::NLOAD;   // DMA ops per thread per stage
 
+  // One k-tile: KS sub-steps of MI x NI MFMAs.  Fragments of sub-step ks+1
+  // are fetched from LDS into a second register set while the MFMAs of
+  // sub-step ks issue.
   static EVT_DEV void compute(const char* lds, const RdA& ra, const RdB& rb,
                               f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
     const char* la = lds;
     const char* lb = lds + Cfg::A_BYTES;
+    u32x4 af[2][Cfg::MI], bf[2][Cfg::NI];
+#ifndef EVT_ABLATE_LDS_READ
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) af[0][mi] = ra.read(la, mi, 0);
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) bf[0][ni] = rb.read(lb, ni, 0);
+#else
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) af[0][mi] = af[1][mi] = u32x4{(uint32_t)threadIdx.x, 1u, 2u, 3u};
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) bf[0][ni] = bf[1][ni] = u32x4{5u, (uint32_t)threadIdx.x, 7u, 8u};
+#endif
 #pragma unroll
     for (int ks = 0; ks < Cfg::KS; ++ks) {
-      u32x4 af[Cfg::MI], bf[Cfg::NI];
+      const int cur = ks & 1, nxt = cur ^ 1;
+#ifndef EVT_ABLATE_LDS_READ
+      if (ks + 1 < Cfg::KS) {
 #pragma unroll
-      for (int mi = 0; mi < Cfg::MI; ++mi) af[mi] = ra.read(la, mi, ks);
+        for (int mi = 0; mi < Cfg::MI; ++mi) af[nxt][mi] = ra.read(la, mi, ks + 1);
 #pragma unroll
-      for (int ni = 0; ni < Cfg::NI; ++ni) bf[ni] = rb.read(lb, ni, ks);
+        for (int ni = 0; ni < Cfg::NI; ++ni) bf[nxt][ni] = rb.read(lb, ni, ks + 1);
+      }
+#endif
 #pragma unroll
       for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
         for (int ni = 0; ni < Cfg::NI; ++ni)
-          acc[mi][ni] = mfma32<Cfg::BF16>(af[mi], bf[ni], acc[mi][ni]);
+          acc[mi][ni] = mfma32<Cfg::BF16>(af[cur][mi], bf[cur][ni], acc[mi][ni]);
     }
+  }
+
+  // ---- look-ahead pipeline (PIPE == 1) -------------------------------------
+  struct Frags {
+    u32x4 a[Cfg::MI];
+    u32x4 b[Cfg::NI];
+  };
+  static constexpr int NMFMA = Cfg::MI * Cfg::NI;
+  static constexpr int NDSREAD = (Cfg::A_LDS_KC ? Cfg::MI : 2 * Cfg::MI) + (Cfg::B_LDS_KC ? Cfg::NI : 2 * Cfg::NI);
+
+  static EVT_DEV void load_frags(Frags& f, const char* lds, const RdA& ra, const RdB& rb, int ks) {
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) f.a[mi] = ra.read(lds, mi, ks);
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) f.b[ni] = rb.read(lds + Cfg::A_BYTES, ni, ks);
+  }
+  static EVT_DEV void mma(const Frags& f, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < Cfg::NI; ++ni) acc[mi][ni] = mfma32<Cfg::BF16>(f.a[mi], f.b[ni], acc[mi][ni]);
+  }
+  // Scheduling directive for one sub-step of NMFMA MFMAs: NR LDS reads and NV
+  // global->LDS transfers are placed between the MFMAs.  The compiler cannot
+  // tell that a transfer and an LDS read touch different stages, so it keeps
+  // their program order; reads therefore go first (behind the leading MFMAs)
+  // and the transfers behind the trailing MFMAs.
+  template <int M, int NR, int NV>
+  static EVT_DEV void pin_order() {
+    if constexpr (M < NMFMA) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr (NV == 0) {
+        constexpr int r = (NR * (M + 1)) / NMFMA - (NR * M) / NMFMA;
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+      } else {
+        constexpr int H = NMFMA / 2;
+        if constexpr (M < H) {
+          constexpr int r = (NR * (M + 1)) / H - (NR * M) / H;
+          if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+        } else {
+          constexpr int v = (NV * (M - H + 1)) / H - (NV * (M - H)) / H;
+          if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+        }
+      }
+      pin_order<M + 1, NR, NV>();
+    }
+  }
+  template <int N>
+  static EVT_DEV void wait_tiles() {   // leave N younger tiles in flight
+    wait_vmcnt<N * LPS>();
+  }
+  static EVT_DEV void wait_tiles_dyn(int n) {
+    static_assert((Cfg::STAGES - 2) * LPS < 64, "vmcnt is a 6-bit counter");
+    if (n <= 0) wait_tiles<0>();
+    else if (n == 1) wait_tiles<1>();
+    else if (n == 2) wait_tiles<2>();
+    else if (n == 3) wait_tiles<(Cfg::STAGES > 4 ? 3 : 0)>();
+    else if (n == 4) wait_tiles<(Cfg::STAGES > 5 ? 4 : 0)>();
+    else if (n == 5) wait_tiles<(Cfg::STAGES > 6 ? 5 : 0)>();
+    else wait_tiles<(Cfg::STAGES > 7 ? 6 : 0)>();
+  }
+
+  template <bool STEADY>
+  static EVT_DEV void lookahead_iter(int kt, int KT, int& stage, const OpA& a, const OpB& b, const RdA& ra,
+                                     const RdB& rb, char* smem, int wave, Frags (&f)[2],
+                                     f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+    constexpr int S = Cfg::STAGES, D = S - 1;
+    if constexpr (STEADY) {
+      wait_tiles<D - 2>();            // tile kt+1 has landed (tiles kt+2.. may be in flight)
+    } else {
+      const int newest = min(kt + D, KT) - 1;
+      if (kt + 1 < KT) wait_tiles_dyn(newest - (kt + 1));
+    }
+    __syncthreads();                  // tile kt+1 visible to all; everyone is done with tile kt-1
+    const char* cur = smem + stage * Cfg::STAGE_BYTES;
+    int nstage = stage + 1 == S ? 0 : stage + 1;
+    const char* nxt = smem + nstage * Cfg::STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < Cfg::KS; ++ks) {
+      if (ks + 1 < Cfg::KS) {
+        load_frags(f[(ks + 1) & 1], cur, ra, rb, ks + 1);
+      } else if (STEADY || kt + 1 < KT) {
+        load_frags(f[0], nxt, ra, rb, 0);
+      }
+      if constexpr (STEADY) {
+        if (ks == Cfg::KS - 1) {   // refill the stage tile kt-1 occupied
+          int ds = stage + D;
+          if (ds >= S) ds -= S;
+          a.dma(kt + D, smem + ds * Cfg::STAGE_BYTES, wave);
+          b.dma(kt + D, smem + ds * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+        }
+      }
+      mma(f[ks & 1], acc);
+      if constexpr (STEADY) {
+        if (ks == Cfg::KS - 1) pin_order<0, NDSREAD, LPS>();
+        else pin_order<0, NDSREAD, 0>();
+      }
+    }
+    stage = nstage;
+  }
+
+  static EVT_DEV void run_lookahead(const OpA& a, const OpB& b, const RdA& ra, const RdB& rb, char* smem,
+                                    int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+    constexpr int S = Cfg::STAGES, D = S - 1;
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+      if (s < KT) {
+        a.dma(s, smem + s * Cfg::STAGE_BYTES, wave);
+        b.dma(s, smem + s * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+      }
+    }
+    wait_tiles_dyn(min(D, KT) - 1);   // tile 0 has landed
+    __syncthreads();
+    Frags f[2];
+    load_frags(f[0], smem, ra, rb, 0);
+    int stage = 0;
+    int kt = 0;
+    for (; kt + D < KT; ++kt) lookahead_iter<true>(kt, KT, stage, a, b, ra, rb, smem, wave, f, acc);
+    for (; kt < KT; ++kt) lookahead_iter<false>(kt, KT, stage, a, b, ra, rb, smem, wave, f, acc);
   }
 
   static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, char* smem,
@@ -365,7 +510,9 @@ struct Mainloop {
 
     const int KT = (g.K + Cfg::BK - 1) / Cfg::BK;
 
-    if constexpr (Cfg::DMA) {
+    if constexpr (Cfg::PIPE == 1) {
+      run_lookahead(a, b, ra, rb, smem, wave, KT, acc);
+    } else if constexpr (Cfg::DMA) {
       // prologue: STAGES-1 tiles in flight
 #pragma unroll
       for (int s = 0; s < Cfg::STAGES - 1; ++s) {
@@ -382,13 +529,17 @@ struct Mainloop {
         } else {
           wait_vmcnt<0>();
         }
+#ifndef EVT_ABLATE_BARRIER
         __syncthreads();   // tile kt visible to all waves; everyone left tile kt-1
+#endif
         const int nk = kt + Cfg::STAGES - 1;
         if (nk < KT) {
           int ns = stage + Cfg::STAGES - 1;
           if (ns >= Cfg::STAGES) ns -= Cfg::STAGES;
+#ifndef EVT_ABLATE_DMA
           a.dma(nk, smem + ns * Cfg::STAGE_BYTES, wave);
           b.dma(nk, smem + ns * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+#endif
         }
         compute(smem + stage * Cfg::STAGE_BYTES, ra, rb, acc);
         stage = (stage + 1 == Cfg::STAGES) ? 0 : stage + 1;

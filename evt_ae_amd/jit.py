@@ -24,7 +24,7 @@ from .codegen import KernelSpec, generate
 from .ir import EpilogueIR
 
 PKG_DIR = Path(__file__).resolve().parent
-CSRC_DIR = PKG_DIR / "csrc"
+CSRC_DIR = Path(os.environ.get("EVT_CSRC_DIR", PKG_DIR / "csrc"))
 INCLUDE_DIR = PKG_DIR.parent / "include"
 KERNEL_DIR = Path(os.environ.get("EVT_KERNEL_DIR", PKG_DIR / "_kernels"))
 CACHE_FILE = KERNEL_DIR / "compiled_cache.db"
@@ -38,7 +38,7 @@ HIPCC_FLAGS = [
     # packed-fp32 VALU forms are kept off on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-value", "-Wno-unknown-attributes",
-]
+] + os.environ.get("EVT_HIPCC_EXTRA", "").split()
 
 
 class EvtTensorArg(ctypes.Structure):

@@ -69,7 +69,8 @@ def test_configs_full_size(cfg):
         assert torch.all((mean - m2).abs() <= 1e-3 * scale) and evt_oracle.max_rel_err(var, v2) <= 2e-3
     if cfg == 4:
         dp, db = outs
-        assert evt_oracle.max_rel_err(db, dp.double().sum(0).float()) <= 2e-3   # checksum of the stored tensor
+        chk = dp.double().sum(0).float()                        # checksum of the stored (fp16-rounded) tensor
+        assert (db - chk).abs().max() <= 2e-3 * chk.abs().max()
     if cfg == 5:
         (loss,) = outs
         assert torch.all(loss > 0)
