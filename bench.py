@@ -172,6 +172,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--configs", default="1,2,3,4,5")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (known traffic) so HBM counters can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU (the fused GEMM+epilogue path has no cross-GPU exchange); "
@@ -225,6 +227,13 @@ def main():
         del case
         torch.cuda.empty_cache()
 
+    if args.copy_calibration:
+        src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)     # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     vcfgs = [c for c in VALUE_CONFIGS if c in details]
     flops = sum(W.CONFIGS[c].flops for c in vcfgs)
     step_ms = sum(details[c]["_ms"] for c in vcfgs)

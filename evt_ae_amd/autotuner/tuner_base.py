@@ -12,8 +12,10 @@ row or the analytic heuristic is used, so tracing never needs a device.
 """
 from __future__ import annotations
 
+import json
 import os
 import sqlite3
+from dataclasses import asdict
 from pathlib import Path
 from typing import List, Optional, Sequence, Tuple
 
@@ -59,8 +61,7 @@ class AutoTunerBase:
     # -- cache -------------------------------------------------------------------
     def _connect(self) -> sqlite3.Connection:
         con = sqlite3.connect(str(self.cache_file), timeout=30)
-        con.execute(f"CREATE TABLE IF NOT EXISTS {self.table}(key TEXT PRIMARY KEY, bm INTEGER, bn INTEGER, "
-                    "bk INTEGER, wm INTEGER, wn INTEGER, stages INTEGER, dma INTEGER, group_m INTEGER, pipe INTEGER, us REAL)")
+        con.execute(f"CREATE TABLE IF NOT EXISTS {self.table}(key TEXT PRIMARY KEY, config TEXT, us REAL)")
         return con
 
     def fetch_cached(self) -> Optional[TileConfig]:
@@ -68,21 +69,22 @@ class AutoTunerBase:
             return None
         try:
             con = self._connect()
-            row = con.execute(f"SELECT bm,bn,bk,wm,wn,stages,dma,group_m,pipe FROM {self.table} WHERE key=?",
-                              (self.key(),)).fetchone()
+            row = con.execute(f"SELECT config FROM {self.table} WHERE key=?", (self.key(),)).fetchone()
             con.close()
         except sqlite3.Error:
             return None
         if row is None:
             return None
-        return TileConfig(row[0], row[1], row[2], row[3], row[4], row[5], bool(row[6]), row[7], row[8])
+        try:
+            return TileConfig(**json.loads(row[0]))
+        except TypeError:
+            return None      # written by an incompatible version: ignore
 
     def store(self, tile: TileConfig, us: float) -> None:
         con = self._connect()
         with con:
-            con.execute(f"INSERT OR REPLACE INTO {self.table} VALUES (?,?,?,?,?,?,?,?,?,?,?)",
-                        (self.key(), tile.bm, tile.bn, tile.bk, tile.wm, tile.wn, tile.stages, int(tile.dma),
-                         tile.group_m, tile.pipe, us))
+            con.execute(f"INSERT OR REPLACE INTO {self.table} VALUES (?,?,?)",
+                        (self.key(), json.dumps(asdict(tile), sort_keys=True), us))
         con.close()
 
     # -- search space --------------------------------------------------------------
@@ -104,9 +106,13 @@ class AutoTunerBase:
                 shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0)]
         else:
             shapes = [(128, 128, 32, 2, 2, 2, 0), (64, 64, 32, 2, 2, 2, 0)]
+        if self.dma and self.K <= 64:
+            # the whole K extent fits one tile: a single LDS stage leaves room for more workgroups per CU
+            bk = 64 if self.K > 32 else 32
+            shapes += [(bm, bn, bk, wm, wn, 1, 0) for (bm, bn, _, wm, wn, st, pipe) in shapes if pipe == 0 and st == 2]
         for bm, bn, bk, wm, wn, st, pipe in shapes:
             t = TileConfig(bm, bn, bk, wm, wn, st, self.dma, 4, pipe)
-            if t.lds_bytes() <= LDS_LIMIT and t.lds_bytes() >= red_lds(t):
+            if t.lds_bytes() <= LDS_LIMIT and t.lds_bytes() >= red_lds(t) and t not in out:
                 out.append(t)
         return out
 
@@ -116,8 +122,8 @@ class AutoTunerBase:
         eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3}
         best, best_cost = None, None
         for t in self.candidates():
-            if t.pipe != 0:
-                continue    # the plain ring is the untuned default
+            if t.pipe != 0 or t.stages == 1:
+                continue    # the plain double-buffered ring is the untuned default
             tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
             wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 else 1
             rounds = -(-tiles // (NUM_CUS * wg_per_cu))

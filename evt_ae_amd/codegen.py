@@ -145,6 +145,7 @@ class Codegen:
             e(f"{const}{DTYPE_CTYPES[s.dtype]}* t{k};  // {s.role} {s.kind} '{s.name}'")
             e(f"int64_t t{k}_sl, t{k}_sm, t{k}_sn; int t{k}_ld; int t{k}_vec;")
         e(f"float s[{max(1, len(self.ir.scalars))}];")
+        e("int fast;   // every per-element tensor is unit-stride / vector-aligned: interior tiles skip all checks")
         e.dedent()
         e("};")
 
@@ -231,7 +232,7 @@ class Codegen:
         hoisted = [n for n in need if not self.var_m[n]]
         inner = [n for n in need if self.var_m[n]]
 
-        e("template <class Cfg, class Tile>")
+        e("template <class Cfg, class Tile, bool FAST>")
         e("static EVT_DEV void tile(const Params& p, const Tile& t, const evt::f32x16 (&acc)[Cfg::MI][Cfg::NI]) {")
         e.indent()
         e("constexpr int MI = Cfg::MI, NI = Cfg::NI;")
@@ -249,9 +250,26 @@ class Codegen:
                 e(f"cst[ni][{r.state_offset}] = {_IDENTITY[r.kind]};")
             e.dedent()
             e("}")
+        aux_nodes = [n for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "aux"]
         e("#pragma unroll")
         e("for (int mi = 0; mi < MI; ++mi) {")
         e.indent()
+        if aux_nodes:
+            e("// issue the full-tensor loads of these 16 rows before any arithmetic or store")
+            for name in aux_nodes:
+                k = ir.nodes[name].slot
+                e(f"{DTYPE_CTYPES[ir.slots[k].dtype]} r_{_cname(name)}[16][NI];")
+            e("#pragma unroll")
+            e("for (int v = 0; v < 16; ++v) {")
+            e.indent()
+            e("const int row = t.row(mi, v);")
+            e("const bool rok = t.row_ok(row);")
+            for name in aux_nodes:
+                k = ir.nodes[name].slot
+                e(f"evt::aux_load<FAST>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
+                  f"p.t{k}_sn, p.t{k}_vec, rok, r_{_cname(name)}[v]);")
+            e.dedent()
+            e("}")
         e("#pragma unroll")
         e("for (int v = 0; v < 16; ++v) {")
         e.indent()
@@ -268,7 +286,7 @@ class Codegen:
                 arr = f"b_{k}"
             else:
                 arr = _cname(src)
-            e(f"evt::aux_store(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
+            e(f"evt::aux_store<FAST>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
               f"p.t{k}_sn, p.t{k}_vec, rok, {arr});")
         if row_reds:
             e(f"float rst[{ir.row_state}];")
@@ -316,8 +334,7 @@ class Codegen:
             base = self.slot_off(k)
             if s.kind == "aux":
                 e(f"float {c}[NI];")
-                e(f"evt::aux_load(t, p.t{k}, {base} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
-                  f"p.t{k}_sn, p.t{k}_vec, rok, {c});")
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = (float)r_{c}[v][ni];")
             elif s.kind == "row":
                 e(f"float {c}[NI];")
                 e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = t.col_ok(ni) ? "
@@ -441,6 +458,8 @@ class Codegen:
         e("g.workspace = nullptr;")
         e("if ((int64_t)g.tiles_m * g.tiles_n * a->L > 0x7fffffffLL) return EVT_ERR_RANGE;")
         e("if (a->N > (1 << 24)) return EVT_ERR_RANGE;   // column indices are carried as fp32")
+        if t.stages == 1:
+            e("if (a->K > Cfg::BK) return EVT_ERR_RANGE;   // single-stage variant: K must fit one tile")
         if t.dma:
             e("// fast path: 16-byte global->LDS transfers, buffer range check for the tails")
             e("if (((uintptr_t)a->A | (uintptr_t)a->B) & 15) return EVT_ERR_ALIGNMENT;")
@@ -466,6 +485,12 @@ class Codegen:
             e(f"  p.t{k}_vec = (x.stride_n == 1 ? 1 : 0) | ((x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "
               f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0) ? 2 : 0); }}")
         e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
+        tile_slots = [k for k, sl in enumerate(ir.slots)
+                      if (sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux")]
+        cond = " && ".join(
+            [f"(p.t{k}_vec & 1) && (!(Cfg::INTERLEAVE && sizeof(*p.t{k}) == 2 && (Cfg::NI == 2 || Cfg::NI == 4)) || (p.t{k}_vec & 2))"
+             for k in tile_slots]) or "true"
+        e(f"p.fast = ({cond}) ? 1 : 0;")
         e("return EVT_OK;")
         e.dedent()
         e("}")

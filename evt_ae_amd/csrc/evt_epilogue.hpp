@@ -120,47 +120,57 @@ struct TileCtx {
   }
 };
 
-// Load NI values of one accumulator row from an (l, m, n)-strided tensor.
-// `off` is the element offset of (batch, row, col(0)).  `flags` bit 0: the
-// tensor has unit stride along n; bit 1: it is also aligned so the NI adjacent
-// elements of an interleaved lane can move as one 4- or 8-byte access.
-template <class T, class Tile>
+// Load NI values of one accumulator row from an (l, m, n)-strided tensor, in
+// its storage type (the generated code issues the loads of 16 rows together,
+// ahead of the arithmetic, because loads may not move above stores by
+// themselves).  `off` is the element offset of (batch, row, col(0)).
+//   FAST   the workgroup tile is interior and the tensor is unit-stride along
+//          n (and aligned for the interleaved vector access): no bound checks,
+//          no flag tests -- straight-line code the scheduler can batch.
+//   else   `flags` bit 0: unit stride along n; bit 1: aligned so the NI
+//          adjacent elements of an interleaved lane move as one access.
+template <bool FAST, class T, class Tile>
 EVT_DEV void aux_load(const Tile& t, const T* p, int64_t off, int64_t sn, int flags, bool rok,
-                      float (&out)[Tile::NI]) {
+                      T (&out)[Tile::NI]) {
   constexpr int NI = Tile::NI;
   const T* rp = p + off;
-  if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4)) {
-    if ((flags & 2) && rok && (Tile::FULL || t.col0 + NI <= t.N)) {
+  constexpr bool kVec = Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4);
+  if constexpr (kVec) {
+    if (FAST || ((flags & 2) && rok && t.col0 + NI <= t.N)) {
       if constexpr (NI == 4) {
         const u32x2 raw = *(const u32x2*)rp;
         const T* e = (const T*)&raw;
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) out[ni] = (float)e[ni];
+        for (int ni = 0; ni < 4; ++ni) out[ni] = e[ni];
       } else {
         const uint32_t raw = *(const uint32_t*)rp;
         const T* e = (const T*)&raw;
-        out[0] = (float)e[0]; out[1] = (float)e[1];
+        out[0] = e[0]; out[1] = e[1];
       }
       return;
     }
   }
-  if (flags & 1) {
+  if constexpr (FAST) {
 #pragma unroll
-    for (int ni = 0; ni < NI; ++ni) out[ni] = (rok && t.col_ok(ni)) ? ld_f32<T>(rp, ni * Tile::COL_STEP) : 0.f;
+    for (int ni = 0; ni < NI; ++ni) out[ni] = rp[ni * Tile::COL_STEP];
+  } else if (flags & 1) {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) out[ni] = (rok && t.col_ok(ni)) ? rp[ni * Tile::COL_STEP] : T(0);
   } else {
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
-      out[ni] = (rok && t.col_ok(ni)) ? ld_f32<T>(rp, (int64_t)ni * Tile::COL_STEP * sn) : 0.f;
+      out[ni] = (rok && t.col_ok(ni)) ? rp[(int64_t)ni * Tile::COL_STEP * sn] : T(0);
   }
 }
 
-template <class T, class Tile>
+template <bool FAST, class T, class Tile>
 EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, bool rok,
                        const float (&val)[Tile::NI]) {
   constexpr int NI = Tile::NI;
   T* rp = p + off;
-  if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4)) {
-    if ((flags & 2) && rok && (Tile::FULL || t.col0 + NI <= t.N)) {
+  constexpr bool kVec = Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4);
+  if constexpr (kVec) {
+    if (FAST || ((flags & 2) && rok && t.col0 + NI <= t.N)) {
       T e[NI];
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) e[ni] = (T)val[ni];
@@ -172,7 +182,10 @@ EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, 
       return;
     }
   }
-  if (flags & 1) {
+  if constexpr (FAST) {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) st_f32<T>(rp, ni * Tile::COL_STEP, val[ni]);
+  } else if (flags & 1) {
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
       if (rok && t.col_ok(ni)) st_f32<T>(rp, ni * Tile::COL_STEP, val[ni]);
@@ -350,22 +363,34 @@ __global__ void __launch_bounds__(256) evt_row_finalize_kernel(typename Epi::Par
   if (live && sub == 0) Epi::row_finalize(p, batch, row, st);
 }
 
-// Phase 2 of per-column reductions: one thread per column folds the tile
-// partials in tile order (adjacent threads read adjacent addresses).
+// Phase 2 of per-column reductions: a block of 256 threads covers 256 / G
+// columns; G threads per column each fold every G-th tile partial (in tile
+// order), LDS combines the G results in order.  Threads of equal share index
+// read adjacent columns, i.e. adjacent addresses.
 template <class Epi>
 __global__ void __launch_bounds__(256) evt_col_finalize_kernel(typename Epi::Params p, const float* part,
-                                                               int N, int L, int tiles_m) {
+                                                               int N, int L, int tiles_m, int G) {
   constexpr int CS = Epi::COL_STATE > 0 ? Epi::COL_STATE : 1;
-  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (gid >= (int64_t)L * N) return;
-  const int batch = (int)(gid / N), col = (int)(gid % N);
-  const float* src = part + ((int64_t)batch * tiles_m * N + col) * CS;
+  __shared__ float lds[256 * CS];
+  const int per = 256 / G;
+  const int sub = threadIdx.x / per, c = threadIdx.x % per;
+  const int64_t colid = (int64_t)blockIdx.x * per + c;
+  const bool live = colid < (int64_t)L * N;
+  const int batch = live ? (int)(colid / N) : 0, col = live ? (int)(colid % N) : 0;
   float st[CS];
+  Epi::col_identity(st);
+  if (live) {
+    const float* src = part + ((int64_t)batch * tiles_m * N + col) * CS;
+#pragma unroll 4
+    for (int j = sub; j < tiles_m; j += G) Epi::col_combine(st, src + (int64_t)j * N * CS);
+  }
 #pragma unroll
-  for (int c = 0; c < CS; ++c) st[c] = src[c];
-#pragma unroll 8
-  for (int j = 1; j < tiles_m; ++j) Epi::col_combine(st, src + (int64_t)j * N * CS);
-  Epi::col_finalize(p, batch, col, st);
+  for (int k = 0; k < CS; ++k) lds[threadIdx.x * CS + k] = st[k];
+  __syncthreads();
+  if (live && sub == 0) {
+    for (int s2 = 1; s2 < G; ++s2) Epi::col_combine(st, lds + (s2 * per + c) * CS);
+    Epi::col_finalize(p, batch, col, st);
+  }
 }
 
 // Host side: enqueue the phase-2 kernels a launch needs (none when a single
@@ -390,9 +415,12 @@ inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hip
   }
   if (Epi::COL_STATE > 0 && g.tiles_m > 1) {
     const float* part = (const float*)(g.workspace + wl.row_bytes);
-    const int64_t threads = (int64_t)g.L * g.N;
-    hipLaunchKernelGGL((evt_col_finalize_kernel<Epi>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
-                       p, part, g.N, g.L, g.tiles_m);
+    int G = 1;
+    while (G < 16 && G * 4 <= g.tiles_m) G *= 2;      // >= 4 partials per thread
+    const int per = 256 / G;
+    const int64_t cols = (int64_t)g.L * g.N;
+    hipLaunchKernelGGL((evt_col_finalize_kernel<Epi>), dim3((unsigned)((cols + per - 1) / per)), dim3(256), 0, stream,
+                       p, part, g.N, g.L, g.tiles_m, G);
   }
   return (int)hipGetLastError();
 }
@@ -431,7 +459,9 @@ EVT_DEV void combine_welford(float& n, float& mean, float& m2, float nb, float m
   n = nt;
 }
 
-// The fused kernel.
+// The fused kernel.  Interior tiles whose epilogue tensors are all unit-stride
+// (p.fast, decided on the host) take the check-free epilogue; everything else
+// takes the guarded one.
 template <class Cfg, class Epi>
 __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
   __shared__ __attribute__((aligned(1024))) char smem[Cfg::LDS_BYTES];
@@ -439,14 +469,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, type
   tile_coords<Cfg::GROUP_M>(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
   f32x16 acc[Cfg::MI][Cfg::NI];
   Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, smem, acc);
-  if ((tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
+  if (p.fast && (tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
     TileCtx<Cfg, true> t;
     t.init(g, batch, tm, tn, smem);
-    Epi::template tile<Cfg>(p, t, acc);
+    Epi::template tile<Cfg, TileCtx<Cfg, true>, true>(p, t, acc);
   } else {
     TileCtx<Cfg, false> t;
     t.init(g, batch, tm, tn, smem);
-    Epi::template tile<Cfg>(p, t, acc);
+    Epi::template tile<Cfg, TileCtx<Cfg, false>, false>(p, t, acc);
   }
 }
 

@@ -85,7 +85,7 @@ struct GemmCfg {
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be 32-aligned");
-  static_assert(STAGES >= 2 && STAGES <= 8, "2..8 stages");
+  static_assert(STAGES >= 1 && STAGES <= 8, "1..8 stages");
   static_assert(PIPE == 0 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
 };
 
@@ -512,6 +512,13 @@ struct Mainloop {
 
     if constexpr (Cfg::PIPE == 1) {
       run_lookahead(a, b, ra, rb, smem, wave, KT, acc);
+    } else if constexpr (Cfg::DMA && Cfg::STAGES == 1) {
+      // K fits one tile (checked by the host): load it, use it
+      a.dma(0, smem, wave);
+      b.dma(0, smem + Cfg::A_BYTES, wave);
+      wait_vmcnt<0>();
+      __syncthreads();
+      compute(smem, ra, rb, acc);
     } else if constexpr (Cfg::DMA) {
       // prologue: STAGES-1 tiles in flight
 #pragma unroll
