@@ -98,7 +98,19 @@ class Case:
         return order
 
 
+def spin_up(torch, fn, seconds=0.15):
+    """Untimed: keep the GPU busy long enough for its clocks to settle."""
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+
+
 def time_loop(torch, fn, steps, warmup):
+    spin_up(torch, fn)
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()

@@ -89,8 +89,9 @@ class AutoTunerBase:
 
     # -- search space --------------------------------------------------------------
     def candidates(self) -> List[TileConfig]:
-        red_lds = lambda t: ((t.wn * t.bm * self.ir.row_state * 4 if self.ir.row_state else 0) +   # noqa: E731
-                             (t.wm * t.bn * self.ir.col_state * 4 if self.ir.col_state else 0))
+        red_lds = lambda t: ((t.wn * t.bm * self.ir.row_state * 4 + 16 if self.ir.row_state else 0) +   # noqa: E731
+                             (max(t.wm, max(1, t.wm * t.wn * 64 // t.bn)) * t.bn * self.ir.col_state * 4 + 16
+                              if self.ir.col_state else 0))
         out = []
         if self.dma:
             # (bm, bn, bk, wave grid, LDS stages, pipeline): plain ring (0) or look-ahead ring (1)
@@ -182,6 +183,7 @@ class AutoTunerBase:
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = module.workspace_bytes(sets[0][0])
         ws = torch.empty(max(nbytes, 4), dtype=torch.uint8, device="cuda")
+        module.workspace_init(ws.data_ptr(), nbytes, stream)
         for i in range(self.warmup_iterations):
             module.launch(sets[i % len(sets)][0], ws.data_ptr(), nbytes, stream)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -233,7 +233,8 @@ class Codegen:
         inner = [n for n in need if self.var_m[n]]
 
         e("template <class Cfg, class Tile, bool FAST>")
-        e("static EVT_DEV void tile(const Params& p, const Tile& t, const evt::f32x16 (&acc)[Cfg::MI][Cfg::NI]) {")
+        e("static EVT_DEV void tile(const Params& p, const Tile& t, const evt::GemmArgs& g, "
+          "const evt::f32x16 (&acc)[Cfg::MI][Cfg::NI]) {")
         e.indent()
         e("constexpr int MI = Cfg::MI, NI = Cfg::NI;")
         if row_reds or col_reds:
@@ -310,10 +311,10 @@ class Codegen:
         e.dedent()
         e("}")
         if row_reds:
-            e("evt::row_reduce_finish<Cfg, Epi>(p, t);")
+            e("evt::row_reduce_finish<Cfg, Epi>(p, t, g);")
         if col_reds:
-            e("evt::col_reduce_finish<Cfg, Epi>(p, t, cst);")
-        e("(void)p; (void)t; (void)acc;")
+            e("evt::col_reduce_finish<Cfg, Epi>(p, t, g, cst);")
+        e("(void)p; (void)t; (void)g; (void)acc;")
         e.dedent()
         e("}")
 
@@ -417,6 +418,7 @@ class Codegen:
         e(f"// module {self.name}")
         e('#include "evt_epilogue.hpp"')
         e('#include "evt_amd.h"')
+        e("#include <stdlib.h>")
         e("")
         e("namespace {")
         e("struct Epi {")
@@ -440,11 +442,16 @@ class Codegen:
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
         red_lds = 0
         if ir.row_state:
-            red_lds += t.wn * t.bm * ir.row_state * 4
+            red_lds += t.wn * t.bm * ir.row_state * 4 + 16
         if ir.col_state:
-            red_lds += t.wm * t.bn * ir.col_state * 4
+            red_lds += max(t.wm, max(1, t.wm * t.wn * 64 // t.bn)) * t.bn * ir.col_state * 4 + 16
         e(f"static_assert(Cfg::LDS_BYTES >= {red_lds}, \"reduction exchange area exceeds the operand LDS\");")
         e("")
+        e("// EVT_TWO_KERNEL_REDUCE=1 forces the separate finalize kernel for every cross-tile reduction")
+        e("bool evt_two_kernel_reduce() {")
+        e("  static const bool v = [] { const char* s = getenv(\"EVT_TWO_KERNEL_REDUCE\"); return s && s[0] == '1'; }();")
+        e("  return v;")
+        e("}")
         e("int fill(const EvtArgs* a, evt::GemmArgs& g, Epi::Params& p) {")
         e.indent()
         e("if (!a || !a->A || !a->B) return EVT_ERR_BAD_ARGS;")
@@ -456,6 +463,9 @@ class Codegen:
         e("g.tiles_m = (a->M + Cfg::BM - 1) / Cfg::BM;")
         e("g.tiles_n = (a->N + Cfg::BN - 1) / Cfg::BN;")
         e("g.workspace = nullptr;")
+        e("// few partials: the last workgroup to arrive combines them; many: a finalize kernel does")
+        e("g.row_inkernel = (g.tiles_n <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
+        e("g.col_inkernel = (g.tiles_m <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
         e("if ((int64_t)g.tiles_m * g.tiles_n * a->L > 0x7fffffffLL) return EVT_ERR_RANGE;")
         e("if (a->N > (1 << 24)) return EVT_ERR_RANGE;   // column indices are carried as fp32")
         if t.stages == 1:
@@ -506,10 +516,11 @@ class Codegen:
         e("  return evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n).total();")
         e("}")
         e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
-        e("  // partials are fully written by every launch before they are read: nothing to clear")
-        e("  (void)stream;")
-        e("  if (bytes > 0 && !ws) return EVT_ERR_WORKSPACE;")
-        e("  return EVT_OK;")
+        e("  if (bytes <= 0) return EVT_OK;")
+        e("  if (!ws || (bytes & 3)) return EVT_ERR_WORKSPACE;")
+        e("  // arrival counters start at zero (a fill kernel, so the call can be captured in a graph)")
+        e("  hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ws, bytes / 4);")
+        e("  return (int)hipGetLastError();")
         e("}")
         e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
         e("  evt::GemmArgs g; Epi::Params p;")

@@ -237,15 +237,19 @@ EVT_DEV float half_wave_max(float x) {
 }
 
 // ---------------------------------------------------------------------------
-// workspace layout (bytes): [row partials | column partials]
+// workspace layout (bytes): [arrival counters | row partials | column partials]
+//   counters        one int per (batch, row block) and per (batch, column block)
 //   row partials    [L][tiles_n][M][ROW_STATE] floats (only if tiles_n > 1)
 //   column partials [L][tiles_m][N][COL_STATE] floats (only if tiles_m > 1)
-// Every element a finalize kernel reads is written by the GEMM kernel of the
-// same launch, so the workspace needs no initialisation.
+// The counters must be zero before the first launch (evt_workspace_init); a
+// launch leaves them zero.  Partials are written before they are read by
+// every launch.
 // ---------------------------------------------------------------------------
+constexpr int kMaxInKernelPartials = 64;
+
 struct WsLayout {
-  int64_t row_bytes, col_bytes;
-  __host__ __device__ int64_t total() const { return row_bytes + col_bytes; }
+  int64_t counter_bytes, row_bytes, col_bytes;
+  __host__ __device__ int64_t total() const { return counter_bytes + row_bytes + col_bytes; }
 };
 
 template <int ROW_STATE, int COL_STATE>
@@ -253,20 +257,52 @@ __host__ __device__ inline WsLayout ws_layout(int M, int N, int L, int tiles_m, 
   WsLayout w;
   const bool row = ROW_STATE > 0 && tiles_n > 1;
   const bool col = COL_STATE > 0 && tiles_m > 1;
+  const int64_t ncnt = (row ? (int64_t)L * tiles_m : 0) + (col ? (int64_t)L * tiles_n : 0);
+  w.counter_bytes = (ncnt * 4 + 255) / 256 * 256;
   w.row_bytes = row ? ((int64_t)L * tiles_n * M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
   w.col_bytes = col ? ((int64_t)L * tiles_m * N * COL_STATE * 4 + 255) / 256 * 256 : 0;
   return w;
 }
 
-// Per-row reductions, phase 1: combine the per-wave states left in LDS by the
-// tile visitor across the WN waves.  With one tile along N the result is
-// final; otherwise it is this tile's partial for phase 2.
-//   LDS layout: state[wn][local_row][ROW_STATE] floats at smem.
+// Device-scope accesses for data exchanged between workgroups inside one
+// kernel.  The eight XCDs have separate L2 caches; a relaxed agent-scope atomic
+// store is written through and a relaxed agent-scope atomic load is served
+// from the coherence point, so neither needs the L2 write-back / invalidate a
+// release / acquire fence would cost.
+EVT_DEV void st_device(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+EVT_DEV float ld_device(const float* p) {
+  return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Count this workgroup in at `counter`; true (in every thread) for the
+// workgroup that arrives last of `expected`.  Every thread's partials were
+// stored with st_device before the call; the wait below lets them complete
+// before the ticket is taken, so the last arriver reads all of them.
+EVT_DEV bool arrive_last(int* counter, int expected, int* smem_flag) {
+  __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0): my device-scope stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *smem_flag = ticket;
+  }
+  __syncthreads();
+  return *smem_flag == expected - 1;
+}
+
+// Per-row reductions: combine the per-wave states left in LDS by the tile
+// visitor across the WN waves.  With one tile along N the result is final;
+// otherwise it is this tile's partial and phase 2 combines the partials in
+// tile order -- in the last workgroup of the row block to arrive (few tiles) or
+// in the finalize kernel (many tiles).
+//   LDS layout: state[wn][local_row][ROW_STATE] floats at smem, then one flag.
 template <class Cfg, class Epi, class Tile>
-EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t) {
+EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
   constexpr int RS = Epi::ROW_STATE;
   if constexpr (RS > 0) {
     const float* lds = (const float*)t.smem;
+    int* flag = (int*)(t.smem + Cfg::WN * Cfg::BM * RS * 4);
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    float* part = (float*)(t.workspace + wl.counter_bytes);
     __syncthreads();
     for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
       const int row = t.m0 + lr;
@@ -279,24 +315,45 @@ EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t) {
       if (t.tiles_n == 1) {
         Epi::row_finalize(p, t.batch, row, st);
       } else {
-        float* dst = (float*)t.workspace + (((int64_t)t.batch * t.tiles_n + t.tile_n) * t.M + row) * RS;
+        float* dst = part + (((int64_t)t.batch * t.tiles_n + t.tile_n) * t.M + row) * RS;
 #pragma unroll
-        for (int c = 0; c < RS; ++c) dst[c] = st[c];
+        for (int c = 0; c < RS; ++c) st_device(dst + c, st[c]);
       }
     }
+    if (t.tiles_n == 1 || !g.row_inkernel) return;
+    int* counter = (int*)t.workspace + t.batch * t.tiles_m + t.tile_m;
+    if (!arrive_last(counter, t.tiles_n, flag)) return;
+    for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
+      const int row = t.m0 + lr;
+      if (row >= t.M) continue;
+      const float* src = part + ((int64_t)t.batch * t.tiles_n * t.M + row) * RS;
+      float st[RS];
+#pragma unroll
+      for (int c = 0; c < RS; ++c) st[c] = ld_device(src + c);
+      for (int j = 1; j < t.tiles_n; ++j) {
+        float o[RS];
+#pragma unroll
+        for (int c = 0; c < RS; ++c) o[c] = ld_device(src + (int64_t)j * t.M * RS + c);
+        Epi::row_combine(st, o);
+      }
+      Epi::row_finalize(p, t.batch, row, st);
+    }
+    if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
-// Per-column reductions, phase 1.  `cs[ni][c]` holds this lane's state for
-// column col(ni) over all its rows.  LDS layout: state[wm][local_col][COL_STATE]
-// floats placed after the row-reduction area.
+// Per-column reductions.  `cs[ni][c]` holds this lane's state for column
+// col(ni) over all its rows.  LDS layout: state[wm][local_col][COL_STATE]
+// floats placed after the row-reduction area, then one flag.
 template <class Cfg, class Epi, class Tile>
-EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t,
+EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g,
                                float (&cs)[Tile::NI][Epi::COL_STATE > 0 ? Epi::COL_STATE : 1]) {
   constexpr int CS = Epi::COL_STATE;
   if constexpr (CS > 0) {
-    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4) : 0;
+    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
+    constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
     float* lds = (float*)(t.smem + ROW_AREA);
+    int* flag = (int*)(t.smem + ROW_AREA + (Cfg::WM > SHARES ? Cfg::WM : SHARES) * Cfg::BN * CS * 4);
     // the two halves of a wave hold different rows of the same columns
 #pragma unroll
     for (int ni = 0; ni < Tile::NI; ++ni) {
@@ -313,7 +370,7 @@ EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t,
     }
     __syncthreads();
     const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
-    float* part = (float*)(t.workspace + wl.row_bytes);
+    float* part = (float*)(t.workspace + wl.counter_bytes + wl.row_bytes);
     for (int lc = t.tid; lc < Cfg::BN; lc += Cfg::THREADS) {
       const int col = t.n0 + lc;
       if (col >= t.N) continue;
@@ -327,9 +384,41 @@ EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t,
       } else {
         float* dst = part + (((int64_t)t.batch * t.tiles_m + t.tile_m) * t.N + col) * CS;
 #pragma unroll
-        for (int c = 0; c < CS; ++c) dst[c] = st[c];
+        for (int c = 0; c < CS; ++c) st_device(dst + c, st[c]);
       }
     }
+    if (t.tiles_m == 1 || !g.col_inkernel) return;
+    const int row_counters = (Epi::ROW_STATE > 0 && t.tiles_n > 1) ? t.L * t.tiles_m : 0;
+    int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
+    if (!arrive_last(counter, t.tiles_m, flag)) return;
+    // SHARES threads per column each fold every SHARES-th partial in tile order
+    // (independent loads in flight together), LDS then combines the shares in order
+    const int lc = t.tid % Cfg::BN, share = t.tid / Cfg::BN;
+    const int col = t.n0 + lc;
+    const bool live = share < SHARES && col < t.N;
+    float st[CS];
+    Epi::col_identity(st);
+    if (live) {
+      const float* src = part + ((int64_t)t.batch * t.tiles_m * t.N + col) * CS;
+#pragma unroll 8
+      for (int j = share; j < t.tiles_m; j += SHARES) {
+        float o[CS];
+#pragma unroll
+        for (int c = 0; c < CS; ++c) o[c] = ld_device(src + (int64_t)j * t.N * CS + c);
+        Epi::col_combine(st, o);
+      }
+    }
+    __syncthreads();   // phase-1 LDS values are no longer needed
+    if (share < SHARES) {
+#pragma unroll
+      for (int c = 0; c < CS; ++c) lds[(share * Cfg::BN + lc) * CS + c] = st[c];
+    }
+    __syncthreads();
+    if (live && share == 0) {
+      for (int s2 = 1; s2 < SHARES; ++s2) Epi::col_combine(st, lds + (s2 * Cfg::BN + lc) * CS);
+      Epi::col_finalize(p, t.batch, col, st);
+    }
+    if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -398,8 +487,8 @@ __global__ void __launch_bounds__(256) evt_col_finalize_kernel(typename Epi::Par
 template <class Epi>
 inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hipStream_t stream) {
   const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n);
-  if (Epi::ROW_STATE > 0 && g.tiles_n > 1) {
-    const float* part = (const float*)g.workspace;
+  if (Epi::ROW_STATE > 0 && g.tiles_n > 1 && !g.row_inkernel) {
+    const float* part = (const float*)(g.workspace + wl.counter_bytes);
     int lg = 0;
     while ((1 << lg) < g.tiles_n && lg < 6) ++lg;
     const int64_t threads = ((int64_t)g.L * g.M) << lg;
@@ -413,8 +502,8 @@ inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hip
       default: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 6>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
     }
   }
-  if (Epi::COL_STATE > 0 && g.tiles_m > 1) {
-    const float* part = (const float*)(g.workspace + wl.row_bytes);
+  if (Epi::COL_STATE > 0 && g.tiles_m > 1 && !g.col_inkernel) {
+    const float* part = (const float*)(g.workspace + wl.counter_bytes + wl.row_bytes);
     int G = 1;
     while (G < 16 && G * 4 <= g.tiles_m) G *= 2;      // >= 4 partials per thread
     const int per = 256 / G;
@@ -472,12 +561,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, type
   if (p.fast && (tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
     TileCtx<Cfg, true> t;
     t.init(g, batch, tm, tn, smem);
-    Epi::template tile<Cfg, TileCtx<Cfg, true>, true>(p, t, acc);
+    Epi::template tile<Cfg, TileCtx<Cfg, true>, true>(p, t, g, acc);
   } else {
     TileCtx<Cfg, false> t;
     t.init(g, batch, tm, tn, smem);
-    Epi::template tile<Cfg, TileCtx<Cfg, false>, false>(p, t, acc);
+    Epi::template tile<Cfg, TileCtx<Cfg, false>, false>(p, t, g, acc);
   }
+}
+
+__global__ void evt_fill_zero_kernel(uint32_t* p, int64_t n) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
 }
 
 }  // namespace evt

@@ -53,6 +53,9 @@ struct GemmArgs {
   int64_t ldb, bsB;   // elements
   int tiles_m, tiles_n;
   char* workspace;
+  // phase 2 of a cross-tile reduction runs inside this kernel (last workgroup
+  // to arrive) instead of in a separate finalize kernel
+  int row_inkernel, col_inkernel;
 };
 
 // Compile-time description of one kernel variant.

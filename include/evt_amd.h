@@ -86,19 +86,19 @@ const char* evt_module_spec(void);
 
 /* Bytes of device workspace `evt_launch` needs for these arguments (0 when the
  * epilogue has no reduction that spans several workgroup tiles).  It holds the
- * per-tile partial results of the two-phase reduction; every launch writes what
- * it later reads, so the contents need no preparation and two launches may
- * share a workspace only if they do not overlap in time.  Takes the place of
- * the host-side pre-zeroing of reduction outputs (evt_fuser.py:217-225). */
+ * per-tile partial results of the two-phase reduction and one arrival counter
+ * per row / column block.  The counters must be zero before the first launch
+ * (evt_workspace_init) and every launch leaves them zero; launches that share
+ * a workspace must not overlap in time.  Takes the place of the host-side
+ * pre-zeroing of reduction outputs (evt_fuser.py:217-225). */
 int64_t evt_workspace_bytes(const EvtArgs* args);
 
-/* Validates a workspace pointer for `bytes`; the workspace needs no clearing,
- * so nothing is enqueued.  Kept so that callers have one place to prepare a
- * fresh workspace. */
+/* Zero-fill a fresh workspace on `stream` with a fill kernel (no memset node,
+ * so the call may be captured in a HIP graph). */
 int evt_workspace_init(void* workspace, int64_t bytes, void* stream);
 
-/* Enqueue the fused kernel (and, for reductions that span several tiles, its
- * small finalize kernel) on `stream` (a hipStream_t).  Asynchronous; returns
+/* Enqueue the fused kernel (and, for reductions that span more than 64 tiles,
+ * its small finalize kernel) on `stream` (a hipStream_t).  Asynchronous; returns
  * EVT_OK, a negative EVT_ERR_* code, or a positive hipError_t.  Replaces
  * `operation.run(arguments, stream=stream.cuda_stream)` (evt_fuser.py:546). */
 int evt_launch(const EvtArgs* args, void* workspace, int64_t workspace_bytes,

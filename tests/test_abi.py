@@ -103,9 +103,10 @@ def test_workspace_size_formula(module):
     op, km = module
     tile = op.tile
     a = _args(op, km); a.M, a.N = 1000, 5 * tile.bn; a.ldb = a.N
-    tiles_n = 5
+    tiles_m, tiles_n = -(-a.M // tile.bm), 5
+    counters = (tiles_m * 4 + 255) // 256 * 256          # one arrival counter per row block
     rows = (tiles_n * a.M * 3 * 4 + 255) // 256 * 256   # one (count, mean, M2) partial per tile and row
-    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) == rows
+    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) == counters + rows
     a.N = tile.bn; a.ldb = a.N
     assert km.lib.evt_workspace_bytes(ctypes.byref(a)) == 0    # one tile along N: finalised in-kernel
 
