@@ -15,7 +15,7 @@ from __future__ import annotations
 import json
 import os
 import sqlite3
-from dataclasses import asdict
+from dataclasses import asdict, fields
 from pathlib import Path
 from typing import List, Optional, Sequence, Tuple
 
@@ -75,10 +75,11 @@ class AutoTunerBase:
             return None
         if row is None:
             return None
-        try:
-            return TileConfig(**json.loads(row[0]))
-        except TypeError:
-            return None      # written by an incompatible version: ignore
+        cfg = json.loads(row[0])
+        known = {f.name for f in fields(TileConfig)}
+        if any(k not in known and v for k, v in cfg.items()):
+            return None      # uses an option this version does not have: ignore the row
+        return TileConfig(**{k: v for k, v in cfg.items() if k in known})
 
     def store(self, tile: TileConfig, us: float) -> None:
         con = self._connect()
