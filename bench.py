@@ -176,6 +176,19 @@ def cpu_baseline(torch, W, evt_oracle, cfgs, reps=3):
     return flops / secs / 1e12, torch.get_num_threads(), secs
 
 
+# L2<->fabric bytes per launch of the fused kernel, from two rocprofv3 --pmc runs of this script (FETCH_SIZE,
+# then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB streaming kernel
+# of --copy-calibration (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Keyed by (config, tile): a launch with another
+# tile has no measurement and reports null.  The summary of those runs is profiles/evt_gemm_kernel_bench_configs_1-5.md.
+MEASURED_TRAFFIC_BYTES = {
+    (1, "256x256x32_w2x4_s4_dma_g4_p1"): int((2.0 * 24711.5 + 32768) * 1024),
+    (2, "128x512x64_w2x4_s1_dma_g4"): int((2.0 * 4243.0 + 33024) * 1024),
+    (3, "128x256x32_w2x4_s4_dma_g4_p1"): int((2.0 * 74099.0 + 17610) * 1024),
+    (4, "128x128x64_w2x2_s2_dma_g4"): int((2.0 * 74029.3 + 16660) * 1024),
+    (5, "256x256x32_w4x2_s4_dma_g4_p1"): int((2.0 * 69818.0 + 18432) * 1024),
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -185,7 +198,7 @@ def main():
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--configs", default="1,2,3,4,5")
     ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run a plain 256 MiB device copy (known traffic) so HBM counters can be scaled")
+                    help="also run a plain 256 MiB streaming kernel (torch.neg, known traffic) so HBM counters can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU (the fused GEMM+epilogue path has no cross-GPU exchange); "
@@ -243,7 +256,7 @@ def main():
         src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)
         for _ in range(3):
-            dst.copy_(src)     # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+            torch.neg(src, out=dst)   # a plain streaming kernel of known traffic: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
     vcfgs = [c for c in VALUE_CONFIGS if c in details]
@@ -271,7 +284,8 @@ def main():
                                "out_proj_residual_ln_stats 8192x1024x4096, ffn_backward_dbias 8192x1024x4096)",
                    "frac_mfma_peak": round(flops / (step_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4)},
         "roofline": {"bound": "mfma", "achieved": round(dom_tflops, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(dom_tflops / PEAK_FP16_TFLOPS, 4), "traffic": None,
+                     "frac": round(dom_tflops / PEAK_FP16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((dom, details[dom]["tile"])),
                      "kernel": f"config {dom} ({details[dom]['workload']}, tile {details[dom]['tile']})",
                      "us": details[dom]["us"]},
         "cpu_baseline": cpu,

@@ -135,3 +135,26 @@ def test_tuner_cache_round_trip(tmp_path, monkeypatch):
     t = TileConfig(128, 256, 64, 2, 4, 2, True, 8)
     tuner.store(t, 12.5)
     assert tuner.get_best_config() == t
+
+
+def test_shipped_tuner_cache_is_read():
+    """Every row of the shipped tile cache parses into a TileConfig of this
+    version and is what tracing the headline workloads selects."""
+    import json
+    import sqlite3
+    from evt_ae_amd import prebuild
+    from evt_ae_amd.autotuner.tuner_base import default_cache_file
+    from evt_ae_amd.codegen import TileConfig
+    con = sqlite3.connect(str(default_cache_file()))
+    rows = {}
+    for table in ("best_config_mm", "best_config_bmm"):
+        for key, cfg, us in con.execute(f"SELECT key, config, us FROM {table}"):
+            rows[key] = TileConfig(**json.loads(cfg))
+    con.close()
+    assert len(rows) >= 5
+    picked = set()
+    for cfg in W.CONFIGS:
+        gm = W.fuse(W.CONFIGS[cfg].module(), prebuild._shapes_of(cfg, None))
+        (n,) = fused_nodes(gm)
+        picked.add(n.target.tile)
+    assert picked <= set(rows.values())
