@@ -15,6 +15,7 @@ from __future__ import annotations
 import json
 import os
 import sqlite3
+from contextlib import contextmanager
 from dataclasses import asdict, fields
 from pathlib import Path
 from typing import List, Optional, Sequence, Tuple
@@ -34,6 +35,21 @@ DTYPE_BY_NAME = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.floa
 
 def default_cache_file() -> Path:
     return Path(os.environ.get("EVT_TUNER_CACHE", Path(__file__).resolve().parent / "tuner_cache.db"))
+
+
+_FORCED_TILE: Optional[TileConfig] = None
+
+
+@contextmanager
+def force_tile(tile: TileConfig):
+    """Every fast-path (DMA) problem traced inside the block uses `tile` instead
+    of the cached / heuristic choice (tests of one pipeline variant, experiments)."""
+    global _FORCED_TILE
+    prev, _FORCED_TILE = _FORCED_TILE, tile
+    try:
+        yield
+    finally:
+        _FORCED_TILE = prev
 
 
 class AutoTunerBase:
@@ -95,7 +111,8 @@ class AutoTunerBase:
                               if self.ir.col_state else 0))
         out = []
         if self.dma:
-            # (bm, bn, bk, wave grid, LDS stages, pipeline): plain ring (0) or look-ahead ring (1)
+            # (bm, bn, bk, wave grid, LDS stages, pipeline): plain ring (0), look-ahead ring (1),
+            # ping-pong with two barriers (2) or one barrier (3) per k-tile
             shapes = [(256, 256, 64, 4, 2, 2, 0), (256, 256, 64, 2, 4, 2, 0), (256, 256, 32, 4, 2, 4, 1),
                       (256, 256, 32, 2, 4, 4, 1), (256, 256, 32, 4, 2, 5, 1), (256, 256, 32, 2, 4, 5, 1),
                       (256, 128, 64, 4, 2, 2, 0), (256, 128, 64, 4, 2, 3, 1), (256, 128, 32, 4, 2, 4, 1),
@@ -104,6 +121,10 @@ class AutoTunerBase:
                       (128, 256, 32, 2, 4, 6, 1),
                       (128, 128, 64, 2, 2, 2, 0), (128, 128, 64, 2, 2, 4, 1), (128, 128, 32, 2, 2, 4, 1),
                       (64, 64, 64, 2, 2, 2, 0), (64, 64, 32, 2, 2, 2, 0)]
+            for pipe in (2, 3):
+                shapes += [(256, 256, 64, 4, 2, 2, pipe), (256, 256, 64, 2, 4, 2, pipe), (256, 256, 32, 2, 4, 4, pipe),
+                           (256, 256, 32, 4, 2, 4, pipe), (256, 128, 64, 4, 2, 3, pipe), (128, 256, 64, 2, 4, 3, pipe),
+                           (128, 256, 32, 2, 4, 4, pipe), (128, 128, 64, 2, 4, 4, pipe)]
             if self.N == 512:     # one tile spans the rows: row statistics complete inside the workgroup
                 shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0)]
         else:
@@ -124,12 +145,12 @@ class AutoTunerBase:
         eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3}
         best, best_cost = None, None
         for t in self.candidates():
-            if t.pipe != 0 or t.stages == 1:
-                continue    # the plain double-buffered ring is the untuned default
+            if t.pipe not in (0, 2) or t.stages == 1:
+                continue    # untuned default: a ping-pong tile or the plain double-buffered ring
             tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
-            wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 else 1
+            wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 and t.pipe == 0 else 1
             rounds = -(-tiles // (NUM_CUS * wg_per_cu))
-            cost = rounds * wg_per_cu * t.bm * t.bn / eff.get((t.bm, t.bn), 0.5)
+            cost = rounds * wg_per_cu * t.bm * t.bn / (eff.get((t.bm, t.bn), 0.5) * (1.15 if t.pipe == 2 else 1.0))
             # deeper k-tiles and fewer stages first on ties
             cost *= 1.0 + 0.01 * (64 // t.bk - 1) + 0.005 * (t.stages - 2) + (0.002 if t.wm < t.wn else 0.0)
             if best_cost is None or cost < best_cost:
@@ -210,6 +231,8 @@ class AutoTunerBase:
         return best
 
     def get_best_config(self) -> TileConfig:
+        if _FORCED_TILE is not None and self.dma:
+            return _FORCED_TILE
         cached = self.fetch_cached()
         if cached is not None:
             return cached

@@ -29,7 +29,10 @@ class TileConfig:
     stages: int = 2
     dma: bool = True
     group_m: int = 4
-    pipe: int = 0       # 0: plain ring; 1: look-ahead ring with pinned instruction order (stages >= 3)
+    # 0: plain ring; 1: look-ahead ring with pinned instruction order (stages >= 3);
+    # 2: ping-pong, the two waves of a SIMD alternate MFMA and LDS-read phases (8 waves, stages >= 2);
+    # 3: ping-pong with one barrier per k-tile
+    pipe: int = 0
 
     def tag(self) -> str:
         return (f"{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_s{self.stages}"

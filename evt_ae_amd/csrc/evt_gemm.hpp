@@ -67,7 +67,16 @@ struct GemmCfg {
   //         iteration early so the first fragments of the next k-tile are
   //         fetched under the MFMAs of the current one, and the instruction
   //         order (MFMA / LDS read / DMA issue) is pinned.
+  // PIPE 2: ping-pong (8 waves, STAGES >= 2): the two waves that share a SIMD
+  //         alternate between a phase of back-to-back MFMAs on fragments held
+  //         in registers and a phase of LDS fragment reads; a workgroup
+  //         barrier ends every phase, so one wave's LDS traffic always runs
+  //         under the other wave's MFMAs.
+  // PIPE 3: ping-pong with one barrier per k-tile: the barrier between a
+  //         group's read phase and its MFMA phase is dropped and wave
+  //         priorities keep the two waves of a SIMD out of step.
   static constexpr int PIPE = PIPE_;
+  static constexpr bool PINGPONG = PIPE_ == 2 || PIPE_ == 3;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DMA = DMA_, BF16 = BF16_;
   static constexpr int STAGES = STAGES_, GROUP_M = GROUP_M_;
@@ -89,7 +98,9 @@ struct GemmCfg {
   static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be 32-aligned");
   static_assert(STAGES >= 1 && STAGES <= 8, "1..8 stages");
-  static_assert(PIPE == 0 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
+  static_assert(PIPE != 1 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
+  static_assert(!PINGPONG || (DMA && STAGES >= 2 && WM * WN == 8), "ping-pong needs DMA, >= 2 stages, 8 waves");
+  static_assert(PIPE >= 0 && PIPE <= 3, "unknown pipeline");
 };
 
 // ---------------------------------------------------------------------------
@@ -197,16 +208,24 @@ struct Operand {
   }
 
   // ---- fast path: global -> LDS DMA of k-tile `kt` into `lds` -------------
-  EVT_DEV void dma(int kt, char* lds, int wave) const {
+  struct DmaTile {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int k0;
+  };
+  EVT_DEV DmaTile dma_begin(int kt) const {
     const int64_t adv = SRC_KC ? (int64_t)kt * BK * 2 : (int64_t)kt * BK * ld * 2;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base + adv);
-    const int k0 = kt * BK;
+    return DmaTile{make_rsrc(base + adv), kt * BK};
+  }
+  // transfer number i (of NLOAD) of this thread
+  EVT_DEV void dma_chunk(const DmaTile& d, char* lds, int wave, int i) const {
+    const uint32_t v = (d.k0 + kin[i] < K) ? voff[i] : kOobOffset;
+    char* dst = lds + (i * THREADS + wave * 64) * 16;   // wave-uniform; lane*16 added by hardware
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(d.rsrc, (lds_void_ptr)dst, 16, v, 0, 0, 0);
+  }
+  EVT_DEV void dma(int kt, char* lds, int wave) const {
+    const DmaTile d = dma_begin(kt);
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const uint32_t v = (k0 + kin[i] < K) ? voff[i] : kOobOffset;
-      char* dst = lds + (i * THREADS + wave * 64) * 16;   // wave-uniform; lane*16 added by hardware
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)dst, 16, v, 0, 0, 0);
-    }
+    for (int i = 0; i < NLOAD; ++i) dma_chunk(d, lds, wave, i);
   }
 
   // ---- safe path: element-wise guarded gather through registers ----------
@@ -241,6 +260,26 @@ struct Operand {
     }
   }
 };
+
+// LDS reads issued through inline assembly.  The compiler orders every LDS
+// access it can see behind all outstanding global->LDS transfers (it cannot
+// tell the ring stages apart), which would drain the DMA ring at each k-tile;
+// these reads are invisible to that logic.  The caller waits for them with
+// lds_wait_all() and then passes every destination through lds_pin().
+EVT_DEV u32x4 lds_read_b128(uint32_t addr) {
+  u32x4 r;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+EVT_DEV u32x2 lds_read_tr16_b64(uint32_t addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+EVT_DEV void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+template <class T>
+EVT_DEV void lds_pin(T& x) { asm volatile("" : "+v"(x)); }
+EVT_DEV uint32_t lds_addr(const char* p) { return (uint32_t)(uintptr_t)p; }
 
 // Per-lane LDS read addressing of MFMA operand fragments (32 rows x 16 k).
 template <int ROWS, int BK, bool LDS_KC, int NFRAG>
@@ -279,6 +318,48 @@ struct FragReader {
       u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
       u32x4 r;
       r.x = l2.x; r.y = l2.y; r.z = h2.x; r.w = h2.y;
+      return r;
+    }
+  }
+
+  // All fragments of one k-tile (ping-pong pipeline), read with the inline
+  // assembly helpers: issue(), then lds_wait_all(), then pin(), then frag().
+  static constexpr int KSN = BK / 16;
+  struct Tile {
+    u32x4 q[LDS_KC ? KSN * NFRAG : 1];
+    u32x2 h[LDS_KC ? 1 : 2 * KSN * NFRAG];
+  };
+  EVT_DEV void issue(uint32_t lds, Tile& t) const {
+#pragma unroll
+    for (int ks = 0; ks < KSN; ++ks) {
+#pragma unroll
+      for (int f = 0; f < NFRAG; ++f) {
+        if constexpr (LDS_KC) {
+          t.q[ks * NFRAG + f] = lds_read_b128(lds + off[ks] + f * (32 * CH * 16));
+        } else {
+          const uint32_t p = lds + off[f] + ks * (16 * RC * 16);
+          t.h[2 * (ks * NFRAG + f)] = lds_read_tr16_b64(p);
+          t.h[2 * (ks * NFRAG + f) + 1] = lds_read_tr16_b64(p + 4 * RC * 16);
+        }
+      }
+    }
+  }
+  EVT_DEV void pin(Tile& t) const {
+    if constexpr (LDS_KC) {
+#pragma unroll
+      for (int i = 0; i < KSN * NFRAG; ++i) lds_pin(t.q[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2 * KSN * NFRAG; ++i) lds_pin(t.h[i]);
+    }
+  }
+  EVT_DEV u32x4 frag(const Tile& t, int f, int ks) const {
+    if constexpr (LDS_KC) {
+      return t.q[ks * NFRAG + f];
+    } else {
+      const u32x2 lo = t.h[2 * (ks * NFRAG + f)], hi = t.h[2 * (ks * NFRAG + f) + 1];
+      u32x4 r;
+      r.x = lo.x; r.y = lo.y; r.z = hi.x; r.w = hi.y;
       return r;
     }
   }
@@ -484,6 +565,150 @@ struct Mainloop {
     for (; kt < KT; ++kt) lookahead_iter<false>(kt, KT, stage, a, b, ra, rb, smem, wave, f, acc);
   }
 
+  // ---- ping-pong pipeline (PIPE == 2) --------------------------------------
+  // Waves w and w+4 run on the same SIMD.  Group 0 (waves 0-3) and group 1
+  // (waves 4-7) each walk the k-tiles with two phases per tile: R(T) reads all
+  // fragments of tile T from LDS into registers, C(T) issues the MFMAs of tile
+  // T.  A workgroup barrier ends every phase and group 1 runs one phase behind
+  // group 0, so at any time one wave of a SIMD is in C and the other in R:
+  //
+  //   phase      2T          2T+1        2T+2        2T+3
+  //   group 0    R(T)        C(T)        R(T+1)      C(T+1)
+  //   group 1    C(T-1)      R(T)        C(T)        R(T+1)
+  //
+  // Tile T is read during phases 2T and 2T+1, so the stage of tile T-1 may be
+  // refilled with tile T+STAGES-1 from phase 2T on.  The texture path moves
+  // only about 64 bytes per clock, so a wave that issues its transfers in one
+  // burst stalls for hundreds of cycles; the transfers are therefore spread
+  // between the MFMAs of a C phase: group 1 issues its share in C(T-1) (phase
+  // 2T) and, with three or more stages, group 0 its share in C(T) (phase
+  // 2T+1).  With two stages group 0 has to issue at the start of R(T) to give
+  // the data two phases to land.  Every wave waits for its share of tile T+1
+  // before the barrier that ends phase 2T+1.  Both groups execute exactly
+  // 1 + 2*KT barriers.  Only the barriers that end the odd phases order memory
+  // (tile T+1 visible, stage of tile T free); the ones that end the even phases
+  // merely pace the two groups, and PIPE 3 leaves them out: group 1 then runs
+  // its MFMA phase at a higher wave priority than group 0, so after each
+  // barrier group 1 computes first while group 0 reads, and they swap.
+  struct TileFrags {
+    typename RdA::Tile a;
+    typename RdB::Tile b;
+  };
+  static constexpr int PP_NM = Cfg::KS * Cfg::MI * Cfg::NI;   // MFMAs per C phase
+  static constexpr bool PP_G0_ISSUES_IN_C = Cfg::STAGES >= 3;
+  // R phase: all fragments of the tile at `lds` are in registers on return
+  static EVT_DEV void pp_read(TileFrags& f, const char* lds, const RdA& ra, const RdB& rb) {
+    ra.issue(lds_addr(lds), f.a);
+    rb.issue(lds_addr(lds + Cfg::A_BYTES), f.b);
+    lds_wait_all();
+    ra.pin(f.a);
+    rb.pin(f.b);
+  }
+  // transfer c (of LPS) goes behind MFMA number (c * PP_NM) / LPS
+  template <int M>
+  static EVT_DEV void pp_pin_order() {
+    if constexpr (M < PP_NM) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      constexpr int n = ((M + 1) * LPS + PP_NM - 1) / PP_NM - (M * LPS + PP_NM - 1) / PP_NM;
+      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x020, n, 0);
+      pp_pin_order<M + 1>();
+    }
+  }
+  // C phase; with ISSUE the transfers of k-tile `nk` into stage `ds` are spread between the MFMAs
+  template <bool ISSUE, int PRIO = 1>
+  static EVT_DEV void pp_mma(const TileFrags& f, const RdA& ra, const RdB& rb, f32x16 (&acc)[Cfg::MI][Cfg::NI],
+                             const OpA& a, const OpB& b, int nk, char* ds, int wave) {
+    typename OpA::DmaTile da;
+    typename OpB::DmaTile db;
+    if constexpr (ISSUE) {
+      da = a.dma_begin(nk);
+      db = b.dma_begin(nk);
+    }
+#ifndef EVT_NO_SETPRIO
+    __builtin_amdgcn_s_setprio(PRIO);
+#endif
+#pragma unroll
+    for (int ks = 0; ks < Cfg::KS; ++ks) {
+#pragma unroll
+      for (int mi = 0; mi < Cfg::MI; ++mi) {
+#pragma unroll
+        for (int ni = 0; ni < Cfg::NI; ++ni) {
+          acc[mi][ni] = mfma32<Cfg::BF16>(ra.frag(f.a, mi, ks), rb.frag(f.b, ni, ks), acc[mi][ni]);
+          if constexpr (ISSUE) {
+            const int m = (ks * Cfg::MI + mi) * Cfg::NI + ni;
+#pragma unroll
+            for (int c = 0; c < LPS; ++c) {
+              if ((c * PP_NM) / LPS == m) {
+                if (c < OpA::NLOAD) a.dma_chunk(da, ds, wave, c);
+                else b.dma_chunk(db, ds + Cfg::A_BYTES, wave, c - OpA::NLOAD);
+              }
+            }
+          }
+        }
+      }
+    }
+    if constexpr (ISSUE) pp_pin_order<0>();
+#ifndef EVT_NO_SETPRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
+  }
+  // Transfers are issued for every T, also past the last k-tile: a tile index
+  // beyond K reads as zeros through the buffer range check (no memory traffic)
+  // and lands in a stage nobody reads any more, which keeps the vmcnt
+  // bookkeeping uniform and the loop free of a second code path.
+  static EVT_DEV char* pp_refill_stage(int stage, char* smem) {   // the stage tile T-1 occupied
+    const int ds = stage == 0 ? Cfg::STAGES - 1 : stage - 1;
+    return smem + ds * Cfg::STAGE_BYTES;
+  }
+  static EVT_DEV void pp_issue(int T, int stage, const OpA& a, const OpB& b, char* smem, int wave) {
+    char* ds = pp_refill_stage(stage, smem);
+    a.dma(T + Cfg::STAGES - 1, ds, wave);
+    b.dma(T + Cfg::STAGES - 1, ds + Cfg::A_BYTES, wave);
+  }
+  // Phase barriers are bare s_barrier instructions: the only memory traffic of
+  // the loop is the DMA (waited for explicitly with vmcnt) and the
+  // inline-assembly LDS reads (waited for inside pp_read); a fence here would
+  // make the compiler drain the DMA ring at every phase.
+  static EVT_DEV void pp_barrier() { __builtin_amdgcn_s_barrier(); }
+  static EVT_DEV void run_pingpong(const OpA& a, const OpB& b, const RdA& ra, const RdB& rb, char* smem,
+                                   int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+    constexpr int S = Cfg::STAGES;
+    static_assert((S - 1) * LPS < 64, "vmcnt is a 6-bit counter");
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+      a.dma(s, smem + s * Cfg::STAGE_BYTES, wave);
+      b.dma(s, smem + s * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+    }
+    wait_tiles<S - 2>();            // tile 0 has landed
+    __syncthreads();
+    TileFrags f;
+    int stage = 0;
+    const int grp = wave >> 2;
+    if (grp == 0) {
+      for (int T = 0; T < KT; ++T) {
+        if constexpr (!PP_G0_ISSUES_IN_C) pp_issue(T, stage, a, b, smem, wave);
+        pp_read(f, smem + stage * Cfg::STAGE_BYTES, ra, rb);
+        if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
+        pp_mma<PP_G0_ISSUES_IN_C>(f, ra, rb, acc, a, b, T + S - 1, pp_refill_stage(stage, smem), wave);
+        wait_tiles<S - 2>();        // my share of tile T+1 has landed
+        pp_barrier();               // ends phase 2T+1
+        stage = stage + 1 == S ? 0 : stage + 1;
+      }
+    } else {
+      pp_issue(0, 0, a, b, smem, wave);
+      for (int T = 0; T < KT; ++T) {
+        if (T > 0) pp_mma<true, 2>(f, ra, rb, acc, a, b, T + S - 1, pp_refill_stage(stage, smem), wave);   // C(T-1)
+        if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
+        pp_read(f, smem + stage * Cfg::STAGE_BYTES, ra, rb);
+        wait_tiles<S - 2>();        // my share of tile T+1 has landed
+        pp_barrier();               // ends phase 2T+1
+        stage = stage + 1 == S ? 0 : stage + 1;
+      }
+      if (KT > 0) pp_mma<false>(f, ra, rb, acc, a, b, 0, smem, wave);   // C(KT-1)
+    }
+    wait_vmcnt<0>();                // the zero-fill transfers past the last tile have landed
+  }
+
   static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, char* smem,
                           f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
     const int tid = threadIdx.x;
@@ -515,6 +740,8 @@ struct Mainloop {
 
     if constexpr (Cfg::PIPE == 1) {
       run_lookahead(a, b, ra, rb, smem, wave, KT, acc);
+    } else if constexpr (Cfg::PINGPONG) {
+      run_pingpong(a, b, ra, rb, smem, wave, KT, acc);
     } else if constexpr (Cfg::DMA && Cfg::STAGES == 1) {
       // K fits one tile (checked by the host): load it, use it
       a.dma(0, smem, wave);

@@ -46,6 +46,11 @@ def register_all() -> List[jit.LazyModule]:
     for cfg in W.CONFIGS:
         for shapes in (None, W.SMALL_SHAPES[cfg], W.RAGGED_SHAPES[cfg], W.UNALIGNED_SHAPES[cfg], W.GOLDEN_SHAPES[cfg]):
             W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
+    from .autotuner.tuner_base import force_tile
+    for tile in W.pipeline_tiles():
+        with force_tile(tile):
+            for cfg in W.CONFIGS:
+                W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, W.PIPELINE_SHAPES[cfg]))
     for name, (cls, _) in W.REFERENCE_PATTERNS.items():
         g = torch.Generator(device="cpu").manual_seed(0)
         # shapes only: generate on CPU lazily is costly for the big patterns, so

@@ -165,6 +165,15 @@ GOLDEN_SHAPES = {
     4: dict(M=96, N=64, K=64),
     5: dict(M=32, N=512, K=64),
 }
+# several workgroup tiles in M and N, several k-tiles with a K tail: the shapes
+# the main-loop pipeline variants (PIPELINE_TILES) are checked on
+PIPELINE_SHAPES = {
+    1: dict(M=300, N=264, K=200),
+    2: dict(L=2, S=200, D=72),
+    3: dict(M=264, N=520, K=328),
+    4: dict(M=520, N=264, K=136),
+    5: dict(M=136, N=1032, K=264),
+}
 # no dimension a multiple of 8: operands are not 16-byte aligned row by row, so
 # these run the element-wise (safe) operand path
 UNALIGNED_SHAPES = {
@@ -180,6 +189,15 @@ def make_inputs(cfg: int, shapes: dict = None, seed: int = None) -> List[torch.T
     g = torch.Generator(device="cpu").manual_seed(CONFIGS[cfg].seed(cfg) if seed is None else seed)
     fn = CONFIGS[cfg].make_inputs
     return fn(g, **(shapes or {}))
+
+
+def pipeline_tiles():
+    """Ping-pong main-loop variants (pipe 2: two barriers per k-tile, pipe 3:
+    one) on every stage count / k-depth / wave grid they are instantiated with."""
+    from .codegen import TileConfig
+    return [TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 2),
+            TileConfig(256, 256, 32, 2, 4, 4, True, 4, 2), TileConfig(256, 128, 64, 4, 2, 3, True, 4, 3),
+            TileConfig(128, 256, 64, 2, 4, 3, True, 4, 3), TileConfig(256, 256, 64, 2, 4, 2, True, 4, 3)]
 
 
 def unfused_eager(cfg: int) -> Callable:

@@ -10,6 +10,7 @@ import pytest
 import torch
 
 from evt_ae_amd import workloads as W
+from evt_ae_amd.autotuner.tuner_base import force_tile
 from oracle import evt_oracle
 from tests.util import fused_nodes
 
@@ -19,10 +20,15 @@ FP16_TOL = 2e-2
 REDUCTION_TOL = 1e-3
 
 
-def _run(cfg, shapes, seed=None):
+def _run(cfg, shapes, seed=None, tile=None):
     wl = W.CONFIGS[cfg]
     inputs = W.make_inputs(cfg, shapes, seed)
-    gm = W.fuse(wl.module(), inputs)
+    if tile is None:
+        gm = W.fuse(wl.module(), inputs)
+    else:
+        with force_tile(tile):
+            gm = W.fuse(wl.module(), inputs)
+        assert fused_nodes(gm)[0].target.tile == tile
     assert len(fused_nodes(gm)) == 1
     outs = gm(*[t.cuda() for t in inputs])
     outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
@@ -44,6 +50,15 @@ def _compare(wl, outs, refs):
 def test_configs_against_oracle(cfg, shapes):
     sh = {"small": W.SMALL_SHAPES, "ragged": W.RAGGED_SHAPES, "unaligned": W.UNALIGNED_SHAPES}[shapes][cfg]
     wl, inputs, gm, outs = _run(cfg, sh)
+    _compare(wl, outs, evt_oracle.eval_fp32(wl.module(), inputs))
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", W.pipeline_tiles(), ids=lambda t: t.tag())
+def test_pipeline_variants_against_oracle(cfg, tile):
+    """Every ping-pong main-loop variant on shapes with several tiles in M, N and
+    K, partial edge tiles and a K tail (one k-tile only for the batched config)."""
+    wl, inputs, gm, outs = _run(cfg, W.PIPELINE_SHAPES[cfg], tile=tile)
     _compare(wl, outs, evt_oracle.eval_fp32(wl.module(), inputs))
 
 
