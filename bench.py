@@ -75,6 +75,27 @@ class Case:
         a, _, _, _, ws_ptr, ws_bytes = self.sets[i % self.nsets]
         self.module.launch(a, ws_ptr, ws_bytes, self.torch.cuda.current_stream().cuda_stream)
 
+    def clock_probe(self, jit, spin_seconds=0.3):
+        """Run the diagnostic build of the same kernel under sustained load and read what workgroup 0 timed:
+        shader clock (cycles per 100 MHz tick) and the split between main loop and epilogue."""
+        probe = jit.load_module(self.op.ir, self.op.spec, clock_probe=True).ensure()
+        stream = self.torch.cuda.current_stream().cuda_stream
+
+        def fn(i):
+            a, _, _, _, ws_ptr, ws_bytes = self.sets[i % self.nsets]
+            probe.launch(a, ws_ptr, ws_bytes, stream)
+        spin_up(self.torch, fn, spin_seconds)
+        samples = []
+        for i in range(8):
+            fn(i)
+            self.torch.cuda.synchronize()
+            samples.append(probe.clock_probe_read())
+        samples.sort(key=lambda s: s[1] + s[3])
+        c_main, r_main, c_epi, r_epi = samples[len(samples) // 2]
+        return {"shader_mhz": round(100.0 * (c_main + c_epi) / max(r_main + r_epi, 1), 0),
+                "wg0_mainloop_us": round(r_main / 100.0, 2), "wg0_epilogue_us": round(r_epi / 100.0, 2),
+                "wg0_mainloop_cycles": c_main, "wg0_epilogue_cycles": c_epi}
+
     def launch_unfused(self, i):
         return self.unfused(*self.sets[i % self.nsets][3])
 
@@ -199,13 +220,16 @@ def main():
     ap.add_argument("--configs", default="1,2,3,4,5")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB streaming kernel (torch.neg, known traffic) so HBM counters can be scaled")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="also run a diagnostic build of each kernel that reports the shader clock it ran at and "
+                         "workgroup 0's main-loop / epilogue split (per_config[*].clock_probe)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU (the fused GEMM+epilogue path has no cross-GPU exchange); "
                  "run with --gpus 1")
 
     import torch
-    from evt_ae_amd import workloads as W
+    from evt_ae_amd import jit, workloads as W
     from oracle import evt_oracle
     fused_nodes = W.fused_nodes
 
@@ -248,6 +272,8 @@ def main():
             "speedup_vs_unfused": round(best_unf / best, 3),
             "max_rel_err": parity, "buffer_sets": case.nsets, "_ms": ms, "_best": best,
         }
+        if args.clock_probe:
+            details[cfg]["clock_probe"] = case.clock_probe(jit)
         log(f"[bench] config {cfg} {wl.name}: {details[cfg]}")
         del case
         torch.cuda.empty_cache()

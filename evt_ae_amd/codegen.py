@@ -96,10 +96,13 @@ class _Emitter:
 
 
 class Codegen:
-    def __init__(self, ir: EpilogueIR, spec: KernelSpec, module_name: str):
+    def __init__(self, ir: EpilogueIR, spec: KernelSpec, module_name: str, clock_probe: bool = False):
         self.ir = ir
         self.spec = spec
         self.name = module_name
+        # diagnostic build: workgroup 0 times its main loop and its epilogue with the shader-clock and the
+        # constant 100 MHz counters, and the module exports evt_clock_probe_read
+        self.clock_probe = clock_probe
         # variance of every node: does it vary along m / along n?
         self.var_m: Dict[str, bool] = {}
         self.var_n: Dict[str, bool] = {}
@@ -419,6 +422,8 @@ class Codegen:
         e = _Emitter()
         e("// Generated by evt_ae_amd.codegen -- do not edit.")
         e(f"// module {self.name}")
+        if self.clock_probe:
+            e("#define EVT_CLOCK_PROBE 1")
         e('#include "evt_epilogue.hpp"')
         e('#include "evt_amd.h"')
         e("#include <stdlib.h>")
@@ -538,8 +543,14 @@ class Codegen:
         e("  if (err != 0) return err;")
         e("  return evt::launch_finalize<Epi>(p, g, (hipStream_t)stream);")
         e("}")
+        if self.clock_probe:
+            e("// out[0..3] = main-loop shader cycles, main-loop 100 MHz ticks, epilogue shader cycles, epilogue ticks")
+            e("// of workgroup 0 in the most recent launch (synchronises the device)")
+            e('extern "C" int evt_clock_probe_read(uint64_t* out) {')
+            e("  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(evt::evt_clock_probe), 4 * sizeof(uint64_t));")
+            e("}")
         return e.text()
 
 
-def generate(ir: EpilogueIR, spec: KernelSpec, module_name: str) -> str:
-    return Codegen(ir, spec, module_name).source()
+def generate(ir: EpilogueIR, spec: KernelSpec, module_name: str, clock_probe: bool = False) -> str:
+    return Codegen(ir, spec, module_name, clock_probe).source()

@@ -551,13 +551,26 @@ EVT_DEV void combine_welford(float& n, float& mean, float& m2, float nb, float m
 // The fused kernel.  Interior tiles whose epilogue tensors are all unit-stride
 // (p.fast, decided on the host) take the check-free epilogue; everything else
 // takes the guarded one.
+#ifdef EVT_CLOCK_PROBE
+// Diagnostic build only: {main-loop shader cycles, main-loop 100 MHz ticks,
+// epilogue shader cycles, epilogue 100 MHz ticks} of workgroup 0.  The ratio
+// cycles / ticks is the shader clock the kernel actually ran at.
+__device__ uint64_t evt_clock_probe[4];
+#endif
+
 template <class Cfg, class Epi>
 __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
   __shared__ __attribute__((aligned(1024))) char smem[Cfg::LDS_BYTES];
   int batch, tm, tn;
   tile_coords<Cfg::GROUP_M>(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
   f32x16 acc[Cfg::MI][Cfg::NI];
+#ifdef EVT_CLOCK_PROBE
+  const uint64_t probe_c0 = __builtin_amdgcn_s_memtime(), probe_r0 = __builtin_amdgcn_s_memrealtime();
+#endif
   Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, smem, acc);
+#ifdef EVT_CLOCK_PROBE
+  const uint64_t probe_c1 = __builtin_amdgcn_s_memtime(), probe_r1 = __builtin_amdgcn_s_memrealtime();
+#endif
   if (p.fast && (tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
     TileCtx<Cfg, true> t;
     t.init(g, batch, tm, tn, smem);
@@ -567,6 +580,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, type
     t.init(g, batch, tm, tn, smem);
     Epi::template tile<Cfg, TileCtx<Cfg, false>, false>(p, t, g, acc);
   }
+#ifdef EVT_CLOCK_PROBE
+  __builtin_amdgcn_s_waitcnt(0);   // the epilogue's stores have been issued and acknowledged
+  const uint64_t probe_c2 = __builtin_amdgcn_s_memtime(), probe_r2 = __builtin_amdgcn_s_memrealtime();
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    evt_clock_probe[0] = probe_c1 - probe_c0;
+    evt_clock_probe[1] = probe_r1 - probe_r0;
+    evt_clock_probe[2] = probe_c2 - probe_c1;
+    evt_clock_probe[3] = probe_r2 - probe_r1;
+  }
+#endif
 }
 
 __global__ void evt_fill_zero_kernel(uint32_t* p, int64_t n) {

@@ -73,6 +73,9 @@ class KernelModule:
         self.lib.evt_launch.argtypes = [ctypes.POINTER(EvtArgs), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         if self.lib.evt_abi_version() != 1:
             raise RuntimeError(f"{path}: ABI version mismatch")
+        if hasattr(self.lib, "evt_clock_probe_read"):      # diagnostic builds only
+            self.lib.evt_clock_probe_read.restype = ctypes.c_int
+            self.lib.evt_clock_probe_read.argtypes = [ctypes.POINTER(ctypes.c_uint64)]
         self.spec = json.loads(self.lib.evt_module_spec().decode())
 
     def workspace_bytes(self, args: EvtArgs) -> int:
@@ -85,6 +88,17 @@ class KernelModule:
         rc = self.lib.evt_workspace_init(ctypes.c_void_p(ptr), nbytes, ctypes.c_void_p(stream))
         if rc != 0:
             raise RuntimeError(f"HIP Error {rc} in evt_workspace_init")
+
+    def clock_probe_read(self):
+        """(main-loop cycles, main-loop 100 MHz ticks, epilogue cycles, epilogue ticks) of workgroup 0 in the
+        last launch; only modules generated with clock_probe=True export it."""
+        if not hasattr(self.lib, "evt_clock_probe_read"):
+            raise RuntimeError(f"{self.path.name} was not built with the clock probe")
+        out = (ctypes.c_uint64 * 4)()
+        rc = self.lib.evt_clock_probe_read(out)
+        if rc != 0:
+            raise RuntimeError(f"HIP Error {rc} in evt_clock_probe_read")
+        return tuple(int(x) for x in out)
 
     def launch(self, args: EvtArgs, ws_ptr: int, ws_bytes: int, stream: int) -> None:
         rc = self.lib.evt_launch(ctypes.byref(args), ctypes.c_void_p(ws_ptr), ws_bytes, ctypes.c_void_p(stream))
@@ -144,11 +158,11 @@ class LazyModule:
     use, so that tracing a graph never needs hipcc or a GPU.  Modules built
     ahead of time (evt_ae_amd.prebuild) are found by their hash."""
 
-    def __init__(self, ir: EpilogueIR, spec: KernelSpec):
+    def __init__(self, ir: EpilogueIR, spec: KernelSpec, clock_probe: bool = False):
         from .codegen import Codegen
         self.ir, self.kernel_spec = ir, spec
-        self.name = f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}"
-        cg = Codegen(ir, spec, self.name)
+        self.name = f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}" + ("_probe" if clock_probe else "")
+        cg = Codegen(ir, spec, self.name, clock_probe)
         self.source = cg.source()
         self.spec_json = json.dumps(cg.module_spec(), sort_keys=True)
         self.hash = module_hash(self.source)
@@ -185,12 +199,15 @@ class LazyModule:
     def launch(self, args: EvtArgs, ws_ptr: int, ws_bytes: int, stream: int) -> None:
         self.ensure().launch(args, ws_ptr, ws_bytes, stream)
 
+    def clock_probe_read(self):
+        return self.ensure().clock_probe_read()
+
 
 _registry: Dict[str, LazyModule] = {}
 
 
-def load_module(ir: EpilogueIR, spec: KernelSpec) -> LazyModule:
-    mod = LazyModule(ir, spec)
+def load_module(ir: EpilogueIR, spec: KernelSpec, clock_probe: bool = False) -> LazyModule:
+    mod = LazyModule(ir, spec, clock_probe)
     with _lock:
         return _registry.setdefault(str(mod.path), mod)
 
