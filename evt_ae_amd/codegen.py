@@ -118,6 +118,8 @@ class Codegen:
                 # a batch-dependent value is re-read per row slot only if it also
                 # depends on m; a pure batch scalar is workgroup-uniform
                 vm = st.stride_m != 0
+                if ir.slots[n.slot].kind == "rand":
+                    vm, vn = True, True
             elif n.op in ("imm", "rres"):
                 vm, vn = False, False
             else:
@@ -339,7 +341,13 @@ class Codegen:
             k = n.slot
             s = self.ir.slots[k]
             base = self.slot_off(k)
-            if s.kind == "aux":
+            if s.kind == "rand":
+                r = self.ir.rng_scalar
+                e(f"float {c}[NI];")
+                e(f"evt::rand_row<Tile>((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r}]) | ((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r + 1}]) << 32), "
+                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u, "
+                  f"{base} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, p.t{k}_sn, {c});")
+            elif s.kind == "aux":
                 e(f"float {c}[NI];")
                 e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = (float)r_{c}[v][ni];")
             elif s.kind == "row":
@@ -415,6 +423,8 @@ class Codegen:
             "tensors": [{"name": s.name, "role": s.role, "dtype": s.dtype, "kind": s.kind,
                          "domain": s.domain} for s in self.ir.slots],
             "num_scalars": len(self.ir.scalars),
+            # scalars[rng_scalars .. +3] = 32-bit patterns of (seed low, seed high, offset, unused) for rand_like
+            "rng_scalars": self.ir.rng_scalar,
         }
 
     def source(self) -> str:
@@ -497,7 +507,10 @@ class Codegen:
         for k, s in enumerate(ir.slots):
             ct = DTYPE_CTYPES[s.dtype]
             e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
-            e("  if (!x.ptr || x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
+            if s.kind == "rand":   # generated values: no storage behind this slot
+                e("  if (x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
+            else:
+                e("  if (!x.ptr || x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
             e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
             e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div;")
             e(f"  p.t{k}_vec = (x.stride_n == 1 ? 1 : 0) | ((x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "

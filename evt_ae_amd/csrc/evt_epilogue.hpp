@@ -197,6 +197,51 @@ EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, 
 }
 
 // ---------------------------------------------------------------------------
+// rand_like: counter-based uniform numbers, one Philox4x32-10 block per four
+// consecutive elements of the rand_like tensor.  Element e (row-major index in
+// that tensor) takes word (e & 3) of
+//   Philox4x32-10(counter = (lo32(e >> 2), hi32(e >> 2), lo32(offset), salt),
+//                 key = (lo32(seed), hi32(seed)))
+// mapped to [0, 1) as (word >> 8) * 2^-24, so the values do not depend on the
+// tile configuration.  Takes the place of VisitorRand (curand Philox4_32_10
+// with a per-thread subsequence,
+// src/cuda/epilogue/threadblock/visitor_load.hpp:79-151).
+// ---------------------------------------------------------------------------
+EVT_DEV void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c[0]), lo0 = 0xD2511F53u * c[0];
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c[2]), lo1 = 0xCD9E8D57u * c[2];
+    c[0] = hi1 ^ c[1] ^ k0;
+    c[1] = lo1;
+    c[2] = hi0 ^ c[3] ^ k1;
+    c[3] = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+}
+
+// NI values of one accumulator row; e0 is the element index of (row, col(0)),
+// sn the index step between neighbouring columns.
+template <class Tile>
+EVT_DEV void rand_row(uint64_t seed, uint32_t offset, uint32_t salt, int64_t e0, int64_t sn, float (&out)[Tile::NI]) {
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  int64_t group = -1;
+#pragma unroll
+  for (int ni = 0; ni < Tile::NI; ++ni) {
+    const int64_t e = e0 + (int64_t)ni * Tile::COL_STEP * sn;
+    if (ni == 0 || (e >> 2) != group) {   // neighbouring columns of an interleaved lane share a block
+      group = e >> 2;
+      w[0] = (uint32_t)group; w[1] = (uint32_t)((uint64_t)group >> 32); w[2] = offset; w[3] = salt;
+      philox4x32_10(w, (uint32_t)seed, (uint32_t)(seed >> 32));
+    }
+    const int sel = (int)(e & 3);
+    const uint32_t word = sel == 0 ? w[0] : sel == 1 ? w[1] : sel == 2 ? w[2] : w[3];
+    out[ni] = (float)(word >> 8) * 5.9604644775390625e-08f;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // cross-lane exchange inside one 32-lane half of a wave (the 32 lanes that hold
 // the 32 columns of one accumulator row).  After the 5 steps every lane of the
 // half holds the combined value.

@@ -11,6 +11,7 @@ un-vendored CUTLASS Python package.
 """
 from __future__ import annotations
 
+import ctypes
 import operator
 import os
 from contextlib import nullcontext
@@ -93,6 +94,11 @@ class FusedOpBase:
         self.slot_sources = epilogue_visitor.slot_sources      # slot -> ('input', idx) | ('output', store name)
         self.store_meta = epilogue_visitor.store_meta          # store name -> (shape, dtype)
         self._workspace = {}
+        # rand_like stream: 64-bit seed (torch's global seed at trace time unless set) and a 32-bit offset that
+        # advances by one per launch, so successive calls draw different numbers
+        self.rand_seed = int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF
+        self.rand_offset = 0
+        self.last_rand_state: Optional[Tuple[int, int]] = None   # (seed, offset) the most recent launch used
 
     # -- to be provided by subclasses -----------------------------------------
     module: jit.KernelModule
@@ -117,15 +123,26 @@ class FusedOpBase:
         a.num_scalars = len(self.ir.scalars)
         keep = [A, B]
         for k, slot in enumerate(self.ir.slots):
-            kind, ref = self.slot_sources[k]
-            t = args[ref] if kind == "input" else visitor_args[ref]
-            keep.append(t)
             ta = a.tensors[k]
-            ta.ptr = t.data_ptr()
+            if slot.kind == "rand":      # generated in the kernel: strides only
+                ta.ptr = None
+            else:
+                kind, ref = self.slot_sources[k]
+                t = args[ref] if kind == "input" else visitor_args[ref]
+                keep.append(t)
+                ta.ptr = t.data_ptr()
             ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
             ta.l_div = slot.strides.l_div
         for i, s in enumerate(self.ir.scalars):
             a.scalars[i] = s
+        if self.ir.rng_scalar is not None:
+            # 32-bit patterns, not float values: written through an integer view of the scalar array
+            bits = (ctypes.c_uint32 * jit.EVT_MAX_SCALARS).from_buffer(a, jit.EvtArgs.scalars.offset)
+            r = self.ir.rng_scalar
+            bits[r], bits[r + 1] = self.rand_seed & 0xFFFFFFFF, (self.rand_seed >> 32) & 0xFFFFFFFF
+            bits[r + 2], bits[r + 3] = self.rand_offset & 0xFFFFFFFF, 0
+            self.last_rand_state = (self.rand_seed, self.rand_offset & 0xFFFFFFFF)
+            self.rand_offset += 1
         return a, keep
 
     def workspace_for(self, a: jit.EvtArgs, stream, device) -> Tuple[int, int]:
@@ -526,7 +543,9 @@ class EVTFuser:
     def _rebuild_slot_sources(self):
         self.slot_sources = {}
         for k, slot in enumerate(self.ir.slots):
-            if slot.role == "load":
+            if slot.kind == "rand":
+                self.slot_sources[k] = ("rand", None)
+            elif slot.role == "load":
                 node = next(n for n in self.input_nodes if n.name == slot.name)
                 self.slot_sources[k] = ("input", self.input_index[node])
             else:
@@ -770,7 +789,21 @@ class EVTFuser:
         return self._visit_compute(node, "where")
 
     def visit_rand_like(self, node: Node):
-        raise NotImplementedError("fused dropout (rand_like) is not provided yet")
+        """Uniform [0, 1) numbers shaped like an accumulator-dependent tensor
+        (the reference's FunctionalOp.Rand, evt_fuser.py:1383-1384).  The values
+        come from a counter-based generator indexed by the element's row-major
+        position in the rand_like tensor, so they do not depend on the tile
+        configuration; seed and per-call offset are run-time scalars."""
+        coord = self._coord_for(node)
+        self.coords[node] = coord
+        st = fit_strides(coord, self.L, self.M, self.N)
+        if st is None or st.kind != "aux":
+            raise NotImplementedError("rand_like of a tensor that is not laid out over (l, m, n)")
+        shape, _ = node_shape_dtype(node)
+        self.ir.add_rand(node.name, st, shape)
+        self.ir_name[node] = node.name
+        self.full.add(node)
+        return node.name
 
     def visit__to_copy(self, node: Node):
         dtype = node.kwargs.get("dtype", None)

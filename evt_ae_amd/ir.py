@@ -259,7 +259,7 @@ class Slot:
     role: str            # 'load' | 'store'
     dtype: str           # key of DTYPE_CTYPES
     domain: str          # 'tile' | 'row' | 'col' : where it is accessed
-    kind: str            # loads: 'aux' | 'row' | 'col' | 'scalar'; stores: 'aux' | 'row' | 'col'
+    kind: str            # loads: 'aux' | 'row' | 'col' | 'scalar' | 'rand' (no storage: generated); stores: 'aux' | 'row' | 'col'
     strides: Strides
     shape: Tuple[int, ...] = ()
 
@@ -302,6 +302,7 @@ class EpilogueIR:
         self.reduces: Dict[str, Reduce] = {}
         self.stores: List[Store] = []
         self.scalars: List[float] = []
+        self.rng_scalar: Optional[int] = None    # first of the four scalars that carry the rand_like seed / offset
         self._imm_count = 0
 
     # -- construction -------------------------------------------------------
@@ -322,6 +323,18 @@ class EpilogueIR:
     def add_slot(self, slot: Slot) -> int:
         self.slots.append(slot)
         return len(self.slots) - 1
+
+    def add_rand(self, name: str, strides: Strides, shape: Tuple[int, ...]) -> str:
+        """Uniform [0, 1) numbers shaped like a tensor of `shape` (rand_like): a
+        load slot without storage whose strides give the element index that
+        seeds the generator.  The seed and the per-call offset travel as four
+        run-time scalars (32-bit patterns), reserved once per module."""
+        if self.rng_scalar is None:
+            self.rng_scalar = len(self.scalars)
+            self.scalars += [0.0, 0.0, 0.0, 0.0]
+        k = self.add_slot(Slot(name, "load", "f32", "tile", "rand", strides, tuple(shape)))
+        self.add_node(Node(name, "load", domain="tile", slot=k))
+        return name
 
     def domain_of(self, names: Sequence[str]) -> str:
         """Join of operand domains.
@@ -451,6 +464,7 @@ class EpilogueIR:
             "slots": [[s.name, s.role, s.dtype, s.domain, s.kind] for s in self.slots],
             "reduces": [[r.name, r.kind, r.axis, r.input, r.state_offset] for r in self.reduces.values()],
             "stores": [[s.slot, s.input, s.domain] for s in self.stores],
+            "rng_scalar": self.rng_scalar,
         }
 
     def key(self) -> str:

@@ -31,7 +31,7 @@ FUSIBLE_TGT = {
     "reciprocal", "gelu", "tanh", "relu", "sigmoid", "tanh_backward", "gelu_backward", "ge", "gt", "le", "lt",
     "ne", "eq", "where", "_to_copy", "to", "one_hot", "gather", "sum", "amax", "mean", "logsumexp", "var_mean",
     "getitem", "view", "_unsafe_view", "reshape", "unsqueeze", "squeeze", "permute", "clone", "expand",
-    "detach", "alias", "contiguous",
+    "detach", "alias", "contiguous", "rand_like",
 }
 _SMALL_SIDE = FUSIBLE_TGT - {"sum", "amax", "mean", "logsumexp", "var_mean", "gather", "one_hot", "getitem"}
 

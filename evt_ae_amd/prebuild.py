@@ -49,6 +49,8 @@ def register_all() -> List[jit.LazyModule]:
             if shapes is None:   # the benchmark's --clock-probe builds of the headline kernels
                 op = W.fused_nodes(gm)[0].target
                 jit.load_module(op.ir, op.spec, clock_probe=True)
+    for name, (cls, _) in W.RANDOM_PATTERNS.items():
+        W.fuse(cls(), _meta(W.pattern_inputs(name)))
     from .autotuner.tuner_base import force_tile
     for tile in W.pipeline_tiles():
         with force_tile(tile):

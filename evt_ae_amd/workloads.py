@@ -385,6 +385,45 @@ def _h(g, shape, scale=1.0):
     return _randn(g, shape, scale)
 
 
+class MMPartition12(torch.nn.Module):
+    """unittest/evt_fuser/mm.py:216-236: relu, its `ne` mask, and a dropout
+    (rand_like / ge / mul) whose mask is returned too."""
+    def forward(self, primals_7, cat, primals_8):
+        permute_11 = aten.permute(primals_7, [1, 0])
+        mm_4 = aten.mm(cat, permute_11)
+        add = aten.add(mm_4, primals_8)
+        relu_3 = aten.relu(add)
+        ne = aten.ne(relu_3, 0)
+        rand_like = torch.rand_like(relu_3)
+        ge = aten.ge(rand_like, 1e-19)
+        mul_1 = aten.mul(relu_3, ge)
+        mul_2 = aten.mul(mul_1, 1.0)
+        return ne, ge, mul_2
+
+
+class Dropout1(torch.nn.Module):
+    """unittest/evt_fuser/dropout.py:33-46 after the reference's decomposition of
+    native_dropout(x, 0.7, True) into ge(rand_like(x), p), two muls
+    (pass_decomposition.py:359-369)."""
+    def forward(self, view_9, primals_16, primals_17, permute_104):
+        permute_115 = aten.permute(primals_16, [1, 0])
+        mm_36 = aten.mm(view_9, permute_115)
+        add_20 = aten.add(mm_36, primals_17)
+        view_10 = aten.view(add_20, [512, 2, 1024])
+        mask = aten.ge(torch.rand_like(view_10), 0.7)
+        output = aten.mul(view_10, mask)
+        scaled_output = aten.mul(output, 1. / (1 - 0.7))
+        add_4 = aten.add(scaled_output, permute_104)
+        return add_4, mask
+
+
+# patterns that draw random numbers in the epilogue: checked with the generator's stream replayed on the CPU
+RANDOM_PATTERNS = {
+    "mm12": (MMPartition12, lambda g: [_h(g, (512, 24576), 0.01), _h(g, (1024, 24576)), _h(g, (512,))]),
+    "dropout1": (Dropout1, lambda g: [_h(g, (1024, 1024)), _h(g, (1024, 1024), 0.03), _h(g, (1024,)),
+                                      _h(g, (512, 2, 1024))]),
+}
+
 # name -> (module class, input generator(generator) -> CPU tensors, allclose criteria of the reference test)
 REFERENCE_PATTERNS = {
     "mm1": (MMPartition1, lambda g: [_h(g, (4096, 1024), 0.03), _h(g, (1024, 1024)), _h(g, (4096,))]),
@@ -407,4 +446,4 @@ REFERENCE_PATTERNS = {
 
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
-    return REFERENCE_PATTERNS[name][1](g)
+    return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS[name])[1](g)

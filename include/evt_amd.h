@@ -46,7 +46,13 @@ extern "C" {
  * A broadcast dimension has stride 0.  Replaces the (M, N, L)-strided
  * tensor arguments of VisitorAuxLoad / VisitorRowBroadcast / VisitorRowStore
  * (src/cuda/epilogue/threadblock/visitor_load.hpp:364-571,
- *  visitor_store.hpp:46-145). */
+ *  visitor_store.hpp:46-145).
+ * A slot the module spec lists with kind "rand" (rand_like) has no storage:
+ * `ptr` is ignored and the strides give the element index e that seeds the
+ * generator -- the value is word (e & 3) of Philox4x32-10(counter = (e >> 2
+ * as two words, offset, slot index), key = seed), mapped to [0, 1) as
+ * (word >> 8) * 2^-24.  Takes the place of VisitorRand's {seed, offset}
+ * arguments (visitor_load.hpp:79-151). */
 typedef struct EvtTensorArg {
   void* ptr;
   int64_t stride_l;
@@ -72,6 +78,9 @@ typedef struct EvtArgs {
   int32_t num_tensors;
   int32_t num_scalars;
   EvtTensorArg tensors[EVT_MAX_TENSORS];
+  /* immediates of the epilogue, in module-spec order.  A module with a "rand"
+   * slot reads four of them as 32-bit patterns, not as float values:
+   * scalars[rng_scalars + 0..2] = seed low word, seed high word, offset. */
   float scalars[EVT_MAX_SCALARS];
 } EvtArgs;
 

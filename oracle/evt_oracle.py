@@ -33,6 +33,7 @@ fork's ActivationOp.Gelu / DGelu denote -- this oracle follows the graph's
 """
 from __future__ import annotations
 
+import contextlib
 import math
 from typing import Dict, List, Sequence, Tuple
 
@@ -54,9 +55,28 @@ def widen(t):
     return t
 
 
-def eval_fp32(module: torch.nn.Module, inputs: Sequence[torch.Tensor]) -> List[torch.Tensor]:
-    """Eager fp32 evaluation on CPU of `module` on the (already fp16-rounded) inputs."""
-    with torch.no_grad():
+@contextlib.contextmanager
+def philox_rand_like(seed: int, offset: int, salt: int):
+    """Inside the block `torch.rand_like(x)` returns the numbers the fused kernels
+    generate for a rand_like tensor shaped like x (oracle/philox.py) under the
+    given (seed, offset) and slot salt, instead of drawing from torch's generator."""
+    from . import philox
+    orig = torch.rand_like
+
+    def replay(x, *a, **k):
+        u = philox.uniform(seed, offset, salt, x.numel())
+        return torch.from_numpy(u).view(x.shape).to(dtype=torch.float32)
+    torch.rand_like = replay
+    try:
+        yield
+    finally:
+        torch.rand_like = orig
+
+
+def eval_fp32(module: torch.nn.Module, inputs: Sequence[torch.Tensor], rand=None) -> List[torch.Tensor]:
+    """Eager fp32 evaluation on CPU of `module` on the (already fp16-rounded) inputs.
+    rand = (seed, offset, salt): replay the kernels' random stream for rand_like."""
+    with torch.no_grad(), (philox_rand_like(*rand) if rand is not None else contextlib.nullcontext()):
         out = module(*[widen(t.cpu() if isinstance(t, torch.Tensor) else t) for t in inputs])
     if isinstance(out, torch.Tensor):
         out = [out]

@@ -8,7 +8,7 @@ import torch
 from evt_ae_amd import workloads as W
 from evt_ae_amd.evt_fuser import EVTFuser, FusedBMM, FusedGEMM
 from oracle import evt_oracle
-from tests.util import fused_nodes, run_emulated
+from tests.util import fused_nodes, rand_slot, run_emulated
 
 
 def _check(module_cls, inputs, n_fused=1, tol=2e-5):
@@ -96,6 +96,39 @@ def test_reference_patterns_shrunk():
     (n,) = fused_nodes(gm)
     # add_19 and its view share one store (the reference's output2store aliasing)
     assert len({v for v in n.target.output2store.values()}) == 3
+
+
+def test_random_patterns_lower_correctly():
+    """rand_like in the epilogue (unittest/evt_fuser/mm.py:216-236 at reduced K,
+    dropout.py:33-46 decomposed): the IR draws from the element-indexed Philox
+    stream; with that stream replayed in the eager module every output matches,
+    masks bit for bit, and successive calls draw different numbers."""
+    g = torch.Generator().manual_seed(5)
+    h = lambda *s: (torch.randn(*s, generator=g) * 0.5).half()   # noqa: E731
+    for cls, inputs in ((W.MMPartition12, [h(512, 64), h(1024, 64), h(512)]),
+                        (W.Dropout1, [h(1024, 32), h(1024, 32), h(1024), h(512, 2, 1024)])):
+        gm = W.fuse(cls(), inputs)
+        (n,) = fused_nodes(gm)
+        op = n.target
+        op.rand_seed = 0x1234_5678_9ABC
+        masks = []
+        for call in range(2):
+            got = run_emulated(gm, inputs)
+            seed, offset = op.last_rand_state
+            assert (seed, offset) == (0x1234_5678_9ABC, call)
+            ref = evt_oracle.eval_fp32(cls(), inputs, rand=(seed, offset, rand_slot(op)))
+            assert len(got) == len(ref)
+            for o, r in zip(got, ref):
+                assert tuple(o.shape) == tuple(r.shape)
+                if r.dtype == torch.bool:
+                    assert torch.equal(o.bool(), r)
+                else:
+                    assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3
+            masks.append([o for o in got if o.dtype == torch.bool][-1])
+        if cls is W.Dropout1:     # (mm12 keeps with probability 1 - 1e-19: its mask is all ones)
+            assert not torch.equal(masks[0], masks[1])
+    keep = masks[0].float().mean().item()      # Dropout1: p = 0.7 dropped
+    assert abs(keep - 0.3) < 5e-3
 
 
 def test_unsupported_ops_raise():

@@ -173,3 +173,26 @@ def test_golden_fixtures_match_oracle():
             g = gold[f"c{cfg}_out{i}"]
             assert O.max_rel_err(o.numpy(), g) <= 1e-6
             assert O.max_rel_err(g.reshape(c.shape), c) <= 2e-4
+
+
+def test_philox_known_answers():
+    """Philox4x32-10 against the known-answer vectors of the Random123
+    distribution (kat_vectors: philox4x32 10), and the [0, 1) mapping."""
+    import numpy as np
+    from oracle import philox
+    kat = [([0, 0, 0, 0], (0, 0), [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+           ([0xffffffff] * 4, (0xffffffff, 0xffffffff), [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+           ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], (0xa4093822, 0x299f31d0),
+            [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1])]
+    for ctr, key, want in kat:
+        got = philox.philox4x32_10(np.array([ctr], dtype=np.uint32), key)[0]
+        assert [int(x) for x in got] == want
+    u = philox.uniform(seed=7, offset=3, salt=1, numel=1 << 18)
+    assert u.dtype == np.float32 and u.min() >= 0.0 and u.max() < 1.0
+    assert abs(float(u.mean()) - 0.5) < 3e-3 and abs(float((u >= 0.7).mean()) - 0.3) < 3e-3
+    # element e is word e & 3 of the block with counter (e >> 2, 0, offset, salt) under key = seed
+    blk = philox.philox4x32_10(np.array([[5, 0, 3, 1]], dtype=np.uint32), (7, 0))[0]
+    assert np.array_equal(u[20:24], (blk >> np.uint32(8)).astype(np.float32) * np.float32(2.0 ** -24))
+    # a different offset or salt is a different stream
+    assert not np.array_equal(u, philox.uniform(7, 4, 1, 1 << 18))
+    assert not np.array_equal(u, philox.uniform(7, 3, 2, 1 << 18))

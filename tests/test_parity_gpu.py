@@ -12,7 +12,7 @@ import torch
 from evt_ae_amd import workloads as W
 from evt_ae_amd.autotuner.tuner_base import force_tile
 from oracle import evt_oracle
-from tests.util import fused_nodes
+from tests.util import fused_nodes, rand_slot
 
 pytestmark = pytest.mark.gpu
 
@@ -131,6 +131,41 @@ def test_reference_fuser_patterns(name):
         is_sum = o.dim() >= 1 and o.numel() < r.numel() + 1 and o.shape != refs[0].shape
         err = evt_oracle.max_rel_err(o, r)
         assert err <= FP16_TOL, f"{name}: max rel err {err:.3e}"
+
+
+@pytest.mark.parametrize("name", ["mm12", "dropout1"])
+def test_random_fuser_patterns(name):
+    """rand_like fused into the epilogue (unittest/evt_fuser/mm.py:216-236,
+    dropout.py:33-75).  The reference can only check the keep rate; here the
+    generator's stream is replayed on the CPU (oracle/philox.py), so the masks
+    must match bit for bit and the values to the fp16 tolerance, and two
+    launches must draw different numbers."""
+    cls, _ = W.RANDOM_PATTERNS[name]
+    inputs = W.pattern_inputs(name)
+    dev = [t.cuda() for t in inputs]
+    gm = W.fuse(cls(), inputs)
+    (node,) = fused_nodes(gm)
+    op = node.target
+    op.rand_seed = 0xC0FFEE_0000_0001
+    masks = []
+    for call in range(2):
+        outs = list(gm(*dev))
+        torch.cuda.synchronize()
+        seed, offset = op.last_rand_state
+        assert offset == call
+        refs = evt_oracle.eval_fp32(cls(), inputs, rand=(seed, offset, rand_slot(op)))
+        assert len(outs) == len(refs)
+        for o, r in zip(outs, refs):
+            assert tuple(o.shape) == tuple(r.shape)
+            if r.dtype == torch.bool:
+                assert o.dtype == torch.bool and torch.equal(o.cpu(), r)
+            else:
+                assert evt_oracle.max_rel_err(o, r) <= FP16_TOL
+        masks.append(outs[1].cpu())
+    if name == "dropout1":
+        assert not torch.equal(masks[0], masks[1])
+        keep = masks[0].float().mean().item()          # the reference's criterion (dropout.py:73-75)
+        assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
 
 
 def test_golden_fixtures():

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from evt_ae_amd.evt_fuser import FusedBMM, FusedGEMM, FusedOpBase
-from oracle import ir_interp
+from oracle import ir_interp, philox
 
 aten = torch.ops.aten
 
@@ -28,6 +28,14 @@ def emulate_fused(op: FusedOpBase, *args):
         kind, ref = op.slot_sources[k]
         if kind == "input":
             loads[k] = args[ref]
+        elif kind == "rand":   # the numbers the kernel generates for this launch
+            numel = 1
+            for d in slot.shape:
+                numel *= d
+            loads[k] = torch.from_numpy(philox.uniform(op.rand_seed, op.rand_offset, k, numel))
+    if op.ir.rng_scalar is not None:
+        op.last_rand_state = (op.rand_seed, op.rand_offset & 0xFFFFFFFF)
+        op.rand_offset += 1
     stored = ir_interp.interpret(op.ir, acc, loads)
     visitor = {}
     for k, slot in enumerate(op.ir.slots):
@@ -66,3 +74,9 @@ def run_emulated(gm, inputs):
         for op, _ in patched:
             op.__class__ = op.__class__.__mro__[1]
     return list(out) if isinstance(out, (tuple, list)) else [out]
+
+
+def rand_slot(op: FusedOpBase) -> int:
+    """Index (= generator salt) of the op's single rand_like slot."""
+    (k,) = [k for k, s in enumerate(op.ir.slots) if s.kind == "rand"]
+    return k
