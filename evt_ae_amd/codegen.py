@@ -260,25 +260,41 @@ class Codegen:
             e.dedent()
             e("}")
         aux_nodes = [n for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "aux"]
+        # rows are processed in batches of MB x 16: the full-tensor loads of a batch are all issued before its
+        # arithmetic and stores (loads do not move above stores by themselves), so a batch costs one round trip
+        # to HBM; two 32-row blocks per batch keep the staging registers bounded on the largest wave tiles
+        e("constexpr int MB = MI >= 2 ? 2 : 1;")
+        e('static_assert(MI % MB == 0, "row blocks per wave must be 1 or even");')
         e("#pragma unroll")
-        e("for (int mi = 0; mi < MI; ++mi) {")
+        e("for (int mb = 0; mb < MI; mb += MB) {")
         e.indent()
         if aux_nodes:
-            e("// issue the full-tensor loads of these 16 rows before any arithmetic or store")
             for name in aux_nodes:
                 k = ir.nodes[name].slot
-                e(f"{DTYPE_CTYPES[ir.slots[k].dtype]} r_{_cname(name)}[16][NI];")
+                e(f"{DTYPE_CTYPES[ir.slots[k].dtype]} rb_{_cname(name)}[MB][16][NI];")
+            e("#pragma unroll")
+            e("for (int mo = 0; mo < MB; ++mo) {")
+            e.indent()
             e("#pragma unroll")
             e("for (int v = 0; v < 16; ++v) {")
             e.indent()
-            e("const int row = t.row(mi, v);")
+            e("const int row = t.row(mb + mo, v);")
             e("const bool rok = t.row_ok(row);")
             for name in aux_nodes:
                 k = ir.nodes[name].slot
                 e(f"evt::aux_load<FAST>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
-                  f"p.t{k}_sn, p.t{k}_vec, rok, r_{_cname(name)}[v]);")
+                  f"p.t{k}_sn, p.t{k}_vec, rok, rb_{_cname(name)}[mo][v]);")
             e.dedent()
             e("}")
+            e.dedent()
+            e("}")
+        e("#pragma unroll")
+        e("for (int mo = 0; mo < MB; ++mo) {")
+        e.indent()
+        e("const int mi = mb + mo;")
+        for name in aux_nodes:
+            k = ir.nodes[name].slot
+            e(f"const {DTYPE_CTYPES[ir.slots[k].dtype]} (&r_{_cname(name)})[16][NI] = rb_{_cname(name)}[mo];")
         e("#pragma unroll")
         e("for (int v = 0; v < 16; ++v) {")
         e.indent()
@@ -314,6 +330,8 @@ class Codegen:
                 e(f"cst[ni][{o}] = (rok && t.col_ok(ni)) ? fmaxf(cst[ni][{o}], {x()}) : cst[ni][{o}];")
             e.dedent()
             e("}")
+        e.dedent()
+        e("}")
         e.dedent()
         e("}")
         e.dedent()
