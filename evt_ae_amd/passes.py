@@ -145,3 +145,95 @@ class Partitioning:
 
 def pass_fusion(module: GraphModule, graph: Graph = None):
     return Partitioning()(module)
+
+
+# ---------------------------------------------------------------------------
+# pass_decomposition: the rewrites in front of the fuser that the fused
+# GEMM/BMM path depends on
+# ---------------------------------------------------------------------------
+
+def _repropagate(module: GraphModule) -> None:
+    """Refresh tensor_meta after a rewrite by running the graph on meta tensors
+    shaped like the placeholders (no data, no device)."""
+    from torch.fx.passes.shape_prop import ShapeProp
+    metas = []
+    for n in module.graph.nodes:
+        if n.op == "placeholder":
+            tm = n.meta.get("tensor_meta")
+            if tm is None:
+                return      # no shapes recorded: the caller runs ShapeProp itself
+            metas.append(torch.empty(tuple(tm.shape), dtype=tm.dtype, device="meta"))
+    ShapeProp(module).propagate(*metas)
+
+
+def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: Sequence[str] = ()):
+    """The subset of the reference's Decomposition pass
+    (python/gtl/compiler/passes/pass_decomposition.py:192-502, entry :817) that
+    the fused GEMM/BMM path needs, with the same replacements:
+
+      addmm(b, x, w)                 -> add(mm(x, w), b)                         (:414-426)
+      t(x) / transpose(x, i, j)      -> permute(x, dims)                         (:448-502)
+      _unsafe_view(x, s)             -> view(x, s)                               (:463-475)
+      rsub(x, y)                     -> sub(y, x)                                (:280-292)
+      native_dropout(x, p, True)     -> mask = ge(rand_like(x), p);
+                                        (mul(mul(x, mask), 1/(1-p)), mask)       (:350-379)
+      native_dropout_backward(g,m,s) -> mul(mul(g, m), s)                        (:381-395)
+      threshold_backward(g, y, t)    -> mul(g, gt(y, t))                         (:397-412; the reference
+                                        writes ne(y, t), equal on ReLU outputs only)
+
+    The reference's other decompositions (log_softmax, nll_loss, layer / batch
+    norm, convolution, pooling) belong to anchors this backend does not provide
+    and are left untouched."""
+    graph = module.graph if graph is None else graph
+    disabled = set(disabled_ops)
+    changed = False
+    for node in list(graph.nodes):
+        if node.op != "call_function":
+            continue
+        name = target_name(node.target)
+        if name in disabled:
+            continue
+        new = None
+        with graph.inserting_before(node):
+            if name == "addmm" and len(node.args) == 3 and not node.kwargs:
+                b, x, w = node.args
+                new = graph.call_function(aten.add, (graph.call_function(aten.mm, (x, w)), b))
+            elif name == "t":
+                new = graph.call_function(aten.permute, (node.args[0], [1, 0]))
+            elif name == "transpose" and len(node.args) == 3:
+                rank = len(node.meta["tensor_meta"].shape)
+                dims = list(range(rank))
+                i, j = node.args[1] % rank, node.args[2] % rank
+                dims[i], dims[j] = j, i
+                new = graph.call_function(aten.permute, (node.args[0], dims))
+            elif name == "_unsafe_view":
+                new = graph.call_function(aten.view, tuple(node.args))
+            elif name == "rsub" and len(node.args) == 2 and node.kwargs.get("alpha", 1) == 1:
+                new = graph.call_function(aten.sub, (node.args[1], node.args[0]))
+            elif name == "native_dropout_backward":
+                g, m, s = node.args
+                new = graph.call_function(aten.mul, (graph.call_function(aten.mul, (g, m)), s))
+            elif name == "threshold_backward":
+                g, y, t = node.args
+                new = graph.call_function(aten.mul, (g, graph.call_function(aten.gt, (y, t))))
+            elif name == "native_dropout" and len(node.args) == 3 and node.args[2] is True:
+                x, p = node.args[0], node.args[1]
+                mask = graph.call_function(aten.ge, (graph.call_function(torch.rand_like, (x,)), p))
+                out = graph.call_function(aten.mul, (graph.call_function(aten.mul, (x, mask)), 1. / (1 - p)))
+                for user in list(node.users):     # getitem(dropout, 0 | 1)
+                    if user.op == "call_function" and user.target is operator.getitem:
+                        user.replace_all_uses_with(out if user.args[1] == 0 else mask)
+                        graph.erase_node(user)
+                if not node.users:
+                    graph.erase_node(node)
+                    changed = True
+                continue
+        if new is not None:
+            node.replace_all_uses_with(new)
+            graph.erase_node(node)
+            changed = True
+    if changed:
+        graph.lint()
+        module.recompile()
+        _repropagate(module)
+    return module

@@ -51,6 +51,8 @@ def register_all() -> List[jit.LazyModule]:
                 jit.load_module(op.ir, op.spec, clock_probe=True)
     for name, (cls, _) in W.RANDOM_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    from .passes import pass_decomposition, pass_fusion
+    W.fuse(W.Dropout1Undecomposed(), _meta(W.pattern_inputs("dropout1")), passes=[pass_decomposition, pass_fusion])
     from .autotuner.tuner_base import force_tile
     for tile in W.pipeline_tiles():
         with force_tile(tile):

@@ -417,6 +417,21 @@ class Dropout1(torch.nn.Module):
         return add_4, mask
 
 
+class Dropout1Undecomposed(torch.nn.Module):
+    """unittest/evt_fuser/dropout.py:33-46 verbatim: native_dropout, decomposed by
+    pass_decomposition before pass_fusion as in the reference's test."""
+    def forward(self, view_9, primals_16, primals_17, permute_104):
+        permute_115 = aten.permute(primals_16, [1, 0])
+        mm_36 = aten.mm(view_9, permute_115)
+        add_20 = aten.add(mm_36, primals_17)
+        view_10 = aten.view(add_20, [512, 2, 1024])
+        dropout = aten.native_dropout(view_10, 0.7, True)
+        getitem_2 = operator.getitem(dropout, 0)
+        getitem_3 = operator.getitem(dropout, 1)
+        add_4 = aten.add(getitem_2, permute_104)
+        return add_4, getitem_3
+
+
 # patterns that draw random numbers in the epilogue: checked with the generator's stream replayed on the CPU
 RANDOM_PATTERNS = {
     "mm12": (MMPartition12, lambda g: [_h(g, (512, 24576), 0.01), _h(g, (1024, 24576)), _h(g, (512,))]),

@@ -131,6 +131,43 @@ def test_random_patterns_lower_correctly():
     assert abs(keep - 0.3) < 5e-3
 
 
+def test_pass_decomposition_rewrites():
+    """The reference's Decomposition replacements this path depends on
+    (pass_decomposition.py:280-502): same values after the rewrite, the targeted
+    ops gone, and the reference's dropout test graph (native_dropout,
+    dropout.py:33-46) becomes one fused kernel that returns the mask."""
+    from evt_ae_amd.passes import pass_decomposition, pass_fusion
+
+    class Mixed(torch.nn.Module):
+        def forward(self, b, x, w, g):
+            y = torch.ops.aten.addmm(b, x, torch.ops.aten.t(w))
+            y = torch.ops.aten._unsafe_view(y, [4, 8, 24])
+            y = torch.ops.aten.transpose(y, 0, 1)
+            r = torch.ops.aten.rsub(y, 1.0)
+            tb = torch.ops.aten.threshold_backward(g, r, 0.5)
+            return torch.ops.aten.native_dropout_backward(tb, tb > 0, 2.0)
+    gen = torch.Generator().manual_seed(11)
+    b, x, w = torch.randn(24, generator=gen), torch.randn(32, 16, generator=gen), torch.randn(24, 16, generator=gen)
+    g = torch.randn(8, 4, 24, generator=gen)
+    gm = W.trace_module(Mixed(), [b, x, w, g])
+    want = Mixed()(b, x, w, g)
+    pass_decomposition(gm, gm.graph)
+    from evt_ae_amd.evt_fuser import target_name
+    names = {target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"}
+    assert not names & {"addmm", "t", "transpose", "_unsafe_view", "rsub", "threshold_backward",
+                        "native_dropout_backward"}
+    assert {"mm", "permute", "view", "sub", "gt", "mul"} <= names
+    assert torch.allclose(gm(b, x, w, g), want, atol=1e-5)
+    assert all("tensor_meta" in n.meta for n in gm.graph.nodes if n.op == "call_function")
+
+    inputs = W.pattern_inputs("dropout1")
+    gm = W.fuse(W.Dropout1Undecomposed(), inputs, passes=[pass_decomposition, pass_fusion])
+    (n,) = fused_nodes(gm)
+    assert not any(target_name(x.target) == "native_dropout" for x in gm.graph.nodes if x.op == "call_function")
+    assert any(s.kind == "rand" for s in n.target.ir.slots)
+    assert [tuple(v[0]) for v in n.target.store_meta.values()] and len(n.target.outputs) == 2
+
+
 def test_unsupported_ops_raise():
     class Bad(torch.nn.Module):
         def forward(self, a, b):

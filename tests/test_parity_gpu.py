@@ -133,6 +133,27 @@ def test_reference_fuser_patterns(name):
         assert err <= FP16_TOL, f"{name}: max rel err {err:.3e}"
 
 
+def test_reference_dropout_test_verbatim():
+    """unittest/evt_fuser/dropout.py:33-75 as written there: native_dropout in the
+    module, pass_decomposition + pass_fusion, reference recomputed from the
+    returned mask, the reference's tolerances and keep-rate window."""
+    from evt_ae_amd.passes import pass_decomposition, pass_fusion
+    inputs = [t.cuda() for t in W.pattern_inputs("dropout1")]
+    view_9, primals_16, primals_17, permute_104 = inputs
+    gm = W.fuse(W.Dropout1Undecomposed(), inputs, passes=[pass_decomposition, pass_fusion])
+    assert len(fused_nodes(gm)) == 1
+    out, mask = gm(*inputs)
+    mm_36 = torch.mm(view_9, primals_16.permute(1, 0))
+    view_10 = (mm_36 + primals_17).view(512, 2, 1024)
+    ref = view_10 * mask / 0.3 + permute_104
+    assert torch.allclose(out, ref, atol=5e-1)        # the reference's check, against fp16 eager
+    ref32 = ((view_9.float() @ primals_16.float().t() + primals_17.float()).view(512, 2, 1024)
+             * mask / (1 - 0.7) + permute_104.float())
+    assert evt_oracle.max_rel_err(out, ref32) <= FP16_TOL
+    keep = torch.mean(mask.to(torch.float32)).item()
+    assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
+
+
 @pytest.mark.parametrize("name", ["mm12", "dropout1"])
 def test_random_fuser_patterns(name):
     """rand_like fused into the epilogue (unittest/evt_fuser/mm.py:216-236,
