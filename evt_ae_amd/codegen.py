@@ -260,6 +260,26 @@ class Codegen:
             e.dedent()
             e("}")
         aux_nodes = [n for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "aux"]
+        # check-free path: wave-uniform row base (scalar registers) + one per-lane offset per tensor
+        for k in [ir.nodes[n].slot for n in aux_nodes] + [s_.slot for s_ in tile_stores]:
+            ct = DTYPE_CTYPES[ir.slots[k].dtype]
+            cq = "const " if ir.slots[k].role == "load" else ""
+            e(f"[[maybe_unused]] {cq}{ct}* ub_{k} = nullptr;")
+            e(f"[[maybe_unused]] uint32_t lo_{k} = 0;")
+            e("if constexpr (FAST) {")
+            e(f"  ub_{k} = p.t{k} + {self.slot_off(k)} + (int64_t)t.row_u * p.t{k}_sm + t.col_u;")
+            e(f"  lo_{k} = (uint32_t)(t.row_l * (int)p.t{k}_sm + t.col_l);")
+            e("}")
+        # With a cross-workgroup reduction in the same epilogue, the arrival ticket has to wait until this wave's
+        # earlier stores are acknowledged; the output-tile values of a small wave tile are therefore kept in
+        # registers and stored after the ticket instead of in front of it.
+        defer = bool(tile_stores) and bool(row_reds or col_reds)
+        e(f"constexpr bool DEFER = {'true' if defer else 'false'} && MI * NI <= 4;")
+        for s_ in tile_stores:
+            e(f"[[maybe_unused]] float sv_{s_.slot}[DEFER ? MI : 1][16][NI];")
+        if any(r.kind == "welford" for r in row_reds):
+            e("const float wcnt = (float)t.wave_cols();")
+            e("const float wrcnt = wcnt > 0.f ? 1.f / wcnt : 0.f;")
         # rows are processed in batches of MB x 16: the full-tensor loads of a batch are all issued before its
         # arithmetic and stores (loads do not move above stores by themselves), so a batch costs one round trip
         # to HBM; two 32-row blocks per batch keep the staging registers bounded on the largest wave tiles
@@ -282,7 +302,9 @@ class Codegen:
             e("const bool rok = t.row_ok(row);")
             for name in aux_nodes:
                 k = ir.nodes[name].slot
-                e(f"evt::aux_load<FAST>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
+                e(f"if constexpr (FAST) evt::row_load<Tile>(ub_{k} + (int64_t)Tile::row_step(mb + mo, v) * p.t{k}_sm, lo_{k}, "
+                  f"rb_{_cname(name)}[mo][v]);")
+                e(f"else evt::aux_load<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
                   f"p.t{k}_sn, p.t{k}_vec, rok, rb_{_cname(name)}[mo][v]);")
             e.dedent()
             e("}")
@@ -311,8 +333,13 @@ class Codegen:
                 arr = f"b_{k}"
             else:
                 arr = _cname(src)
-            e(f"evt::aux_store<FAST>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
-              f"p.t{k}_sn, p.t{k}_vec, rok, {arr});")
+            e("if constexpr (DEFER) {")
+            e(f"  #pragma unroll\n  for (int ni = 0; ni < NI; ++ni) sv_{k}[mi][v][ni] = {arr}[ni];")
+            e("} else {")
+            e.indent()
+            self.emit_tile_store(e, k, arr)
+            e.dedent()
+            e("}")
         if row_reds:
             e(f"float rst[{ir.row_state}];")
             for r in row_reds:
@@ -337,12 +364,42 @@ class Codegen:
         e.dedent()
         e("}")
         if row_reds:
-            e("evt::row_reduce_finish<Cfg, Epi>(p, t, g);")
+            e("const bool row_last = evt::row_reduce_publish<Cfg, Epi>(p, t, g);")
         if col_reds:
-            e("evt::col_reduce_finish<Cfg, Epi>(p, t, g, cst);")
+            e("const bool col_last = evt::col_reduce_publish<Cfg, Epi>(p, t, g, cst);")
+        if defer:
+            e("if constexpr (DEFER) {")
+            e.indent()
+            e("#pragma unroll")
+            e("for (int mi = 0; mi < MI; ++mi) {")
+            e.indent()
+            e("#pragma unroll")
+            e("for (int v = 0; v < 16; ++v) {")
+            e.indent()
+            e("const int row = t.row(mi, v);")
+            e("const bool rok = t.row_ok(row);")
+            for s_ in tile_stores:
+                self.emit_tile_store(e, s_.slot, f"sv_{s_.slot}[mi][v]")
+            e("(void)row; (void)rok;")
+            e.dedent()
+            e("}")
+            e.dedent()
+            e("}")
+            e.dedent()
+            e("}")
+        if row_reds:
+            e("if (row_last) evt::row_reduce_complete<Cfg, Epi>(p, t, g);")
+        if col_reds:
+            e("if (col_last) evt::col_reduce_complete<Cfg, Epi>(p, t, g);")
         e("(void)p; (void)t; (void)g; (void)acc;")
         e.dedent()
         e("}")
+
+    def emit_tile_store(self, e: _Emitter, k: int, arr: str):
+        """Store the NI values `arr` of row (mi, v) to tile slot k (inside the row loops)."""
+        e(f"if constexpr (FAST) evt::row_store<Tile>(ub_{k} + (int64_t)Tile::row_step(mi, v) * p.t{k}_sm, lo_{k}, {arr});")
+        e(f"else evt::aux_store<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
+          f"p.t{k}_sn, p.t{k}_vec, rok, {arr});")
 
     def emit_node(self, e: _Emitter, n: Node, hoisted: bool):
         c = _cname(n.name)
@@ -414,11 +471,11 @@ class Codegen:
             e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) se += t.col_ok(ni) ? evt::op_exp({x} - mx) : 0.f;")
             e(f"rst[{o}] = mx; rst[{o + 1}] = evt::half_wave_sum(se);")
         elif r.kind == "welford":
-            e("const float cnt = (float)t.wave_cols();")
+            e("const float cnt = wcnt;")
             e("float sx = 0.f;")
             e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) sx += t.col_ok(ni) ? {x} : 0.f;")
             e("sx = evt::half_wave_sum(sx);")
-            e("const float mean = cnt > 0.f ? sx / cnt : 0.f;")
+            e("const float mean = sx * wrcnt;")
             e("float sq = 0.f;")
             e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {{ const float d = {x} - mean; sq += t.col_ok(ni) ? d * d : 0.f; }}")
             e(f"rst[{o}] = cnt; rst[{o + 1}] = mean; rst[{o + 2}] = evt::half_wave_sum(sq);")
@@ -538,6 +595,7 @@ class Codegen:
                       if (sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux")]
         cond = " && ".join(
             [f"(p.t{k}_vec & 1) && (!(Cfg::INTERLEAVE && sizeof(*p.t{k}) == 2 && (Cfg::NI == 2 || Cfg::NI == 4)) || (p.t{k}_vec & 2))"
+             f" && p.t{k}_sm >= 0 && p.t{k}_sm < (1 << 28)"
              for k in tile_slots]) or "true"
         e(f"p.fast = ({cond}) ? 1 : 0;")
         e("return EVT_OK;")

@@ -91,6 +91,8 @@ struct TileCtx {
   int batch, tile_m, tile_n, tiles_m, tiles_n;
   int m0, n0;          // tile origin
   int row0, col0;      // this lane's first row / column
+  int row_u, col_u;    // their wave-uniform parts (scalar registers) ...
+  int row_l, col_l;    // ... and per-lane parts: row0 = row_u + row_l, col0 = col_u + col_l
   int tid, lane, wm, wn;
   char* smem;
   char* workspace;
@@ -100,13 +102,17 @@ struct TileCtx {
     batch = batch_; tile_m = tm; tile_n = tn; tiles_m = g.tiles_m; tiles_n = g.tiles_n;
     m0 = tm * Cfg::BM; n0 = tn * Cfg::BN;
     tid = threadIdx.x; lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     wm = wave / Cfg::WN; wn = wave % Cfg::WN;
-    row0 = m0 + wm * Cfg::TM + 4 * (lane >> 5);
-    col0 = n0 + wn * Cfg::TN + (INTERLEAVE ? (lane & 31) * NI : (lane & 31));
+    row_u = m0 + wm * Cfg::TM; row_l = 4 * (lane >> 5);
+    col_u = n0 + wn * Cfg::TN; col_l = INTERLEAVE ? (lane & 31) * NI : (lane & 31);
+    row0 = row_u + row_l;
+    col0 = col_u + col_l;
     smem = smem_; workspace = g.workspace;
   }
   EVT_DEV int row(int mi, int v) const { return row0 + mi * 32 + 8 * (v >> 2) + (v & 3); }
+  // row of register (mi, v) relative to row0: a compile-time constant once the loops are unrolled
+  static EVT_DEV int row_step(int mi, int v) { return mi * 32 + 8 * (v >> 2) + (v & 3); }
   EVT_DEV int col(int ni) const { return col0 + ni * COL_STEP; }
   EVT_DEV bool col_ok(int ni) const { return FULL || col(ni) < N; }
   EVT_DEV bool row_ok(int r) const { return FULL || r < M; }
@@ -193,6 +199,46 @@ EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, 
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
       if (rok && t.col_ok(ni)) st_f32<T>(rp, (int64_t)ni * Tile::COL_STEP * sn, val[ni]);
+  }
+}
+
+// Check-free access to one accumulator row of a unit-stride tensor: `rowp` is
+// wave-uniform (a scalar-register pointer the compiler advances with scalar
+// arithmetic), `lo` is this lane's element offset inside the row, computed once
+// per tile -- no per-row 64-bit vector address arithmetic.
+template <class Tile, class T>
+EVT_DEV void row_load(const T* rowp, uint32_t lo, T (&out)[Tile::NI]) {
+  constexpr int NI = Tile::NI;
+  const char* base = (const char*)rowp;
+  if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && NI == 4) {
+    const u32x2 raw = *(const u32x2*)(base + lo * 2u);
+    const T* e = (const T*)&raw;
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) out[ni] = e[ni];
+  } else if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && NI == 2) {
+    const uint32_t raw = *(const uint32_t*)(base + lo * 2u);
+    const T* e = (const T*)&raw;
+    out[0] = e[0]; out[1] = e[1];
+  } else {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) out[ni] = *(const T*)(base + (lo + (uint32_t)(ni * Tile::COL_STEP)) * (uint32_t)sizeof(T));
+  }
+}
+
+template <class Tile, class T>
+EVT_DEV void row_store(T* rowp, uint32_t lo, const float (&val)[Tile::NI]) {
+  constexpr int NI = Tile::NI;
+  char* base = (char*)rowp;
+  if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4)) {
+    T e[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) e[ni] = (T)val[ni];
+    if constexpr (NI == 4) *(u32x2*)(base + lo * 2u) = *(const u32x2*)e;
+    else *(uint32_t*)(base + lo * 2u) = *(const uint32_t*)e;
+  } else {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+      st_f32<T>((T*)(base + (lo + (uint32_t)(ni * Tile::COL_STEP)) * (uint32_t)sizeof(T)), 0, val[ni]);
   }
 }
 
@@ -340,8 +386,15 @@ EVT_DEV bool arrive_last(int* counter, int expected, int* smem_flag) {
 // tile order -- in the last workgroup of the row block to arrive (few tiles) or
 // in the finalize kernel (many tiles).
 //   LDS layout: state[wn][local_row][ROW_STATE] floats at smem, then one flag.
+// Phase 1 of a per-row reduction: combine the waves' row states in LDS and
+// either finalize (one tile spans the row) or publish this tile's partials.
+// Returns true when phase 2 runs in this kernel and this workgroup is the last
+// of its row block to arrive: it must then call row_reduce_complete.  Split in
+// two so the caller can issue its output-tile stores in between: the arrival
+// ticket has to wait for this wave's earlier stores to be acknowledged, and
+// 64 KB of tile stores in front of it cost microseconds.
 template <class Cfg, class Epi, class Tile>
-EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
+EVT_DEV bool row_reduce_publish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
   constexpr int RS = Epi::ROW_STATE;
   if constexpr (RS > 0) {
     const float* lds = (const float*)t.smem;
@@ -365,9 +418,22 @@ EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t, con
         for (int c = 0; c < RS; ++c) st_device(dst + c, st[c]);
       }
     }
-    if (t.tiles_n == 1 || !g.row_inkernel) return;
+    if (t.tiles_n == 1 || !g.row_inkernel) return false;
     int* counter = (int*)t.workspace + t.batch * t.tiles_m + t.tile_m;
-    if (!arrive_last(counter, t.tiles_n, flag)) return;
+    return arrive_last(counter, t.tiles_n, flag);
+  } else {
+    return false;
+  }
+}
+
+// Phase 2 in the last workgroup of a row block: fold the partials in tile order.
+template <class Cfg, class Epi, class Tile>
+EVT_DEV void row_reduce_complete(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
+  constexpr int RS = Epi::ROW_STATE;
+  if constexpr (RS > 0) {
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    const float* part = (const float*)(t.workspace + wl.counter_bytes);
+    int* counter = (int*)t.workspace + t.batch * t.tiles_m + t.tile_m;
     for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
       const int row = t.m0 + lr;
       if (row >= t.M) continue;
@@ -385,13 +451,14 @@ EVT_DEV void row_reduce_finish(const typename Epi::Params& p, const Tile& t, con
     }
     if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  (void)g;
 }
 
 // Per-column reductions.  `cs[ni][c]` holds this lane's state for column
 // col(ni) over all its rows.  LDS layout: state[wm][local_col][COL_STATE]
 // floats placed after the row-reduction area, then one flag.
 template <class Cfg, class Epi, class Tile>
-EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g,
+EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g,
                                float (&cs)[Tile::NI][Epi::COL_STATE > 0 ? Epi::COL_STATE : 1]) {
   constexpr int CS = Epi::COL_STATE;
   if constexpr (CS > 0) {
@@ -432,10 +499,27 @@ EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t, con
         for (int c = 0; c < CS; ++c) st_device(dst + c, st[c]);
       }
     }
-    if (t.tiles_m == 1 || !g.col_inkernel) return;
+    if (t.tiles_m == 1 || !g.col_inkernel) return false;
     const int row_counters = (Epi::ROW_STATE > 0 && t.tiles_n > 1) ? t.L * t.tiles_m : 0;
     int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
-    if (!arrive_last(counter, t.tiles_m, flag)) return;
+    return arrive_last(counter, t.tiles_m, flag);
+  } else {
+    return false;
+  }
+}
+
+// Phase 2 in the last workgroup of a column block.
+template <class Cfg, class Epi, class Tile>
+EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
+  constexpr int CS = Epi::COL_STATE;
+  if constexpr (CS > 0) {
+    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
+    constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
+    float* lds = (float*)(t.smem + ROW_AREA);
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    const float* part = (const float*)(t.workspace + wl.counter_bytes + wl.row_bytes);
+    const int row_counters = (Epi::ROW_STATE > 0 && t.tiles_n > 1) ? t.L * t.tiles_m : 0;
+    int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
     // SHARES threads per column each fold every SHARES-th partial in tile order
     // (independent loads in flight together), LDS then combines the shares in order
     const int lc = t.tid % Cfg::BN, share = t.tid / Cfg::BN;
@@ -465,6 +549,7 @@ EVT_DEV void col_reduce_finish(const typename Epi::Params& p, const Tile& t, con
     }
     if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  (void)g;
 }
 
 // Phase 2 of per-row reductions: 2^LG lanes share one row; each folds every

@@ -141,7 +141,9 @@ def test_reference_dropout_test_verbatim():
     inputs = [t.cuda() for t in W.pattern_inputs("dropout1")]
     view_9, primals_16, primals_17, permute_104 = inputs
     gm = W.fuse(W.Dropout1Undecomposed(), inputs, passes=[pass_decomposition, pass_fusion])
-    assert len(fused_nodes(gm)) == 1
+    (node,) = fused_nodes(gm)
+    # fixed stream: the reference's +-1e-3 keep-rate window is 2.2 sigma wide for 2^20 elements
+    node.target.rand_seed = 0xC0FFEE_0000_0001
     out, mask = gm(*inputs)
     mm_36 = torch.mm(view_9, primals_16.permute(1, 0))
     view_10 = (mm_36 + primals_17).view(512, 2, 1024)
