@@ -304,6 +304,19 @@ def main():
         mhz = details[dom]["clock_probe"]["shader_mhz"]
         clock = {"shader_mhz": mhz, "peak_at_shader_mhz": round(PEAK_FP16_TFLOPS * mhz / 2400.0, 1),
                  "frac_at_shader_mhz": round(dom_tflops / (PEAK_FP16_TFLOPS * mhz / 2400.0), 4)}
+    # what the matrix cores alone sustain (register-only MFMA loop, no memory traffic) on operands distributed
+    # like the benchmark's, and on zeros: the first is the practical MFMA ceiling for this data on this part
+    mfma_only = None
+    if args.clock_probe:
+        probe = jit.MfmaProbe()
+        g = torch.Generator(device="cpu").manual_seed(0xE7A0)
+        rnd = torch.randn(1 << 16, generator=g).half().cuda()
+        t_rnd, mhz_rnd = probe.run(rnd)
+        t_zero, mhz_zero = probe.run(torch.zeros_like(rnd))
+        mfma_only = {"normal_operands_tflops": round(t_rnd, 1), "normal_operands_shader_mhz": round(mhz_rnd),
+                     "zero_operands_tflops": round(t_zero, 1), "zero_operands_shader_mhz": round(mhz_zero)}
+        clock["frac_of_mfma_only_normal_operands"] = round(dom_tflops / t_rnd, 4)
+        log(f"[bench] register-only MFMA loop: {mfma_only}")
     for d in details.values():
         d.pop("_ms"); d.pop("_best")
     line = {
@@ -320,7 +333,7 @@ def main():
                      "frac": round(dom_tflops / PEAK_FP16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get((dom, details[dom]["tile"])),
                      "kernel": f"config {dom} ({details[dom]['workload']}, tile {details[dom]['tile']})",
-                     "us": details[dom]["us"], **clock},
+                     "us": details[dom]["us"], **clock, "mfma_only": mfma_only},
         "cpu_baseline": cpu,
         "per_config": details,
     }
