@@ -58,7 +58,7 @@ class Case:
         per_set = sum(t.numel() * t.element_size() for t in self.cpu_inputs)
         per_set += sum(int(torch.tensor(s).prod()) * torch.empty(0, dtype=d).element_size()
                        for s, d in self.op.store_meta.values())
-        self.nsets = max(2, -(-ROTATE_BYTES // per_set))
+        self.nsets = max(4, -(-ROTATE_BYTES // per_set))
         self.sets = []
         stream = torch.cuda.current_stream()
         for _ in range(self.nsets):
@@ -130,18 +130,24 @@ def spin_up(torch, fn, seconds=0.15):
         torch.cuda.synchronize()
 
 
-def time_loop(torch, fn, steps, warmup):
+def time_loop(torch, fn, steps, warmup, repeats=1):
+    """ms per call: `steps` back-to-back calls between two HIP events on the launch stream, after a clock
+    spin-up and `warmup` untimed calls; the median of `repeats` such regions."""
     spin_up(torch, fn)
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(steps):
-        fn(i)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps   # ms per call
+    samples = []
+    for _ in range(repeats):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        samples.append(e0.elapsed_time(e1) / steps)
+    samples.sort()
+    return samples[len(samples) // 2]
 
 
 def time_graph(torch, fn, steps, warmup, span):
@@ -215,6 +221,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="timed regions of --steps launches per config; the median is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--configs", default="1,2,3,4,5")
@@ -242,7 +250,7 @@ def main():
         case = Case(cfg, torch, W, fused_nodes)
         wl = case.wl
         # parity first: a number from a kernel that computes something else is void
-        parity = None
+        parity = normwise = None
         if not args.no_check:
             case.launch(0)
             torch.cuda.synchronize()
@@ -254,12 +262,21 @@ def main():
                 if not ok:
                     sys.exit(f"bench.py: config {cfg} output {i} fails parity (max rel err {err:.3e})")
             parity = max(errs)
-        ms = time_loop(torch, case.launch, args.steps, args.warmup)
+            normwise = max(float((o.detach().cpu().float() - r).abs().max() / r.abs().max().clamp_min(1e-30))
+                           for o, r in zip(case.outputs(0), refs))
+        ms = time_loop(torch, case.launch, args.steps, args.warmup, args.repeats)
         ms_graph = time_graph(torch, case.launch, args.steps, args.warmup, span=case.nsets * 4)
         ms_unf = time_loop(torch, case.launch_unfused, max(20, args.steps // 4), max(5, args.warmup // 4))
         ms_unf_graph = time_graph(torch, case.launch_unfused, max(20, args.steps // 4), 5, span=case.nsets)
         best = min(x for x in (ms, ms_graph) if x)
         best_unf = min(x for x in (ms_unf, ms_unf_graph) if x)
+        ms_unf_lib = None
+        if cfg == 1:   # the library-fused form of the same graph: bias folded into the GEMM (addmm), then GELU
+            gelu = torch.nn.functional.gelu
+            ms_unf_lib = time_loop(torch, lambda i: gelu(torch.addmm(case.sets[i % case.nsets][3][2],
+                                                                     case.sets[i % case.nsets][3][0],
+                                                                     case.sets[i % case.nsets][3][1]), approximate="tanh"),
+                                   max(20, args.steps // 4), 5)
         details[cfg] = {
             "workload": wl.name, "dims_MNKL": list(wl.dims), "tile": case.op.tile.tag(),
             "us": round(ms * 1e3, 2), "us_graph": None if ms_graph is None else round(ms_graph * 1e3, 2),
@@ -270,8 +287,10 @@ def main():
             "unfused_us": round(ms_unf * 1e3, 2),
             "unfused_us_graph": None if ms_unf_graph is None else round(ms_unf_graph * 1e3, 2),
             "speedup_vs_unfused": round(best_unf / best, 3),
-            "max_rel_err": parity, "buffer_sets": case.nsets, "_ms": ms, "_best": best,
+            "max_rel_err": parity, "normwise_err": normwise, "buffer_sets": case.nsets, "_ms": ms, "_best": best,
         }
+        if ms_unf_lib is not None:
+            details[cfg]["unfused_addmm_gelu_us"] = round(ms_unf_lib * 1e3, 2)
         if args.clock_probe:
             details[cfg]["clock_probe"] = case.clock_probe(jit)
         log(f"[bench] config {cfg} {wl.name}: {details[cfg]}")
@@ -294,7 +313,8 @@ def main():
     cpu = None
     if not args.no_cpu_baseline:
         v, cores, secs = cpu_baseline(torch, W, evt_oracle, vcfgs)
-        cpu = {"value": round(v, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        cpu_model = next((ln.split(":", 1)[1].strip() for ln in open("/proc/cpuinfo") if ln.startswith("model name")), "")
+        cpu = {"value": round(v, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port", "cpu": cpu_model,
                "sample": f"configs {vcfgs} at full size, PyTorch fp32 eager on CPU, median of 3 after 1 warm-up "
                          f"({secs:.2f} s per pass)"}
     # the published peak assumes 2.4 GHz; under this load the part clocks lower, so also relate the kernel to the
@@ -322,7 +342,7 @@ def main():
     line = {
         "metric": "fused GEMM+epilogue TFLOP/s, % MI355X fp16 MFMA peak, speedup vs unfused",
         "value": round(flops / (step_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_ms, 5),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "repeats": args.repeats, "ms_per_step": round(step_ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "one fused launch each of configs " + ",".join(map(str, vcfgs)) +
