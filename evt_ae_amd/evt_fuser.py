@@ -87,6 +87,7 @@ class FusedOpBase:
         self.mode = os.environ.get("MODE", "RUN")
         self.launched = False
         self.partition_names = epilogue_visitor.partition_names
+        self.reference_module: GraphModule = epilogue_visitor.reference_gm
         self.rtol = 1e-2
         self.atol = 1e-3
         self.ir: EpilogueIR = epilogue_visitor.ir
@@ -216,10 +217,54 @@ class FusedOpBase:
                 self.reference(args, results)
             return results
 
+    def anchor_eager(self, A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+        """The anchor (mm / bmm with its fused operand permutes) run eagerly."""
+        raise NotImplementedError("Should be Overwritten by child class")
+
     def reference(self, args, results):
-        """MODE=DEBUG self check against the eager fp32 evaluation of the
-        partition (reference: evt_fuser.py:98-172, rtol 1e-2)."""
-        raise NotImplementedError()
+        """MODE=DEBUG self check on the first call (reference: evt_fuser.py:551-553,
+        :688-689 -> reference_base)."""
+        return self.reference_base(args, results)
+
+    @staticmethod
+    def pass_rate(out: torch.Tensor, ref: torch.Tensor, criteria: dict) -> float:
+        return float(torch.sum(torch.isclose(out, ref, **criteria)) / max(out.numel(), 1))
+
+    def reference_base(self, args, results, verbose: bool = True) -> List[dict]:
+        """In-situ checker (reference: FusedOpBase.reference_base,
+        evt_fuser.py:98-172): run the anchor eagerly in the operands' dtype, feed
+        it as `accum` to the extracted epilogue module together with the
+        partition inputs, and compare every output of the fused kernel with
+        allclose(rtol=self.rtol); on a mismatch report maximum absolute /
+        relative error and the atol / rtol pass rates.  Returns one record per
+        output; nothing is raised (the reference prints and drops into a
+        debugger)."""
+        accum = self.anchor_eager(args[-2], args[-1])
+        named = dict(zip(self.input_names, args[:len(self.input_names)]))
+        inputs = {n.name: named[n.name] for n in self.reference_module.graph.nodes
+                  if n.op == "placeholder" and n.name != "accum"}
+        with torch.no_grad():
+            refs = self.reference_module(accum=accum, **inputs)
+        report = []
+        for output, out, ref in zip(self.outputs, results, refs):
+            o = out.contiguous().view(-1)
+            r = ref.contiguous().view(-1).to(o.dtype) if ref.dtype != o.dtype else ref.contiguous().view(-1)
+            rec = {"name": self.get_output_name(output), "match": bool(torch.allclose(o, r, rtol=self.rtol))}
+            if not rec["match"] and o.dtype != torch.bool:
+                of, rf = o.float(), r.float()
+                rec.update(max_abs=float(torch.max(torch.abs(of - rf))),
+                           max_rel=float(torch.max(torch.abs(of - rf) / torch.abs(rf).clamp_min(1e-30))),
+                           atol_pass_rate=self.pass_rate(of, rf, {"atol": self.atol, "rtol": 0.0}),
+                           rtol_pass_rate=self.pass_rate(of, rf, {"rtol": self.rtol, "atol": 0.0}))
+                if verbose:
+                    print(f"!!!!!!!!!!!!!!result mismatch: {rec['name']}!!!!!!!!!!!!!!")
+                    print("maximum abs error: ", rec["max_abs"])
+                    print("maximum relative error: ", rec["max_rel"])
+                    print("atol passed rate: ", rec["atol_pass_rate"])
+                    print("rtol passed rate: ", rec["rtol_pass_rate"])
+            report.append(rec)
+        self.last_reference_report = report
+        return report
 
     def get_src(self, node: Node) -> Node:
         if packet(node.target) in self.mainloop_fusion_targets and node.name in self.partition_names:
@@ -292,6 +337,9 @@ class FusedGEMM(FusedOpBase):
         A = A.contiguous()
         B = B.contiguous()
         return A, self.lda, 0, B, self.ldb, 0
+
+    def anchor_eager(self, A, B):
+        return torch.mm(A if self.a_kc else A.t(), B.t() if self.b_kc else B)
 
     def get_src_layout(self, node: Node) -> str:
         if packet(node.target) == aten.permute and node.name in self.partition_names:
@@ -375,6 +423,9 @@ class FusedBMM(FusedOpBase):
         if self.copy_B:
             B = aten.permute(B, self.permute_B).contiguous()
         return A, self.lda, self.bsa, B, self.ldb, self.bsb
+
+    def anchor_eager(self, A, B):
+        return torch.bmm(aten.permute(A, self.permute_A), aten.permute(B, self.permute_B))
 
 
 def _unsupported_anchor(name: str, where: str):
@@ -466,6 +517,7 @@ class EVTFuser:
         self.inputs = inputs
         self.outputs = outputs
         self.outputs_subgraph = set(outputs)
+        self.reference_gm = self._extract_reference(graph_module, anchor, epilogue_partition, inputs, outputs)
 
         # Step 3: build the IR
         (ashape, adtype) = node_shape_dtype(anchor)
@@ -527,6 +579,23 @@ class EVTFuser:
             graph_module.graph.inserting_after(view_node)
         self.fused_kernel = fused_kernel
         return fused_kernel
+
+    @staticmethod
+    def _extract_reference(graph_module: GraphModule, anchor: Node, epilogue_partition, inputs, outputs) -> GraphModule:
+        """The epilogue as a module of its own: placeholder `accum` for the anchor's
+        result plus one placeholder per partition input, returning the
+        partition's outputs in order (the reference's `reference_gm`, consumed by
+        FusedOpBase.reference_base, evt_fuser.py:98-126)."""
+        import torch.fx as fx
+        g = fx.Graph()
+        env: Dict[Node, Node] = {anchor: g.placeholder("accum")}
+        for inp in inputs:
+            if inp is not anchor:
+                env[inp] = g.placeholder(inp.name)
+        for node in epilogue_partition:
+            env[node] = g.node_copy(node, lambda n: env[n])
+        g.output(tuple(env[o] for o in outputs))
+        return GraphModule(graph_module, g)
 
     def _accum_dependents(self, anchor: Node, epi_set) -> set:
         full = {anchor}

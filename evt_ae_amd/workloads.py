@@ -385,6 +385,23 @@ def _h(g, shape, scale=1.0):
     return _randn(g, shape, scale)
 
 
+class BMMPartition2(torch.nn.Module):
+    """unittest/evt_fuser/bmm.py:48-67.  Its sum runs over the sequence axis and
+    over half of the batch axis (l = b*16 + h, summed over b): the epilogue's
+    reductions cover exactly N or exactly M, so pass_fusion fuses the BMM with
+    the permuted store and leaves sum / div as eager kernels."""
+    def forward(self, view_3, view_83):
+        permute_128 = aten.permute(view_3, [1, 2, 0])
+        bmm_10 = aten.bmm(permute_128, view_83)
+        permute_177 = aten.permute(bmm_10, [2, 0, 1])
+        view_84 = aten.view(permute_177, [512, 2, 1024])
+        sum_15 = aten.sum(view_84, [0, 1], True)
+        clone_11 = aten.clone(view_84, memory_format=torch.contiguous_format)
+        view_101 = aten.view(clone_11, [1024, 1024])
+        div = aten.div(sum_15, 20)
+        return view_101, div
+
+
 class MMPartition12(torch.nn.Module):
     """unittest/evt_fuser/mm.py:216-236: relu, its `ne` mask, and a dropout
     (rand_like / ge / mul) whose mask is returned too."""
@@ -454,6 +471,7 @@ REFERENCE_PATTERNS = {
     "mm10": (MMPartition10, lambda g: [_h(g, (16384, 1024), 0.05), _h(g, (1024, 4096), 0.05)]),
     "mm11": (MMPartition11, lambda g: [_h(g, (33792, 768), 0.01), _h(g, (33792, 768))]),
     "bmm1": (BMMPartition1, lambda g: [_h(g, (512, 32, 64)), _h(g, (32, 512, 512), 0.05)]),
+    "bmm2": (BMMPartition2, lambda g: [_h(g, (512, 32, 64), 0.3), _h(g, (32, 512, 512), 0.05)]),
     "bmm3": (BMMPartition3, lambda g: [_h(g, (512, 32, 64)), _h(g, (512, 32, 64), 0.2), _h(g, (2, 512)),
                                        _h(g, (1,)), _h(g, (1,)), _h(g, (1,))]),
 }

@@ -83,6 +83,21 @@ def test_reference_patterns_lower_correctly(name):
     _check(cls, inputs)
 
 
+def test_bmm_partition2_is_fused_up_to_its_cross_batch_sum():
+    """bmm.py:48-67: the store through permute/view/clone is fused; the sum over
+    the sequence axis and half of the batch axis stays outside the kernel."""
+    from evt_ae_amd.evt_fuser import target_name
+    inputs = W.pattern_inputs("bmm2")
+    gm = W.fuse(W.BMMPartition2(), inputs)
+    (n,) = fused_nodes(gm)
+    assert [(s.role, s.kind) for s in n.target.ir.slots] == [("store", "aux")]
+    assert "sum" in {target_name(x.target) for x in gm.graph.nodes if x.op == "call_function"}
+    got = run_emulated(gm, inputs)
+    ref = evt_oracle.eval_fp32(W.BMMPartition2(), inputs)
+    assert evt_oracle.max_rel_err(got[0].float(), ref[0]) <= 5e-3
+    assert torch.allclose(got[1].float(), ref[1], atol=2e-1)      # eager fp16 tail, the reference's criterion
+
+
 def test_reference_patterns_shrunk():
     """mm1/mm6/mm7 at reduced sizes (same graphs; the view shapes are fixed by
     the reference so M = 1024 / 2048 stays, K is what the CPU pays for)."""
@@ -166,6 +181,29 @@ def test_pass_decomposition_rewrites():
     assert not any(target_name(x.target) == "native_dropout" for x in gm.graph.nodes if x.op == "call_function")
     assert any(s.kind == "rand" for s in n.target.ir.slots)
     assert [tuple(v[0]) for v in n.target.store_meta.values()] and len(n.target.outputs) == 2
+
+
+def test_in_situ_checker():
+    """FusedOpBase.reference_base (the reference's MODE=DEBUG self check,
+    evt_fuser.py:98-172): the extracted epilogue module fed with the eager anchor
+    agrees with the fused result, and a corrupted result is reported with its
+    error figures."""
+    for cls, inputs in ((W.CONFIGS[3].module, W.make_inputs(3, W.SMALL_SHAPES[3])),
+                        (W.BMMPartition1, W.pattern_inputs("bmm1"))):
+        gm = W.fuse(cls(), inputs)
+        (n,) = fused_nodes(gm)
+        op = n.target
+        ph = [x for x in gm.graph.nodes if x.op == "placeholder"]
+        args = [inputs[ph.index(a)].float() for a in n.args]      # fp32 on the CPU: eager half matmul is slow there
+        from tests.util import emulate_fused
+        results = [r.float() for r in emulate_fused(op, *[inputs[ph.index(a)] for a in n.args])]
+        report = op.reference_base(args, results, verbose=False)
+        assert [r["name"] for r in report] == [op.get_output_name(o) for o in op.outputs]
+        assert all(r["match"] or r["rtol_pass_rate"] > 0.99 for r in report), report
+        bad = [r.clone() for r in results]
+        bad[0].view(-1)[::7] += 1.0
+        report = op.reference_base(args, bad, verbose=False)
+        assert not report[0]["match"] and report[0]["max_abs"] >= 0.9 and report[0]["rtol_pass_rate"] < 0.9
 
 
 def test_unsupported_ops_raise():

@@ -109,7 +109,7 @@ def test_reductions_are_deterministic_and_workspace_reusable():
 PATTERN_ATOL = 2e-1   # the reference's own criterion (unittest/evt_fuser/mm.py:28, bmm.py:27)
 
 
-@pytest.mark.parametrize("name", ["mm1", "mm2", "mm3", "mm4", "mm5", "mm6", "mm7", "mm9", "mm10", "mm11", "bmm1", "bmm3"])
+@pytest.mark.parametrize("name", ["mm1", "mm2", "mm3", "mm4", "mm5", "mm6", "mm7", "mm9", "mm10", "mm11", "bmm1", "bmm2", "bmm3"])
 def test_reference_fuser_patterns(name):
     """The graph patterns of the reference's fuser tests, through pass_fusion,
     checked as the reference does (fused vs the same module run eagerly in
@@ -125,10 +125,11 @@ def test_reference_fuser_patterns(name):
     eager = list(eager) if isinstance(eager, (tuple, list)) else [eager]
     torch.cuda.synchronize()
     refs = evt_oracle.eval_fp32(cls(), inputs)
-    for o, e, r in zip(outs, eager, refs):
+    for i, (o, e, r) in enumerate(zip(outs, eager, refs)):
         assert tuple(o.shape) == tuple(e.shape)
         assert torch.allclose(o.float(), e.float(), atol=PATTERN_ATOL, rtol=1e-2)
-        is_sum = o.dim() >= 1 and o.numel() < r.numel() + 1 and o.shape != refs[0].shape
+        if name == "bmm2" and i == 1:
+            continue    # produced by eager fp16 kernels from the fused kernel's fp16 output, not by the epilogue
         err = evt_oracle.max_rel_err(o, r)
         assert err <= FP16_TOL, f"{name}: max rel err {err:.3e}"
 
@@ -189,6 +190,25 @@ def test_random_fuser_patterns(name):
         assert not torch.equal(masks[0], masks[1])
         keep = masks[0].float().mean().item()          # the reference's criterion (dropout.py:73-75)
         assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
+
+
+def test_debug_mode_self_check():
+    """MODE=DEBUG (evt_fuser.py:98-172): the first call compares the kernel with
+    the eager anchor + extracted epilogue module and records the verdict."""
+    for cfg in (1, 4):
+        wl = W.CONFIGS[cfg]
+        inputs = [t.cuda() for t in W.make_inputs(cfg, W.SMALL_SHAPES[cfg])]
+        gm = W.fuse(wl.module(), inputs)
+        (node,) = fused_nodes(gm)
+        op = node.target
+        op.mode = "DEBUG"
+        gm(*inputs)
+        assert op.launched
+        report = op.last_reference_report
+        assert len(report) == len(op.outputs)
+        # eager runs in fp16 (two extra roundings), so elements near zero may miss the pure rtol 1e-2 test;
+        # the report's pass rates are what a developer reads then
+        assert all(r["match"] or r["atol_pass_rate"] > 0.999 or r["rtol_pass_rate"] > 0.98 for r in report), report
 
 
 def test_golden_fixtures():
