@@ -192,6 +192,44 @@ def test_random_fuser_patterns(name):
         assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
 
 
+def test_launch_is_graph_capturable():
+    """evt_launch allocates nothing and never synchronises, so a fused call with a
+    cross-workgroup reduction can be captured in a HIP graph (the reference runs
+    whole models from CUDA graphs, bert_modeling.py:170-182).  Every replay,
+    with eager work and synchronisations in between, must reproduce the eager
+    launch bit for bit (the workspace counters return to zero by themselves)."""
+    wl = W.CONFIGS[3]
+    inputs = [t.cuda() for t in W.make_inputs(3, W.SMALL_SHAPES[3])]
+    gm = W.fuse(wl.module(), inputs)
+    (node,) = fused_nodes(gm)
+    op = node.target
+    ph = [n for n in gm.graph.nodes if n.op == "placeholder"]
+    args = [inputs[ph.index(a)] for a in node.args]
+    eager = [o.clone() for o in op(*args)]
+    torch.cuda.synchronize()
+    outs = op.allocate_outputs("cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        a, keep = op.build_arguments(outs, *args)
+        ws_ptr, ws_bytes = op.workspace_for(a, side, "cuda")     # allocated and initialised before capture
+        for _ in range(2):
+            op.module.launch(a, ws_ptr, ws_bytes, side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        op.module.launch(a, ws_ptr, ws_bytes, torch.cuda.current_stream().cuda_stream)
+    for rep in range(4):
+        for t in outs.values():
+            t.zero_()
+        _ = (inputs[0].float() @ inputs[1].float()).sum().item()   # unrelated eager work + a sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, e in zip((op.output2store[op.get_output_name(o)] for o in op.outputs), eager):
+            assert torch.equal(outs[name].view(-1), e.contiguous().view(-1)), (rep, name)
+
+
 def test_debug_mode_self_check():
     """MODE=DEBUG (evt_fuser.py:98-172): the first call compares the kernel with
     the eager anchor + extracted epilogue module and records the verdict."""
