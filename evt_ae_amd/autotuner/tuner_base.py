@@ -126,7 +126,10 @@ class AutoTunerBase:
                            (256, 256, 32, 4, 2, 4, pipe), (256, 128, 64, 4, 2, 3, pipe), (128, 256, 64, 2, 4, 3, pipe),
                            (128, 256, 32, 2, 4, 4, pipe), (128, 128, 64, 2, 4, 4, pipe)]
             if self.N == 512:     # one tile spans the rows: row statistics complete inside the workgroup
-                shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0)]
+                shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0),
+                           # 32 x 256 wave tiles: 8 columns per lane halve the cross-lane steps per element of a
+                           # per-row reduction
+                           (128, 512, 64, 4, 2, 2, 0)]
         else:
             shapes = [(128, 128, 32, 2, 2, 2, 0), (64, 64, 32, 2, 2, 2, 0)]
         if self.dma and self.K <= 64:
