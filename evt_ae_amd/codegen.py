@@ -142,7 +142,7 @@ class Codegen:
         raise NotImplementedError(n.op)
 
     def slot_off(self, k: int, batch: str = "t.batch") -> str:
-        return f"(int64_t)({batch} / p.t{k}_ld) * p.t{k}_sl"
+        return f"(int64_t)evt::batch_index({batch}, p.t{k}_lm, p.t{k}_ld) * p.t{k}_sl"
 
     # -- sections ---------------------------------------------------------------
     def emit_params(self, e: _Emitter):
@@ -151,7 +151,7 @@ class Codegen:
         for k, s in enumerate(self.ir.slots):
             const = "const " if s.role == "load" else ""
             e(f"{const}{DTYPE_CTYPES[s.dtype]}* t{k};  // {s.role} {s.kind} '{s.name}'")
-            e(f"int64_t t{k}_sl, t{k}_sm, t{k}_sn; int t{k}_ld; int t{k}_vec;")
+            e(f"int64_t t{k}_sl, t{k}_sm, t{k}_sn; int t{k}_ld; int t{k}_lm; int t{k}_vec;")
         e(f"float s[{max(1, len(self.ir.scalars))}];")
         e("int fast;   // every per-element tensor is unit-stride / vector-aligned: interior tiles skip all checks")
         e.dedent()
@@ -486,7 +486,7 @@ class Codegen:
     def module_spec(self) -> dict:
         t = self.spec.tile
         return {
-            "abi": 1,
+            "abi": 2,
             "name": self.name,
             "tile": asdict(t),
             "a_k_contiguous": self.spec.a_kc,
@@ -556,8 +556,21 @@ class Codegen:
         e("g.tiles_m = (a->M + Cfg::BM - 1) / Cfg::BM;")
         e("g.tiles_n = (a->N + Cfg::BN - 1) / Cfg::BN;")
         e("g.workspace = nullptr;")
+        e("g.row_fold_mod = 0; g.row_fold_step = 1; g.row_fold_count = 1;")
+        folds = {(r.fold) for r in ir.reduces.values() if r.axis == "row"}
+        if folds - {""}:
+            # batches fold into one per-row result the way the reduction's output tensor shares elements between them
+            (fold,) = folds
+            k = next(s_.slot for s_ in ir.stores if s_.domain == "row")
+            e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
+            if fold == "mod":
+                e("  if (x.l_mod <= 0 || x.l_div != 1 || a->L % x.l_mod) return EVT_ERR_BAD_ARGS;")
+                e("  g.row_fold_mod = 1; g.row_fold_step = (int)x.l_mod; g.row_fold_count = a->L / (int)x.l_mod; }")
+            else:
+                e("  if (x.l_mod != 0 || x.l_div <= 1 || a->L % x.l_div) return EVT_ERR_BAD_ARGS;")
+                e("  g.row_fold_count = (int)x.l_div; }")
         e("// few partials: the last workgroup to arrive combines them; many: a finalize kernel does")
-        e("g.row_inkernel = (g.tiles_n <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
+        e("g.row_inkernel = (g.tiles_n * g.row_fold_count <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
         e("g.col_inkernel = (g.tiles_m <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
         e("if ((int64_t)g.tiles_m * g.tiles_n * a->L > 0x7fffffffLL) return EVT_ERR_RANGE;")
         e("if (a->N > (1 << 24)) return EVT_ERR_RANGE;   // column indices are carried as fp32")
@@ -583,11 +596,12 @@ class Codegen:
             ct = DTYPE_CTYPES[s.dtype]
             e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
             if s.kind == "rand":   # generated values: no storage behind this slot
-                e("  if (x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
+                e("  if (x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
             else:
-                e("  if (!x.ptr || x.l_div <= 0) return EVT_ERR_BAD_ARGS;")
+                e("  if (!x.ptr || x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
             e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
-            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div;")
+            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div; "
+              f"p.t{k}_lm = (int)x.l_mod;")
             e(f"  p.t{k}_vec = (x.stride_n == 1 ? 1 : 0) | ((x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "
               f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0) ? 2 : 0); }}")
         e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
@@ -610,7 +624,7 @@ class Codegen:
         e("  evt::GemmArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  return evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n).total();")
+        e("  return evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
         e("}")
         e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
         e("  if (bytes <= 0) return EVT_OK;")
@@ -623,7 +637,7 @@ class Codegen:
         e("  evt::GemmArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  const int64_t need = evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n).total();")
+        e("  const int64_t need = evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
         e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
         e("  g.workspace = (char*)ws;")
         e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L);")

@@ -343,16 +343,33 @@ struct WsLayout {
   __host__ __device__ int64_t total() const { return counter_bytes + row_bytes + col_bytes; }
 };
 
+// a per-row reduction goes through the workspace when several tiles span the
+// row or several batches fold into one result
+__host__ __device__ inline bool row_uses_workspace(const GemmArgs& g) { return g.tiles_n > 1 || g.row_fold_count > 1; }
+
 template <int ROW_STATE, int COL_STATE>
-__host__ __device__ inline WsLayout ws_layout(int M, int N, int L, int tiles_m, int tiles_n) {
+__host__ __device__ inline WsLayout ws_layout(const GemmArgs& g) {
   WsLayout w;
-  const bool row = ROW_STATE > 0 && tiles_n > 1;
-  const bool col = COL_STATE > 0 && tiles_m > 1;
-  const int64_t ncnt = (row ? (int64_t)L * tiles_m : 0) + (col ? (int64_t)L * tiles_n : 0);
+  const bool row = ROW_STATE > 0 && row_uses_workspace(g);
+  const bool col = COL_STATE > 0 && g.tiles_m > 1;
+  const int64_t ncnt = (row ? (int64_t)g.L * g.tiles_m : 0) + (col ? (int64_t)g.L * g.tiles_n : 0);
   w.counter_bytes = (ncnt * 4 + 255) / 256 * 256;
-  w.row_bytes = row ? ((int64_t)L * tiles_n * M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
-  w.col_bytes = col ? ((int64_t)L * tiles_m * N * COL_STATE * 4 + 255) / 256 * 256 : 0;
+  w.row_bytes = row ? ((int64_t)g.L * g.tiles_n * g.M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
+  w.col_bytes = col ? ((int64_t)g.L * g.tiles_m * g.N * COL_STATE * 4 + 255) / 256 * 256 : 0;
   return w;
+}
+
+// batch index of a tensor argument: batches that agree modulo l_mod, or l_div
+// consecutive ones, share elements
+__host__ __device__ inline int batch_index(int batch, int l_mod, int l_div) {
+  return (l_mod > 0 ? batch % l_mod : batch) / l_div;
+}
+// folded per-row reductions: the result a batch contributes to, and the j-th batch that contributes to a result
+__host__ __device__ inline int fold_key(const GemmArgs& g, int batch) {
+  return g.row_fold_count == 1 ? batch : (g.row_fold_mod ? batch % g.row_fold_step : batch / g.row_fold_count);
+}
+__host__ __device__ inline int fold_member(const GemmArgs& g, int key, int j) {
+  return g.row_fold_count == 1 ? key : (g.row_fold_mod ? key + j * g.row_fold_step : key * g.row_fold_count + j);
 }
 
 // Device-scope accesses for data exchanged between workgroups inside one
@@ -399,7 +416,7 @@ EVT_DEV bool row_reduce_publish(const typename Epi::Params& p, const Tile& t, co
   if constexpr (RS > 0) {
     const float* lds = (const float*)t.smem;
     int* flag = (int*)(t.smem + Cfg::WN * Cfg::BM * RS * 4);
-    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     float* part = (float*)(t.workspace + wl.counter_bytes);
     __syncthreads();
     for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
@@ -410,7 +427,7 @@ EVT_DEV bool row_reduce_publish(const typename Epi::Params& p, const Tile& t, co
       for (int c = 0; c < RS; ++c) st[c] = lds[lr * RS + c];
 #pragma unroll
       for (int w = 1; w < Cfg::WN; ++w) Epi::row_combine(st, lds + (w * Cfg::BM + lr) * RS);
-      if (t.tiles_n == 1) {
+      if (!row_uses_workspace(g)) {
         Epi::row_finalize(p, t.batch, row, st);
       } else {
         float* dst = part + (((int64_t)t.batch * t.tiles_n + t.tile_n) * t.M + row) * RS;
@@ -418,9 +435,9 @@ EVT_DEV bool row_reduce_publish(const typename Epi::Params& p, const Tile& t, co
         for (int c = 0; c < RS; ++c) st_device(dst + c, st[c]);
       }
     }
-    if (t.tiles_n == 1 || !g.row_inkernel) return false;
-    int* counter = (int*)t.workspace + t.batch * t.tiles_m + t.tile_m;
-    return arrive_last(counter, t.tiles_n, flag);
+    if (!row_uses_workspace(g) || !g.row_inkernel) return false;
+    int* counter = (int*)t.workspace + fold_key(g, t.batch) * t.tiles_m + t.tile_m;
+    return arrive_last(counter, t.tiles_n * g.row_fold_count, flag);
   } else {
     return false;
   }
@@ -431,23 +448,26 @@ template <class Cfg, class Epi, class Tile>
 EVT_DEV void row_reduce_complete(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
   constexpr int RS = Epi::ROW_STATE;
   if constexpr (RS > 0) {
-    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     const float* part = (const float*)(t.workspace + wl.counter_bytes);
-    int* counter = (int*)t.workspace + t.batch * t.tiles_m + t.tile_m;
+    const int key = fold_key(g, t.batch);
+    int* counter = (int*)t.workspace + key * t.tiles_m + t.tile_m;
     for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
       const int row = t.m0 + lr;
       if (row >= t.M) continue;
-      const float* src = part + ((int64_t)t.batch * t.tiles_n * t.M + row) * RS;
       float st[RS];
+      Epi::row_identity(st);
+      // batches in fold order, tiles in tile order: the same sum whichever workgroup arrives last
+      for (int f = 0; f < g.row_fold_count; ++f) {
+        const float* src = part + ((int64_t)fold_member(g, key, f) * t.tiles_n * t.M + row) * RS;
+        for (int j = 0; j < t.tiles_n; ++j) {
+          float o[RS];
 #pragma unroll
-      for (int c = 0; c < RS; ++c) st[c] = ld_device(src + c);
-      for (int j = 1; j < t.tiles_n; ++j) {
-        float o[RS];
-#pragma unroll
-        for (int c = 0; c < RS; ++c) o[c] = ld_device(src + (int64_t)j * t.M * RS + c);
-        Epi::row_combine(st, o);
+          for (int c = 0; c < RS; ++c) o[c] = ld_device(src + (int64_t)j * t.M * RS + c);
+          Epi::row_combine(st, o);
+        }
       }
-      Epi::row_finalize(p, t.batch, row, st);
+      Epi::row_finalize(p, fold_member(g, key, 0), row, st);
     }
     if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -481,7 +501,7 @@ EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, co
         for (int c = 0; c < CS; ++c) lds[(t.wm * Cfg::BN + t.lcol(ni)) * CS + c] = cs[ni][c];
     }
     __syncthreads();
-    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     float* part = (float*)(t.workspace + wl.counter_bytes + wl.row_bytes);
     for (int lc = t.tid; lc < Cfg::BN; lc += Cfg::THREADS) {
       const int col = t.n0 + lc;
@@ -500,7 +520,7 @@ EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, co
       }
     }
     if (t.tiles_m == 1 || !g.col_inkernel) return false;
-    const int row_counters = (Epi::ROW_STATE > 0 && t.tiles_n > 1) ? t.L * t.tiles_m : 0;
+    const int row_counters = (Epi::ROW_STATE > 0 && row_uses_workspace(g)) ? t.L * t.tiles_m : 0;
     int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
     return arrive_last(counter, t.tiles_m, flag);
   } else {
@@ -516,9 +536,9 @@ EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, c
     constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
     constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
     float* lds = (float*)(t.smem + ROW_AREA);
-    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(t.M, t.N, t.L, t.tiles_m, t.tiles_n);
+    const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     const float* part = (const float*)(t.workspace + wl.counter_bytes + wl.row_bytes);
-    const int row_counters = (Epi::ROW_STATE > 0 && t.tiles_n > 1) ? t.L * t.tiles_m : 0;
+    const int row_counters = (Epi::ROW_STATE > 0 && row_uses_workspace(g)) ? t.L * t.tiles_m : 0;
     int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
     // SHARES threads per column each fold every SHARES-th partial in tile order
     // (independent loads in flight together), LDS then combines the shares in order
@@ -556,21 +576,25 @@ EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, c
 // 2^LG-th tile partial (in tile order), then the lanes combine pairwise.  The
 // combination tree is fixed by (tiles_n, LG), so results are reproducible.
 template <class Epi, int LG>
-__global__ void __launch_bounds__(256) evt_row_finalize_kernel(typename Epi::Params p, const float* part,
-                                                               int M, int L, int tiles_n) {
+__global__ void __launch_bounds__(256) evt_row_finalize_kernel(typename Epi::Params p, const float* part, GemmArgs g) {
   constexpr int RS = Epi::ROW_STATE > 0 ? Epi::ROW_STATE : 1;
   constexpr int G = 1 << LG;
+  const int M = g.M, tiles_n = g.tiles_n;
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t rowid = gid >> LG;
   const int sub = (int)(gid & (G - 1));
-  const bool live = rowid < (int64_t)L * M;
-  const int batch = live ? (int)(rowid / M) : 0;
+  const bool live = rowid < (int64_t)(g.L / g.row_fold_count) * M;
+  const int key = live ? (int)(rowid / M) : 0;
   const int row = live ? (int)(rowid % M) : 0;
+  const int batch = fold_member(g, key, 0);
   float st[RS];
   Epi::row_identity(st);
   if (live) {
-    const float* src = part + ((int64_t)batch * tiles_n * M + row) * RS;
-    for (int j = sub; j < tiles_n; j += G) Epi::row_combine(st, src + (int64_t)j * M * RS);
+    // partial q = (batch f of the fold, tile j); lane `sub` folds every G-th one
+    for (int q = sub; q < tiles_n * g.row_fold_count; q += G) {
+      const int f = q / tiles_n, j = q - f * tiles_n;
+      Epi::row_combine(st, part + (((int64_t)fold_member(g, key, f) * tiles_n + j) * M + row) * RS);
+    }
   }
 #pragma unroll
   for (int o = G >> 1; o > 0; o >>= 1) {
@@ -616,20 +640,20 @@ __global__ void __launch_bounds__(256) evt_col_finalize_kernel(typename Epi::Par
 // tile spans the reduced axis).
 template <class Epi>
 inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hipStream_t stream) {
-  const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g.M, g.N, g.L, g.tiles_m, g.tiles_n);
-  if (Epi::ROW_STATE > 0 && g.tiles_n > 1 && !g.row_inkernel) {
+  const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
+  if (Epi::ROW_STATE > 0 && row_uses_workspace(g) && !g.row_inkernel) {
     const float* part = (const float*)(g.workspace + wl.counter_bytes);
     int lg = 0;
-    while ((1 << lg) < g.tiles_n && lg < 6) ++lg;
-    const int64_t threads = ((int64_t)g.L * g.M) << lg;
+    while ((1 << lg) < g.tiles_n * g.row_fold_count && lg < 6) ++lg;
+    const int64_t threads = ((int64_t)(g.L / g.row_fold_count) * g.M) << lg;
     const unsigned grid = (unsigned)((threads + 255) / 256);
     switch (lg) {
-      case 1: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 1>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
-      case 2: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 2>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
-      case 3: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 3>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
-      case 4: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 4>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
-      case 5: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 5>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
-      default: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 6>), dim3(grid), dim3(256), 0, stream, p, part, g.M, g.L, g.tiles_n); break;
+      case 1: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 1>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
+      case 2: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 2>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
+      case 3: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 3>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
+      case 4: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 4>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
+      case 5: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 5>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
+      default: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 6>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
     }
   }
   if (Epi::COL_STATE > 0 && g.tiles_m > 1 && !g.col_inkernel) {

@@ -56,6 +56,11 @@ struct GemmArgs {
   // phase 2 of a cross-tile reduction runs inside this kernel (last workgroup
   // to arrive) instead of in a separate finalize kernel
   int row_inkernel, col_inkernel;
+  // A per-row reduction may also fold batches into one result: row_fold_count
+  // batches share a result; with row_fold_mod they are l, l + row_fold_step, ...
+  // (result keyed by l % row_fold_step), otherwise row_fold_count consecutive
+  // ones (keyed by l / row_fold_count).  (0, 1, 1): every batch on its own.
+  int row_fold_mod, row_fold_step, row_fold_count;
 };
 
 // Compile-time description of one kernel variant.

@@ -134,6 +134,7 @@ class FusedOpBase:
                 ta.ptr = t.data_ptr()
             ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
             ta.l_div = slot.strides.l_div
+            ta.l_mod = slot.strides.l_mod
         for i, s in enumerate(self.ir.scalars):
             a.scalars[i] = s
         if self.ir.rng_scalar is not None:
@@ -653,7 +654,7 @@ class EVTFuser:
                 post.insert(0, ("view", list(nshape)))
             node = src
         sshape, _ = node_shape_dtype(node)
-        key = (value, st.stride_l, st.stride_m, st.stride_n, st.l_div, dtype, domain)
+        key = (value, st.stride_l, st.stride_m, st.stride_n, st.l_div, st.l_mod, dtype, domain)
         if key in store_key:
             self.output2store[name] = store_key[key]
             stored_shape = self.store_meta[store_key[key]][0]
@@ -691,7 +692,7 @@ class EVTFuser:
             st = fit_strides(coord, self.L, self.M, self.N)
             if st is None:
                 raise NotImplementedError(f"input {node.name}: broadcast pattern is not strided in (l, m, n)")
-            key = (node.name, (st.stride_l, st.stride_m, st.stride_n, st.l_div))
+            key = (node.name, (st.stride_l, st.stride_m, st.stride_n, st.l_div, st.l_mod))
             if key in self.load_cache:
                 return self.load_cache[key]
             if dtype not in DTYPE_NAMES:
@@ -946,15 +947,30 @@ class EVTFuser:
         if st is None:
             raise NotImplementedError(f"{node.name}: reduction result is not strided in (l, m, n)")
         numel = rc.numel()
+        fold, fold_step, fold_count = "", 1, 1
         if st.stride_n == 0 and numel == self.L * self.M:
             axis = "row"
+        elif st.stride_n == 0 and st.l_mod and st.l_div == 1 and numel == st.l_mod * self.M:
+            # also summed over the batches that agree modulo l_mod (e.g. a [S, B, H*D] view of a BMM over
+            # L = B*H batches, reduced over S and B: unittest/evt_fuser/bmm.py:48-67)
+            axis, fold, fold_step, fold_count = "row", "mod", st.l_mod, self.L // st.l_mod
+        elif st.stride_n == 0 and not st.l_mod and st.l_div > 1 and numel == (self.L // st.l_div) * self.M:
+            axis, fold, fold_step, fold_count = "row", "div", 1, st.l_div     # l_div consecutive batches summed
         elif st.stride_m == 0 and numel == self.L * self.N and (self.L == 1 or st.stride_l != 0):
             axis = "col"
         else:
             raise NotImplementedError(
-                f"{node.name}: reduces over something other than exactly the N axis or exactly the M axis")
+                f"{node.name}: reduces over something other than the N axis (optionally with batches folded) "
+                f"or exactly the M axis")
+        if fold and kind not in ("sum", "max"):
+            raise NotImplementedError(f"{node.name}: {kind} reduction that also folds batches")
+        if axis == "row":
+            for other in self.ir.reduces.values():
+                if other.axis == "row" and (other.fold, other.fold_step, other.fold_count) != (fold, fold_step, fold_count):
+                    raise NotImplementedError(f"{node.name}: per-row reductions of one epilogue fold batches differently")
         rname = f"{node.name}_red"
-        self.ir.add_reduce(rname, kind, axis, value)
+        red = self.ir.add_reduce(rname, kind, axis, value)
+        red.fold, red.fold_step, red.fold_count = fold, fold_step, fold_count
         names = []
         for c in comps:
             n = f"{node.name}_r{c}"

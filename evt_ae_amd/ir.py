@@ -148,10 +148,17 @@ def accum_coord(L: int, M: int, N: int, batched: bool) -> Coord:
 
 @dataclass
 class Strides:
+    """offset(l, m, n) = (lb // l_div) * stride_l + m * stride_m + n * stride_n,
+    lb = l % l_mod if l_mod else l."""
     stride_l: int
     stride_m: int
     stride_n: int
     l_div: int = 1
+    l_mod: int = 0       # > 0: the batch index enters modulo l_mod (batches l and l + l_mod share elements)
+
+    def batch_index(self, l):
+        lb = l % self.l_mod if self.l_mod else l
+        return lb // self.l_div
 
     @property
     def kind(self) -> str:
@@ -169,7 +176,8 @@ class Strides:
 
 def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Sequence[int]] = None,
                 seed: int = 0) -> Optional[Strides]:
-    """Fit  offset(l, m, n) = (l // l_div) * sl + m * sm + n * sn  to `coord`.
+    """Fit  offset(l, m, n) = (lb // l_div) * sl + m * sm + n * sn,  lb = l % l_mod
+    (or l), to `coord`.
 
     `elem_strides` are the memory strides of the tensor (default: contiguous).
     Returns None when the mapping is not of that form (checked on the corners,
@@ -201,7 +209,7 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
     sm = int(offset(z, z + 1, z)[0]) if M > 1 else 0
     sn = int(offset(z, z, z + 1)[0]) if N > 1 else 0
     # batch: find the smallest l at which the offset changes
-    sl, l_div = 0, 1
+    sl, l_div, l_mod = 0, 1, 0
     if L > 1:
         ls = np.arange(L, dtype=np.int64)
         offs = offset(ls, np.zeros_like(ls), np.zeros_like(ls))
@@ -209,7 +217,12 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
         if len(nz):
             l_div = int(nz[0])
             sl = int(offs[l_div])
-    st = Strides(sl, sm, sn, l_div)
+            # periodic in l: the smallest period that divides L (a full period is no period)
+            for period in range(l_div + 1, L):
+                if L % period == 0 and np.array_equal(offs, offs[ls % period]):
+                    l_mod = period
+                    break
+    st = Strides(sl, sm, sn, l_div, l_mod)
     rng = np.random.default_rng(seed)
     npts = 4096
     l = rng.integers(0, L, npts)
@@ -218,7 +231,7 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
     # always include the far corner
     l[0], m[0], n[0] = L - 1, M - 1, N - 1
     want = offset(l, m, n)
-    got = (l // l_div) * sl + m * sm + n * sn
+    got = st.batch_index(l) * sl + m * sm + n * sn
     if not np.array_equal(want, got):
         return None
     return st
@@ -283,6 +296,11 @@ class Reduce:
     axis: str            # 'row' (over n, one value per row) | 'col' (over m, one per column)
     input: str
     state_offset: int = 0
+    # a per-row reduction may also fold batches: 'mod' -> batches l, l + fold_step, ... (fold_count of them)
+    # share one result (keyed by l % fold_step); 'div' -> fold_count consecutive batches do (keyed by l // fold_count)
+    fold: str = ""
+    fold_step: int = 1
+    fold_count: int = 1
 
 
 @dataclass
@@ -462,7 +480,7 @@ class EpilogueIR:
             "nodes": [[n.name, n.op, n.inputs, n.domain, n.slot, n.reduce, n.comp]
                       for n in self.nodes.values()],
             "slots": [[s.name, s.role, s.dtype, s.domain, s.kind] for s in self.slots],
-            "reduces": [[r.name, r.kind, r.axis, r.input, r.state_offset] for r in self.reduces.values()],
+            "reduces": [[r.name, r.kind, r.axis, r.input, r.state_offset, r.fold] for r in self.reduces.values()],
             "stores": [[s.slot, s.input, s.domain] for s in self.stores],
             "rng_scalar": self.rng_scalar,
         }

@@ -29,6 +29,7 @@ INCLUDE_DIR = PKG_DIR.parent / "include"
 KERNEL_DIR = Path(os.environ.get("EVT_KERNEL_DIR", PKG_DIR / "_kernels"))
 CACHE_FILE = KERNEL_DIR / "compiled_cache.db"
 
+EVT_ABI_VERSION = 2
 EVT_MAX_TENSORS = 16
 EVT_MAX_SCALARS = 16
 
@@ -43,7 +44,7 @@ HIPCC_FLAGS = [
 
 class EvtTensorArg(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("stride_l", ctypes.c_int64), ("stride_m", ctypes.c_int64),
-                ("stride_n", ctypes.c_int64), ("l_div", ctypes.c_int64)]
+                ("stride_n", ctypes.c_int64), ("l_div", ctypes.c_int64), ("l_mod", ctypes.c_int64)]
 
 
 class EvtArgs(ctypes.Structure):
@@ -71,7 +72,7 @@ class KernelModule:
         self.lib.evt_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         self.lib.evt_launch.restype = ctypes.c_int
         self.lib.evt_launch.argtypes = [ctypes.POINTER(EvtArgs), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
-        if self.lib.evt_abi_version() != 1:
+        if self.lib.evt_abi_version() != EVT_ABI_VERSION:
             raise RuntimeError(f"{path}: ABI version mismatch")
         if hasattr(self.lib, "evt_clock_probe_read"):      # diagnostic builds only
             self.lib.evt_clock_probe_read.restype = ctypes.c_int

@@ -51,6 +51,7 @@ def register_all() -> List[jit.LazyModule]:
                 jit.load_module(op.ir, op.spec, clock_probe=True)
     for name, (cls, _) in W.RANDOM_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
     from .passes import pass_decomposition, pass_fusion
     W.fuse(W.Dropout1Undecomposed(), _meta(W.pattern_inputs("dropout1")), passes=[pass_decomposition, pass_fusion])
     from .autotuner.tuner_base import force_tile

@@ -386,10 +386,9 @@ def _h(g, shape, scale=1.0):
 
 
 class BMMPartition2(torch.nn.Module):
-    """unittest/evt_fuser/bmm.py:48-67.  Its sum runs over the sequence axis and
-    over half of the batch axis (l = b*16 + h, summed over b): the epilogue's
-    reductions cover exactly N or exactly M, so pass_fusion fuses the BMM with
-    the permuted store and leaves sum / div as eager kernels."""
+    """unittest/evt_fuser/bmm.py:48-67.  Its sum runs over the sequence axis (N)
+    and over half of the batch axis (l = b*16 + h, summed over b): a per-row
+    reduction that folds the batches which agree modulo 16."""
     def forward(self, view_3, view_83):
         permute_128 = aten.permute(view_3, [1, 2, 0])
         bmm_10 = aten.bmm(permute_128, view_83)
@@ -400,6 +399,22 @@ class BMMPartition2(torch.nn.Module):
         view_101 = aten.view(clone_11, [1024, 1024])
         div = aten.div(sum_15, 20)
         return view_101, div
+
+
+class FoldConsecutiveBatches(torch.nn.Module):
+    """Not a reference test: a BMM whose per-row sum also runs over pairs of
+    consecutive batches (the other way batches can fold into one result)."""
+    def forward(self, a, b, r):
+        bmm = aten.bmm(a, b)
+        y = aten.add(bmm, r)
+        v = aten.view(y, [3, 2, 40, 72])
+        s = aten.sum(v, [1, 3])
+        return y, aten.mul(s, 0.5)
+
+
+def fold_consecutive_inputs():
+    g = torch.Generator(device="cpu").manual_seed(17)
+    return [_h(g, (6, 40, 24), 0.3), _h(g, (6, 24, 72), 0.3), _h(g, (6, 40, 72), 0.3)]
 
 
 class MMPartition12(torch.nn.Module):

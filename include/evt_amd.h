@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define EVT_ABI_VERSION 1
+#define EVT_ABI_VERSION 2
 #define EVT_MAX_TENSORS 16
 #define EVT_MAX_SCALARS 16
 
@@ -42,8 +42,13 @@ extern "C" {
 
 /* One epilogue tensor (load or store).  Element (l, m, n) of the logical
  * [L, M, N] iteration space lives at
- *     ptr + (l / l_div) * stride_l + m * stride_m + n * stride_n   (elements).
- * A broadcast dimension has stride 0.  Replaces the (M, N, L)-strided
+ *     ptr + (lb / l_div) * stride_l + m * stride_m + n * stride_n   (elements),
+ *     lb = l_mod > 0 ? l % l_mod : l.
+ * A broadcast dimension has stride 0.  l_div > 1: l_div consecutive batches
+ * share elements (a [B, ...] tensor against L = B*H batches); l_mod > 0: batches
+ * that agree modulo l_mod do (an [H, ...] tensor against the same L).  For the
+ * output of a per-row reduction, batches that share elements are summed into
+ * them (the reduction then runs over N and over those batches).  Replaces the (M, N, L)-strided
  * tensor arguments of VisitorAuxLoad / VisitorRowBroadcast / VisitorRowStore
  * (src/cuda/epilogue/threadblock/visitor_load.hpp:364-571,
  *  visitor_store.hpp:46-145).
@@ -59,6 +64,7 @@ typedef struct EvtTensorArg {
   int64_t stride_m;
   int64_t stride_n;
   int64_t l_div;
+  int64_t l_mod;
 } EvtTensorArg;
 
 /* Launch arguments.  A is [L, M, K], B is [L, K, N]; which of the two

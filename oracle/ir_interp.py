@@ -3,7 +3,7 @@
 Evaluates an `EpilogueIR` (duck-typed: .nodes, .slots, .reduces, .stores,
 .scalars, .L/.M/.N) on fp32 torch tensors exactly as the generated kernels are
 specified to: every node once per (l, m, n), loads through the fitted
-(l // l_div, m, n) strides, reductions over the N axis ('row') or the M axis
+(batch index, m, n) strides, reductions over the N axis ('row') or the M axis
 ('col'), per-row / per-column post expressions, one rounding per store.  Used
 by the CPU tests to check that `EVTFuser.trace` (the host-side mirror of
 python/gtl/compiler/passes/evt_fuser.py:1065-1235) lowers a graph to an IR
@@ -67,7 +67,7 @@ def _gather_strided(t: torch.Tensor, st, L, M, N) -> torch.Tensor:
     l = torch.arange(L).view(L, 1, 1)
     m = torch.arange(M).view(1, M, 1)
     n = torch.arange(N).view(1, 1, N)
-    off = (l // st.l_div) * st.stride_l + m * st.stride_m + n * st.stride_n
+    off = st.batch_index(l) * st.stride_l + m * st.stride_m + n * st.stride_n
     return flat[off.reshape(-1)].reshape(L, M, N).to(torch.float32)
 
 
@@ -104,6 +104,15 @@ def interpret(ir, accum: torch.Tensor, slot_tensors: Dict[int, torch.Tensor]) ->
                        else ((x - mean) ** 2).sum(dim, keepdim=True))
             else:
                 raise NotImplementedError(r.kind)
+            if getattr(r, "fold", ""):
+                # batches that share a result are reduced together; every one of them then carries the total
+                if r.kind not in ("sum", "max"):
+                    raise NotImplementedError(f"folded {r.kind}")
+                cnt = r.fold_count
+                grouped = out.view(cnt, L // cnt, M, 1) if r.fold == "mod" else out.view(L // cnt, cnt, M, 1)
+                axis = 0 if r.fold == "mod" else 1
+                tot = grouped.sum(axis, keepdim=True) if r.kind == "sum" else grouped.amax(axis, keepdim=True)
+                out = tot.expand_as(grouped).reshape(L, M, 1)
             val[name] = out
         else:
             val[name] = _apply(node.op, [val[i] for i in node.inputs])
@@ -115,7 +124,7 @@ def interpret(ir, accum: torch.Tensor, slot_tensors: Dict[int, torch.Tensor]) ->
         slot = ir.slots[s.slot]
         st = slot.strides
         v = val[s.input].expand(L, M, N)
-        off = ((l // st.l_div) * st.stride_l + m * st.stride_m + n * st.stride_n).expand(L, M, N)
+        off = (st.batch_index(l) * st.stride_l + m * st.stride_m + n * st.stride_n).expand(L, M, N)
         size = int(off.max()) + 1
         buf = torch.zeros(size, dtype=torch.float32)
         buf[off.reshape(-1)] = v.reshape(-1)

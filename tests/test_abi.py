@@ -43,17 +43,17 @@ def test_every_built_module_exports_the_abi():
         for sym in declared_symbols():
             assert hasattr(lib, sym), f"{p.name} lacks {sym}"
         lib.evt_abi_version.restype = ctypes.c_int
-        assert lib.evt_abi_version() == 1
+        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 2
         lib.evt_module_spec.restype = ctypes.c_char_p
         spec = json.loads(lib.evt_module_spec().decode())
-        assert spec["abi"] == 1 and spec["element"] in ("f16", "bf16") and "tile" in spec
+        assert spec["abi"] == 2 and spec["element"] in ("f16", "bf16") and "tile" in spec
 
 
 def test_struct_layout_matches_header():
-    # EvtTensorArg: pointer + 4 x int64 ; EvtArgs: 4 x int32, 2 x (ptr, int64, int64), 2 x int32, arrays
-    assert ctypes.sizeof(jit.EvtTensorArg) == 40
-    assert ctypes.sizeof(jit.EvtArgs) == 16 + 48 + 8 + 16 * 40 + 16 * 4
-    assert jit.EvtArgs.tensors.offset == 72 and jit.EvtArgs.scalars.offset == 72 + 640
+    # EvtTensorArg: pointer + 5 x int64 ; EvtArgs: 4 x int32, 2 x (ptr, int64, int64), 2 x int32, arrays
+    assert ctypes.sizeof(jit.EvtTensorArg) == 48
+    assert ctypes.sizeof(jit.EvtArgs) == 16 + 48 + 8 + 16 * 48 + 16 * 4
+    assert jit.EvtArgs.tensors.offset == 72 and jit.EvtArgs.scalars.offset == 72 + 768
 
 
 def test_module_spec_describes_slots(module):
@@ -89,6 +89,8 @@ def test_argument_validation_happens_before_launch(module):
     bad = _args(op, km); bad.lda += 1
     assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -2
     bad = _args(op, km); bad.tensors[0].l_div = 0
+    assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -1
+    bad = _args(op, km); bad.tensors[0].l_mod = -3
     assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -1
     # a reduction module needs its workspace
     big = _args(op, km); big.N = 4096; big.ldb = 4096

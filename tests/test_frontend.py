@@ -73,7 +73,7 @@ def test_operand_layouts_follow_permutes():
     assert (b1.target.b_kc, b1.target.ldb, b1.target.bsb) == (False, 2048, 64)
 
 
-SMALL_PATTERNS = ["mm2", "mm3", "mm4", "mm5", "mm9", "bmm1", "bmm3"]
+SMALL_PATTERNS = ["mm2", "mm3", "mm4", "mm5", "mm9", "bmm1", "bmm3"]   # (bmm2 has its own test below)
 
 
 @pytest.mark.parametrize("name", SMALL_PATTERNS)
@@ -83,19 +83,35 @@ def test_reference_patterns_lower_correctly(name):
     _check(cls, inputs)
 
 
-def test_bmm_partition2_is_fused_up_to_its_cross_batch_sum():
-    """bmm.py:48-67: the store through permute/view/clone is fused; the sum over
-    the sequence axis and half of the batch axis stays outside the kernel."""
-    from evt_ae_amd.evt_fuser import target_name
+def test_batch_folded_row_reductions_lower_correctly():
+    """bmm.py:48-67 (sum over the sequence axis and over the batches that agree
+    modulo 16) and a sum over pairs of consecutive batches: one fused kernel
+    each, the fold recorded in the IR and in the output tensor's batch term."""
     inputs = W.pattern_inputs("bmm2")
-    gm = W.fuse(W.BMMPartition2(), inputs)
+    gm = _check(W.BMMPartition2, inputs)
     (n,) = fused_nodes(gm)
-    assert [(s.role, s.kind) for s in n.target.ir.slots] == [("store", "aux")]
-    assert "sum" in {target_name(x.target) for x in gm.graph.nodes if x.op == "call_function"}
-    got = run_emulated(gm, inputs)
-    ref = evt_oracle.eval_fp32(W.BMMPartition2(), inputs)
-    assert evt_oracle.max_rel_err(got[0].float(), ref[0]) <= 5e-3
-    assert torch.allclose(got[1].float(), ref[1], atol=2e-1)      # eager fp16 tail, the reference's criterion
+    (red,) = n.target.ir.reduces.values()
+    assert (red.axis, red.fold, red.fold_step, red.fold_count) == ("row", "mod", 16, 2)
+    (st,) = [s.strides for s in n.target.ir.slots if s.domain == "row"]
+    assert (st.l_mod, st.l_div, st.stride_l, st.stride_m, st.stride_n) == (16, 1, 64, 1, 0)
+
+    gm = _check(W.FoldConsecutiveBatches, W.fold_consecutive_inputs())
+    (n,) = fused_nodes(gm)
+    (red,) = n.target.ir.reduces.values()
+    assert (red.fold, red.fold_count) == ("div", 2)
+
+
+def test_fit_strides_batch_terms():
+    from evt_ae_amd.ir import Coord, accum_coord, fit_strides
+    L, M, N = 12, 5, 7
+    c = accum_coord(L, M, N, True)
+    assert fit_strides(c, L, M, N).l_mod == 0
+    per_head = c.reshape((3, 4, M, N)).reduce([0, 3], False)      # l = b*4 + h, reduced over b and n -> [h, m]
+    st = fit_strides(per_head, L, M, N)
+    assert (st.l_mod, st.l_div, st.stride_l, st.stride_m, st.stride_n) == (4, 1, M, 1, 0)
+    per_group = c.reshape((3, 4, M, N)).reduce([1, 3], False)     # reduced over h and n -> [b, m]
+    st = fit_strides(per_group, L, M, N)
+    assert (st.l_mod, st.l_div, st.stride_l, st.stride_m, st.stride_n) == (0, 4, M, 1, 0)
 
 
 def test_reference_patterns_shrunk():

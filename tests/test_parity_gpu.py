@@ -125,11 +125,9 @@ def test_reference_fuser_patterns(name):
     eager = list(eager) if isinstance(eager, (tuple, list)) else [eager]
     torch.cuda.synchronize()
     refs = evt_oracle.eval_fp32(cls(), inputs)
-    for i, (o, e, r) in enumerate(zip(outs, eager, refs)):
+    for o, e, r in zip(outs, eager, refs):
         assert tuple(o.shape) == tuple(e.shape)
         assert torch.allclose(o.float(), e.float(), atol=PATTERN_ATOL, rtol=1e-2)
-        if name == "bmm2" and i == 1:
-            continue    # produced by eager fp16 kernels from the fused kernel's fp16 output, not by the epilogue
         err = evt_oracle.max_rel_err(o, r)
         assert err <= FP16_TOL, f"{name}: max rel err {err:.3e}"
 
@@ -190,6 +188,26 @@ def test_random_fuser_patterns(name):
         assert not torch.equal(masks[0], masks[1])
         keep = masks[0].float().mean().item()          # the reference's criterion (dropout.py:73-75)
         assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
+
+
+@pytest.mark.parametrize("two_kernel", [False, True])
+def test_batch_folded_row_reductions(two_kernel, monkeypatch):
+    """Per-row reductions that also fold batches: modulo (bmm.py partition 2 at a
+    reduced size) and consecutive groups, with phase 2 inside the kernel and in
+    the finalize kernel."""
+    if two_kernel:
+        monkeypatch.setenv("EVT_TWO_KERNEL_REDUCE", "1")
+    cases = [(W.FoldConsecutiveBatches, W.fold_consecutive_inputs()), (W.BMMPartition2, W.pattern_inputs("bmm2"))]
+    for cls, inputs in cases:
+        gm = W.fuse(cls(), inputs)
+        (node,) = fused_nodes(gm)
+        assert any(r.fold for r in node.target.ir.reduces.values())
+        outs = list(gm(*[t.cuda() for t in inputs]))
+        again = list(gm(*[t.cuda() for t in inputs]))
+        refs = evt_oracle.eval_fp32(cls(), inputs)
+        for o, o2, r in zip(outs, again, refs):
+            assert torch.equal(o, o2)
+            assert evt_oracle.max_rel_err(o, r) <= FP16_TOL
 
 
 def test_launch_is_graph_capturable():
