@@ -481,7 +481,10 @@ class EVTFuser:
         return False
 
     # -- tracing ------------------------------------------------------------------
-    def trace(self, graph_module: GraphModule, partition_: Sequence[str]):
+    def trace(self, graph_module: GraphModule, partition_: Sequence[str], dry_run: bool = False):
+        """Lower one partition to a fused kernel and splice it into the graph.
+        With `dry_run` the analysis runs (and raises NotImplementedError for
+        a partition the epilogue cannot express) but the graph is left alone."""
         self.partition_names = list(partition_)
         try:
             graph_module.graph.lint()
@@ -560,6 +563,8 @@ class EVTFuser:
 
         # Step 5: compose the fused kernel and rewire the graph
         fused_kernel = self.get_fused_node(anchor)
+        if dry_run:
+            return fused_kernel
         args = [i for i in inputs if i is not anchor] + fused_kernel.args
         graph_module.graph.inserting_after(anchor)
         fused_node = graph_module.graph.call_function(fused_kernel, args=tuple(args))

@@ -3,17 +3,18 @@
 Mirror of the call surface of python/gtl/compiler/passes/pass_fusion.py:1383-1385
 (`pass_fusion` -> `Partitioning` -> `EVTFuser.fusible / EVTFuser().trace`,
 :1356-1374).  The reference decides partitions with an ILP over the whole joint
-graph (:216-983); this backend covers the fused GEMM/BMM path only, so the
-partitioner here grows one partition per mm/bmm anchor greedily: operand
-permutes in front of the anchor (main-loop fusion, :1019-1030), then every
-downstream node from FUSIBLE_TGT whose other operands do not depend on the
-anchor, then small broadcast-side expressions that only feed the partition.
-If the fuser rejects a partition (NotImplementedError) the partition is
-shrunk from the end until it is accepted.
+graph (:216-983); this backend lowers the fused GEMM/BMM partitions only, so
+every partition is one mm/bmm anchor, operand permutes in front of it
+(main-loop fusion, :1019-1030), downstream nodes from FUSIBLE_TGT, and small
+broadcast-side expressions that only feed the partition.  Which anchor gets
+which downstream node is decided by the integer program in partitioner.py
+(default) or greedily in graph order.  A partition the fuser rejects
+(NotImplementedError) is shrunk from the end until it is accepted.
 """
 from __future__ import annotations
 
 import operator
+import os
 from typing import List, Sequence, Set
 
 import torch
@@ -51,13 +52,37 @@ def _descendants(anchor: Node) -> Set[Node]:
     return seen
 
 
-def _grow(anchor: Node, taken: Set[Node]) -> List[Node]:
-    part: List[Node] = []
-    # main-loop fusion: a 2-D/3-D permute that only feeds the anchor
+def _mainloop_permutes(anchor: Node, taken: Set[Node]) -> List[Node]:
+    """Main-loop fusion: a permute that only feeds the anchor is read through
+    the operand's strides (reference: pass_fusion.py:773-781, 1019-1030)."""
+    out = []
     for arg in anchor.args[:2]:
         if (isinstance(arg, Node) and arg.op == "call_function" and packet(arg.target) == aten.permute
                 and len(arg.users) == 1 and arg not in taken):
-            part.append(arg)
+            out.append(arg)
+    return out
+
+
+def _absorb_side_expressions(anchor: Node, inside: Set[Node], desc: Set[Node], taken: Set[Node]) -> None:
+    """Broadcast-side expressions (e.g. a mask built from a small tensor) whose
+    every user is inside the partition join it.  They are not downstream of the
+    anchor, so this cannot close a cycle between partitions."""
+    changed = True
+    while changed:
+        changed = False
+        for node in list(inside):
+            for i in node.all_input_nodes:
+                if (i in inside or i in desc or i in taken or i.op != "call_function"
+                        or target_name(i.target) not in _SMALL_SIDE or node is anchor
+                        or (packet(node.target) == aten.permute and anchor in node.users)):
+                    continue
+                if all(u in inside for u in i.users):
+                    inside.add(i)
+                    changed = True
+
+
+def _grow(anchor: Node, taken: Set[Node]) -> List[Node]:
+    part: List[Node] = _mainloop_permutes(anchor, taken)
     part.append(anchor)
     inside = set(part)
     desc = _descendants(anchor)
@@ -85,25 +110,47 @@ def _grow(anchor: Node, taken: Set[Node]) -> List[Node]:
                     if u in inside:
                         inside.discard(u)
                         part.remove(u)
-    # broadcast-side expressions (e.g. a mask built from a small tensor) whose
-    # every user is inside the partition
-    changed = True
-    while changed:
-        changed = False
-        for node in list(inside):
-            for i in node.all_input_nodes:
-                if (i in inside or i in desc or i in taken or i.op != "call_function"
-                        or target_name(i.target) not in _SMALL_SIDE or node is anchor
-                        or (packet(node.target) == aten.permute and anchor in node.users)):
-                    continue
-                if all(u in inside for u in i.users):
-                    inside.add(i)
-                    changed = True
+    _absorb_side_expressions(anchor, inside, desc, taken)
     return [n for n in anchor.graph.nodes if n in inside]
 
 
+def internal_volume_bits(graph_module: GraphModule, partitions: Sequence[Sequence[str]]) -> int:
+    """Bits of the anchor-downstream edges that the partitions keep on chip:
+    the partitioner's objective (reference: pass_fusion.py:518-535)."""
+    from .partitioner import _volume_bits
+    by_name = {n.name: n for n in graph_module.graph.nodes}
+    total = 0
+    for names in partitions:
+        nodes = [by_name[x] for x in names]
+        anchor = next(n for n in nodes if n.op == "call_function" and packet(n.target) in EVTFuser.supported_targets)
+        desc = _descendants(anchor) | {anchor}
+        inside = set(nodes)
+        for j in nodes:
+            if j is anchor or j not in desc:
+                continue
+            for i in j.all_input_nodes:
+                if i in inside and i in desc:
+                    total += _volume_bits(i, j.args[1] if target_name(j.target) == "getitem" else None)
+    return total
+
+
 class Partitioning:
-    """Callable pass object, as in the reference (pass_fusion.py:1185-1380)."""
+    """Callable pass object, as in the reference (pass_fusion.py:1185-1380).
+
+    `strategy="ilp"` (default, or EVT_PARTITIONER) solves one integer program
+    over all anchors of the graph; `"greedy"` grows the anchors one after the
+    other in graph order.  Either way a partition the fuser turns down is
+    shrunk from its end until it is accepted."""
+
+    MAX_RESOLVES = 64
+
+    def __init__(self, strategy: str = None) -> None:
+        self.strategy = strategy or os.environ.get("EVT_PARTITIONER", "ilp")
+        if self.strategy not in ("ilp", "greedy"):
+            raise ValueError(f"unknown partitioning strategy {self.strategy!r}")
+        self.partitions: List[List[str]] = []
+        self.objective_bits = 0
+        self.resolves = 0
 
     def __call__(self, graph_module: GraphModule) -> GraphModule:
         self.call(graph_module)
@@ -114,27 +161,74 @@ class Partitioning:
         graph = graph_module.graph
         anchors = [n for n in graph.nodes
                    if n.op == "call_function" and packet(n.target) in EVTFuser.supported_targets]
+        planned = self.plan_ilp(graph_module, anchors) if self.strategy == "ilp" \
+            else self.plan_greedy(graph_module, anchors)
+        self.objective_bits = internal_volume_bits(graph_module, planned)
+        self.partitions = []
+        for names in planned:
+            EVTFuser().trace(graph_module, names)
+            self.partitions.append(names)
+
+    # -- planning (no graph mutation) ---------------------------------------------
+    @staticmethod
+    def _accepted(graph_module: GraphModule, names: List[str]) -> bool:
+        try:
+            EVTFuser().trace(graph_module, names, dry_run=True)
+            return True
+        except NotImplementedError:
+            return False
+
+    def plan_greedy(self, graph_module: GraphModule, anchors: List[Node]) -> List[List[str]]:
         taken: Set[Node] = set()
-        self.partitions: List[List[str]] = []
+        planned: List[List[str]] = []
         for anchor in anchors:
             if anchor in taken:
                 continue
             part = _grow(anchor, taken)
             names = [n.name for n in part]
-            while True:
-                if not EVTFuser.fusible(names, graph_module):
-                    break
-                try:
-                    EVTFuser().trace(graph_module, names)
-                    self.partitions.append(names)
+            while EVTFuser.fusible(names, graph_module):
+                if self._accepted(graph_module, names):
+                    planned.append(names)
                     taken.update(n for n in part if n.name in names)
                     break
-                except NotImplementedError:
-                    # drop the last epilogue node (never the anchor or its operand permutes)
-                    idx = names.index(anchor.name)
-                    if len(names) - 1 <= idx:
-                        break
-                    names = names[:-1]
+                # drop the last epilogue node (never the anchor or its operand permutes)
+                if len(names) - 1 <= names.index(anchor.name):
+                    break
+                names = names[:-1]
+        return planned
+
+    def plan_ilp(self, graph_module: GraphModule, anchors: List[Node]) -> List[List[str]]:
+        from .partitioner import AnchorPartitionILP
+        reserved = {}
+        for anchor in anchors:
+            for p in _mainloop_permutes(anchor, set(reserved)):
+                reserved[p] = anchor
+        ilp = AnchorPartitionILP(graph_module, anchors, _fusible, reserved)
+        dead: Set[Node] = set()            # anchors the fuser refuses even alone
+        order = list(graph_module.graph.nodes)
+        for self.resolves in range(self.MAX_RESOLVES):
+            assign = ilp.solve()
+            taken = set(reserved) | set(anchors)
+            for s in anchors:
+                taken.update(assign[s])
+            planned, rejected = [], False
+            for s in anchors:
+                if s in dead:
+                    continue
+                inside = {s, *assign[s], *(p for p, a in reserved.items() if a is s)}
+                _absorb_side_expressions(s, inside, ilp._desc[s], taken)
+                names = [n.name for n in order if n in inside]
+                if self._accepted(graph_module, names):
+                    planned.append(names)
+                elif assign[s]:
+                    ilp.ban(assign[s][-1], s)
+                    rejected = True
+                else:
+                    dead.add(s)
+            if not rejected:
+                self.ilp = ilp
+                return planned
+        raise RuntimeError("partitioning did not settle: the fuser kept turning partitions down")
 
     def ensures(self, graph_module: GraphModule) -> None:
         legalize_graph(graph_module)

@@ -52,6 +52,8 @@ def register_all() -> List[jit.LazyModule]:
     for name, (cls, _) in W.RANDOM_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
     W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
+    for name, (cls, _) in W.MULTI_ANCHOR_PATTERNS.items():
+        W.fuse(cls(), _meta(W.pattern_inputs(name)))
     from .passes import pass_decomposition, pass_fusion
     W.fuse(W.Dropout1Undecomposed(), _meta(W.pattern_inputs("dropout1")), passes=[pass_decomposition, pass_fusion])
     from .autotuner.tuner_base import force_tile

@@ -492,6 +492,80 @@ REFERENCE_PATTERNS = {
 }
 
 
+# ---------------------------------------------------------------------------
+# graphs with several anchors: which epilogue takes a shared node is the
+# partitioner's decision (reference: the ILP of pass_fusion.py:216-983)
+# ---------------------------------------------------------------------------
+
+class TwoAnchorsMixedWidth(torch.nn.Module):
+    """z can join either GEMM; joining the second keeps a 32-bit edge on chip,
+    joining the first (what graph order suggests) only a 16-bit one.  y1 and t
+    are results of the graph as well, so neither can be recomputed inside the
+    other GEMM's epilogue: the kernels move 96 M N bits of epilogue tensors
+    with z in the second partition and 112 M N with z in the first."""
+    def forward(self, a, b, c, d):
+        y1 = aten.mm(a, b)
+        y2 = aten.mm(c, d)
+        y2f = aten._to_copy(y2, dtype=torch.float32)
+        t = aten.exp(y2f)
+        z = aten.mul(t, y1)
+        return y1, t, z
+
+
+class CrossedAnchors(torch.nn.Module):
+    """Each GEMM's epilogue candidate needs the other GEMM's result through an
+    op no epilogue can hold: fusing both would make the two kernels wait for
+    each other."""
+    def forward(self, a, b, c, d):
+        y1 = aten.mm(a, b)
+        y2 = aten.mm(c, d)
+        u1 = aten.flip(y1, [1])
+        u2 = aten.flip(y2, [1])
+        e1 = aten.mul(y1, u2)
+        e2 = aten.mul(y2, u1)
+        return e1, e2
+
+
+class ThreeAnchorsDiamond(torch.nn.Module):
+    """Two GEMMs meet in a product that a third GEMM's result scales, followed
+    by a column sum of magnitudes.  (Products and magnitudes rather than sums:
+    tensors that cross from one kernel to the next are rounded to fp16 on the
+    way, and an element-wise relative tolerance is only meaningful where that
+    rounding is not amplified by cancellation.)"""
+    def forward(self, a, b, c, d, e, f, bias):
+        y1 = aten.mm(a, b)
+        y2 = aten.mm(c, d)
+        y3 = aten.mm(e, f)
+        p = aten.add(y1, bias)
+        q = aten.gelu(y2, approximate="tanh")
+        r = aten.mul(p, q)
+        rf = aten._to_copy(r, dtype=torch.float32)
+        s = aten.mul(rf, y3)
+        sa = aten.abs(s)
+        col = aten.sum(sa, [0])
+        return r, s, col
+
+
+_MA = (384, 512, 256)   # M, N, K of every GEMM in the multi-anchor graphs
+
+
+def _ma_inputs(g, n_gemms: int, bias: bool):
+    M, N, K = _MA
+    out = []
+    for _ in range(n_gemms):
+        out += [_h(g, (M, K), 0.25), _h(g, (K, N), 0.25)]
+    if bias:
+        out.append(_h(g, (N,)))
+    return out
+
+
+MULTI_ANCHOR_PATTERNS = {
+    "two_mixed_width": (TwoAnchorsMixedWidth, lambda g: _ma_inputs(g, 2, False)),
+    "crossed": (CrossedAnchors, lambda g: _ma_inputs(g, 2, False)),
+    "three_diamond": (ThreeAnchorsDiamond, lambda g: _ma_inputs(g, 3, True)),
+}
+
+
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
-    return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS[name])[1](g)
+    return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS[name])[1](g)

@@ -287,3 +287,26 @@ def test_bf16_operands():
     out = gm(*[t.cuda() for t in inputs])
     ref = evt_oracle.eval_fp32(wl.module(), inputs)[0]
     assert evt_oracle.max_rel_err(out, ref) <= 4e-2   # bf16 store: 8 mantissa bits
+
+
+@pytest.mark.parametrize("name", list(W.MULTI_ANCHOR_PATTERNS))
+def test_multi_anchor_graphs(name):
+    """Several GEMMs in one graph: the partitioner decides which epilogue takes
+    the nodes they share (reference: pass_fusion.py:216-983), every GEMM becomes
+    one fused launch, and the graph's results match the fp32 oracle.  Tensors
+    that pass from one kernel to the next go through HBM in fp16."""
+    cls, _ = W.MULTI_ANCHOR_PATTERNS[name]
+    inputs = W.pattern_inputs(name)
+    dev = [t.cuda() for t in inputs]
+    gm = W.fuse(cls(), inputs)
+    n_gemms = sum(1 for t in inputs if t.dim() == 2) // 2
+    assert len(fused_nodes(gm)) == n_gemms
+    outs = list(gm(*dev))
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(cls(), inputs)
+    assert len(outs) == len(refs)
+    for k, (o, r) in enumerate(zip(outs, refs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        red = o.dim() == 1
+        err = evt_oracle.max_rel_err(o, r)
+        assert err <= (REDUCTION_TOL if red else FP16_TOL), f"{name} output {k}: max rel err {err:.3e}"
