@@ -20,7 +20,6 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 import torch
 from torch.fx import Node
 from torch.fx.graph_module import GraphModule
-from torch.fx.passes.tools_common import legalize_graph
 from torch.utils._python_dispatch import _len_torch_dispatch_stack, _pop_mode_temporarily
 
 from . import jit
@@ -57,6 +56,56 @@ def node_shape_dtype(node: Node) -> Tuple[Tuple[int, ...], torch.dtype]:
         v = node.meta["val"]
         return tuple(int(s) for s in v.shape), v.dtype
     raise ValueError(f"node {node.name} carries no shape metadata (run ShapeProp first)")
+
+
+def legalize_graph(graph_module: GraphModule) -> GraphModule:
+    """Stable topological sort of the graph, in place: every node is moved
+    behind its latest operand and otherwise keeps its place.  (torch.fx's own
+    legalize_graph sorts breadth first, which interleaves the forward and
+    backward halves of a joint graph; the forward/backward partitioner of
+    AOT autograd goes by node position, as the reference's flow does through
+    `default_partition`, python/gtl/helper/aot_helper.py:24-28.)"""
+    graph = graph_module.graph
+    pos = {n: k for k, n in enumerate(graph.nodes)}
+    pending = list(graph.nodes)
+    placed: set = set()
+    order: List[Node] = []
+    waiting: Dict[Node, List[Node]] = {}
+
+    def place(n: Node):
+        stack = [n]
+        while stack:
+            m = stack.pop()
+            missing = [i for i in m.all_input_nodes if i not in placed]
+            if missing:
+                # wait for the operand that comes last in the present order
+                waiting.setdefault(max(missing, key=pos.__getitem__), []).append(m)
+                continue
+            order.append(m)
+            placed.add(m)
+            stack.extend(reversed(waiting.pop(m, [])))
+
+    for n in pending:
+        place(n)
+    if len(order) != len(pending):
+        rest = [n.name for n in pending if n not in placed]
+        raise RuntimeError("the graph has a cycle through " + ", ".join(rest[:8]))
+    out = [n for n in order if n.op == "output"]
+    order = [n for n in order if n.op != "output"] + out
+    prev = None
+    for n in order:
+        if prev is None:
+            if n.prev is not graph._root:
+                graph._root.append(n)
+        elif n.prev is not prev:
+            prev.append(n)
+        prev = n
+    return graph_module
+
+
+def _tensor_meta(shape: Sequence[int], dtype: torch.dtype):
+    from torch.fx.passes.shape_prop import _extract_tensor_metadata
+    return _extract_tensor_metadata(torch.empty(tuple(shape), dtype=dtype, device="meta"))
 
 
 def _contig_strides(shape: Sequence[int]) -> Tuple[int, ...]:
@@ -568,14 +617,19 @@ class EVTFuser:
         args = [i for i in inputs if i is not anchor] + fused_kernel.args
         graph_module.graph.inserting_after(anchor)
         fused_node = graph_module.graph.call_function(fused_kernel, args=tuple(args))
-        fused_node.meta = {"evt": True}
+        # the forward/backward split of AOT autograd reads these tags and wants
+        # tensor metadata on every tensor-valued node
+        carried = {k: anchor.meta[k] for k in ("partitioner_tag", "seq_nr", "autograd_backward") if k in anchor.meta}
+        fused_node.meta = {"evt": True, **carried}
         graph_module.graph.inserting_after(fused_node)
         for idx, output_node in enumerate(outputs):
             get_item_node = graph_module.graph.call_function(operator.getitem, args=(fused_node, idx))
             graph_module.graph.inserting_after(get_item_node)
-            shape, _ = node_shape_dtype(output_node)
+            shape, dtype = node_shape_dtype(output_node)
+            get_item_node.meta = {"tensor_meta": _tensor_meta(shape, dtype), **carried}
             view_node = graph_module.graph.call_function(aten.view, args=(get_item_node, list(shape)))
-            view_node.meta = {k: v for k, v in output_node.meta.items() if k in ("tensor_meta", "val")}
+            view_node.meta = {k: v for k, v in output_node.meta.items()
+                              if k in ("tensor_meta", "val", "partitioner_tag", "seq_nr", "autograd_backward")}
             if output_node is anchor:
                 for user in list(anchor.users):
                     if user not in epi_set and user is not fused_node:

@@ -19,9 +19,10 @@ from typing import List, Sequence, Set
 
 import torch
 from torch.fx import Graph, GraphModule, Node
-from torch.fx.passes.tools_common import legalize_graph
 
-from .evt_fuser import EVTFuser, packet, target_name
+from .evt_fuser import EVTFuser, legalize_graph, packet, target_name
+from .frontend_passes import (GTLFrontend, inherit_meta, pass_clean_up, pass_cse,  # noqa: F401  (one namespace,
+                              pass_loss_elimination)                                # as gtl.compiler.passes)
 
 aten = torch.ops.aten
 
@@ -247,17 +248,55 @@ def pass_fusion(module: GraphModule, graph: Graph = None):
 # ---------------------------------------------------------------------------
 
 def _repropagate(module: GraphModule) -> None:
-    """Refresh tensor_meta after a rewrite by running the graph on meta tensors
-    shaped like the placeholders (no data, no device)."""
+    """Refresh tensor_meta after a rewrite without touching data: on the fake
+    tensors AOT autograd recorded for the placeholders when there are any (they
+    carry the real device, which `_to_copy(..., device=...)` nodes need), else
+    on meta tensors shaped like the placeholders."""
+    from torch._subclasses.fake_tensor import FakeTensor
     from torch.fx.passes.shape_prop import ShapeProp
+    holders = [n for n in module.graph.nodes if n.op == "placeholder"]
+    vals = [n.meta.get("val") for n in holders]
+    if holders and all(isinstance(v, FakeTensor) for v in vals):
+        class _WithVals(ShapeProp):
+            # AOT autograd reads meta["val"] of whatever becomes a saved activation
+            def run_node(self, n):
+                result = super().run_node(n)
+                n.meta["val"] = result
+                return result
+        _WithVals(module, fake_mode=vals[0].fake_mode).propagate(*vals)
+        return
     metas = []
-    for n in module.graph.nodes:
-        if n.op == "placeholder":
-            tm = n.meta.get("tensor_meta")
-            if tm is None:
-                return      # no shapes recorded: the caller runs ShapeProp itself
-            metas.append(torch.empty(tuple(tm.shape), dtype=tm.dtype, device="meta"))
+    for n in holders:
+        tm = n.meta.get("tensor_meta")
+        if tm is None:
+            return      # no shapes recorded: the caller runs ShapeProp itself
+        metas.append(torch.empty(tuple(tm.shape), dtype=tm.dtype, device="meta"))
     ShapeProp(module).propagate(*metas)
+
+
+def _fold_permutes(graph: Graph) -> bool:
+    """permute(permute(x, p), q) -> permute(x, p o q), or x when that is the
+    identity (the transposes AOT autograd writes around weights come in such
+    pairs; the reference folds them in pass_permute_propagation.py)."""
+    changed = False
+    for node in list(graph.nodes):
+        if node.op != "call_function" or target_name(node.target) != "permute":
+            continue
+        src = node.args[0]
+        if not (isinstance(src, Node) and src.op == "call_function" and target_name(src.target) == "permute"):
+            continue
+        p, q = [int(i) for i in src.args[1]], [int(i) for i in node.args[1]]
+        rank = len(p)
+        comp = [p[i % rank] % rank for i in q]
+        if comp == list(range(rank)):
+            node.replace_all_uses_with(src.args[0])
+            graph.erase_node(node)
+        else:
+            node.args = (src.args[0], comp)
+        if not src.users:
+            graph.erase_node(src)
+        changed = True
+    return changed
 
 
 def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: Sequence[str] = ()):
@@ -275,9 +314,15 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
       threshold_backward(g, y, t)    -> mul(g, gt(y, t))                         (:397-412; the reference
                                         writes ne(y, t), equal on ReLU outputs only)
 
-    The reference's other decompositions (log_softmax, nll_loss, layer / batch
-    norm, convolution, pooling) belong to anchors this backend does not provide
-    and are left untouched."""
+      _log_softmax(x, d, h)          -> log(_softmax(x, d, h))                   (:261-278)
+      _log_softmax_backward_data     -> sub(g, mul(sum(g, d, keepdim), softmax)) (:428-446)
+      nll_loss_backward (2-D, no weight, sum | mean)
+                                     -> mul(mul(neg(one_hot(target)), tangent),
+                                            unsqueeze(ne(target, ignore_index), 1)) [/ batch]   (:294-348;
+                                        the reference compares with -1 instead of ignore_index)
+    and permute(permute(x)) folded into one permute or none.  The reference's
+    other decompositions (layer / batch norm, convolution, pooling, spmm)
+    belong to anchors this backend does not provide and are left untouched."""
     graph = module.graph if graph is None else graph
     disabled = set(disabled_ops)
     changed = False
@@ -287,33 +332,63 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
         name = target_name(node.target)
         if name in disabled:
             continue
+
+        def mk(target, args, kwargs=None, _node=node):
+            # nodes of a replacement stand where the replaced node stood, also
+            # for the forward/backward split of the joint graph
+            return inherit_meta(graph.call_function(target, tuple(args), kwargs or {}), _node)
+
         new = None
         with graph.inserting_before(node):
             if name == "addmm" and len(node.args) == 3 and not node.kwargs:
                 b, x, w = node.args
-                new = graph.call_function(aten.add, (graph.call_function(aten.mm, (x, w)), b))
+                new = mk(aten.add, (mk(aten.mm, (x, w)), b))
             elif name == "t":
-                new = graph.call_function(aten.permute, (node.args[0], [1, 0]))
+                new = mk(aten.permute, (node.args[0], [1, 0]))
             elif name == "transpose" and len(node.args) == 3:
                 rank = len(node.meta["tensor_meta"].shape)
                 dims = list(range(rank))
                 i, j = node.args[1] % rank, node.args[2] % rank
                 dims[i], dims[j] = j, i
-                new = graph.call_function(aten.permute, (node.args[0], dims))
+                new = mk(aten.permute, (node.args[0], dims))
             elif name == "_unsafe_view":
-                new = graph.call_function(aten.view, tuple(node.args))
+                new = mk(aten.view, node.args)
             elif name == "rsub" and len(node.args) == 2 and node.kwargs.get("alpha", 1) == 1:
-                new = graph.call_function(aten.sub, (node.args[1], node.args[0]))
+                new = mk(aten.sub, (node.args[1], node.args[0]))
             elif name == "native_dropout_backward":
                 g, m, s = node.args
-                new = graph.call_function(aten.mul, (graph.call_function(aten.mul, (g, m)), s))
+                new = mk(aten.mul, (mk(aten.mul, (g, m)), s))
             elif name == "threshold_backward":
                 g, y, t = node.args
-                new = graph.call_function(aten.mul, (g, graph.call_function(aten.gt, (y, t))))
+                new = mk(aten.mul, (g, mk(aten.gt, (y, t))))
+            elif name == "_log_softmax" and len(node.args) == 3:
+                x, dim, half_to_float = node.args
+                new = mk(aten.log, (mk(aten._softmax, (x, dim, half_to_float)),))
+            elif name == "_log_softmax_backward_data" and len(node.args) == 4:
+                g, out, dim, _dtype = node.args
+                # d log_softmax: g - softmax * sum(g); softmax is at hand when
+                # `out` is the log(_softmax(x)) written above, else exp(out)
+                if (isinstance(out, Node) and out.op == "call_function" and target_name(out.target) == "log"
+                        and isinstance(out.args[0], Node) and target_name(out.args[0].target) == "_softmax"):
+                    soft = out.args[0]
+                else:
+                    soft = mk(aten.exp, (out,))
+                total = mk(aten.sum, (g, [dim], True))
+                new = mk(aten.sub, (g, mk(aten.mul, (total, soft))))
+            elif name == "nll_loss_backward" and len(node.args) == 7 and node.args[3] is None \
+                    and node.args[4] in (1, 2) and "tensor_meta" in node.args[1].meta:
+                tangent, logp, target, _w, reduction, ignore_index, _total = node.args
+                shape = logp.meta["tensor_meta"].shape
+                if len(shape) == 2:
+                    grad = mk(aten.mul, (mk(aten.neg, (mk(aten.one_hot, (target, int(shape[-1]))),)), tangent))
+                    keep = mk(aten.unsqueeze, (mk(aten.ne, (target, ignore_index)), 1))
+                    new = mk(aten.mul, (grad, keep))
+                    if reduction == 1:       # mean over the batch (labels equal to ignore_index are
+                        new = mk(aten.div, (new, int(shape[0])))     # not discounted, as in the reference)
             elif name == "native_dropout" and len(node.args) == 3 and node.args[2] is True:
                 x, p = node.args[0], node.args[1]
-                mask = graph.call_function(aten.ge, (graph.call_function(torch.rand_like, (x,)), p))
-                out = graph.call_function(aten.mul, (graph.call_function(aten.mul, (x, mask)), 1. / (1 - p)))
+                mask = mk(aten.ge, (mk(torch.rand_like, (x,)), p))
+                out = mk(aten.mul, (mk(aten.mul, (x, mask)), 1. / (1 - p)))
                 for user in list(node.users):     # getitem(dropout, 0 | 1)
                     if user.op == "call_function" and user.target is operator.getitem:
                         user.replace_all_uses_with(out if user.args[1] == 0 else mask)
@@ -323,9 +398,13 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                     changed = True
                 continue
         if new is not None:
+            for k in ("tensor_meta", "val"):     # same value: later rewrites of this sweep read its shape
+                if k in node.meta and k not in new.meta:
+                    new.meta[k] = node.meta[k]
             node.replace_all_uses_with(new)
             graph.erase_node(node)
             changed = True
+    changed = _fold_permutes(graph) or changed
     if changed:
         graph.lint()
         module.recompile()

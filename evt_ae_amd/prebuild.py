@@ -54,6 +54,17 @@ def register_all() -> List[jit.LazyModule]:
     W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
     for name, (cls, _) in W.MULTI_ANCHOR_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    from .aot_helper import aot_capture, evt_backend
+    aot_capture(*W.mlp_classifier())
+    # the same step through torch.compile: Dynamo's graph differs slightly, so
+    # its kernels are registered as well (tracing stops at the first launch
+    # when there is no GPU)
+    model, inputs = W.mlp_classifier()
+    try:
+        torch.compile(model, backend=evt_backend)(*inputs)
+    except RuntimeError as e:
+        if "HIP device only" not in str(e):
+            raise
     from .passes import pass_decomposition, pass_fusion
     W.fuse(W.Dropout1Undecomposed(), _meta(W.pattern_inputs("dropout1")), passes=[pass_decomposition, pass_fusion])
     from .autotuner.tuner_base import force_tile

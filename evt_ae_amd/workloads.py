@@ -566,6 +566,41 @@ MULTI_ANCHOR_PATTERNS = {
 }
 
 
+# ---------------------------------------------------------------------------
+# a whole training step through AOT autograd: the joint graph holds the
+# forward GEMMs (bias + GELU, bias + cast) and the backward ones (data
+# gradient with GELU' and the bias gradient, two weight gradients)
+# ---------------------------------------------------------------------------
+
+class MLPClassifier(torch.nn.Module):
+    """fp16 two-layer classifier with a summed cross-entropy loss, the shape
+    of the reference's XML-CNN head (benchmark/subgraphs/xmlcnn/xmlcnn.py)."""
+    def __init__(self, d_in: int = 256, hidden: int = 1024, classes: int = 128) -> None:
+        super().__init__()
+        self.l1 = torch.nn.Linear(d_in, hidden)
+        self.l2 = torch.nn.Linear(hidden, classes)
+
+    def forward(self, x, y):
+        z = self.l2(torch.nn.functional.gelu(self.l1(x), approximate="tanh"))
+        return torch.nn.functional.cross_entropy(z.float(), y, reduction="sum")
+
+
+MLP_BATCH = 512
+
+
+def mlp_classifier(seed: int = 0, device: str = "cpu", dtype=torch.float16):
+    """(model, (x, labels)) with seeded fp16 parameters and inputs."""
+    g = torch.Generator(device="cpu").manual_seed(0xA07 + seed)
+    model = MLPClassifier()
+    with torch.no_grad():
+        for p in model.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * (0.05 if p.dim() == 2 else 0.02))
+    model = model.to(dtype).to(device)
+    x = torch.randn(MLP_BATCH, model.l1.in_features, generator=g).to(dtype).to(device)
+    y = torch.randint(0, model.l2.out_features, (MLP_BATCH,), generator=g).to(device)
+    return model, (x, y)
+
+
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
     return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS[name])[1](g)

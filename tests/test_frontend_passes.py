@@ -1,0 +1,212 @@
+"""Front-end passes and the AOT-autograd glue without a GPU.
+
+The decompositions are pinned by value: the joint graph after frontend +
+decomposition + CSE (no fusion, so it runs on the CPU) must give the loss and
+the gradients PyTorch's own autograd gives for the same fp32 model.  The
+reference exercises these passes only inside whole-model GPU tests
+(unittest/fx_passes/xmlcnn.py:48-62, 82-89).
+"""
+import operator
+
+import pytest
+import torch
+from torch.fx import symbolic_trace
+
+from evt_ae_amd import workloads as W
+from evt_ae_amd.aot_helper import aot_capture, joint_optimization
+from evt_ae_amd.evt_fuser import legalize_graph, target_name
+from evt_ae_amd.passes import (GTLFrontend, pass_clean_up, pass_cse, pass_decomposition, pass_loss_elimination)
+from evt_ae_amd.workloads import fused_nodes
+
+aten = torch.ops.aten
+
+
+def names_of(gm):
+    return [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+
+
+def without_fusion(joint_module):
+    joint_module, _ = GTLFrontend()(joint_module)
+    pass_decomposition(joint_module, joint_module.graph)
+    pass_cse(joint_module, joint_module.graph)
+    return joint_module
+
+
+@pytest.mark.parametrize("reduction", ["sum", "mean"])
+def test_decomposed_joint_graph_matches_autograd(reduction):
+    class Net(W.MLPClassifier):
+        def forward(self, x, y):
+            z = self.l2(torch.nn.functional.gelu(self.l1(x), approximate="tanh"))
+            return torch.nn.functional.cross_entropy(z, y, reduction=reduction)
+
+    g = torch.Generator().manual_seed(3)
+    model = Net(24, 40, 12)
+    x, y = torch.randn(16, 24, generator=g), torch.randint(0, 12, (16,), generator=g)
+    box = aot_capture(model, (x, y), joint_compiler=without_fusion)
+    ops = set(names_of(box["joint"]))
+    assert not ops & {"addmm", "t", "detach", "_log_softmax", "_log_softmax_backward_data", "nll_loss_backward"}
+    assert {"mm", "permute", "_softmax", "log", "one_hot", "ne", "gelu_backward"} <= ops
+    # run the split graphs by hand: forward returns (loss, *saved), backward takes (*saved, tangent)
+    primals = [p.detach() for p in model.parameters()] + [x, y]
+    fw_out = box["fw"](*primals)
+    loss, saved = fw_out[0], fw_out[1:]
+    grads = box["bw"](*saved, torch.ones_like(loss))
+    ref_loss = model(x, y)
+    ref_grads = torch.autograd.grad(ref_loss, list(model.parameters()))
+    assert torch.allclose(loss, ref_loss, rtol=1e-5, atol=1e-6)
+    got = [t for t in grads if t is not None]
+    assert len(got) == len(ref_grads)
+    for a, b in zip(got, ref_grads):
+        assert a.shape == b.shape
+        assert torch.allclose(a, b, rtol=1e-4, atol=1e-6), float((a - b).abs().max())
+
+
+def test_joint_graph_is_fused_and_split():
+    """Five GEMMs in the training step of the classifier: two in the forward
+    graph (bias + GELU with the pre-activation saved; bias + cast), three in
+    the backward graph (data gradient with GELU' and the bias gradient fused,
+    two weight gradients)."""
+    model, inputs = W.mlp_classifier()
+    box = aot_capture(model, inputs)
+    assert len(fused_nodes(box["joint"])) == 5
+    fw, bw = box["fw"], box["bw"]
+    assert len(fused_nodes(fw)) == 2 and len(fused_nodes(bw)) == 3
+    assert "mm" not in names_of(fw) + names_of(bw) and "addmm" not in names_of(fw)
+    first = fused_nodes(fw)[0].target
+    assert first.ir.epilogue_counts()[1] == 1                       # the bias, broadcast along rows
+    assert len([s for s in first.ir.slots if s.role == "store"]) == 2   # GELU output and pre-activation
+    dgrad = [n.target for n in fused_nodes(bw) if any(s.role == "store" and s.domain != "tile" for s in n.target.ir.slots)]
+    assert len(dgrad) == 1                                           # GELU' and the hidden bias gradient in one launch
+    # no backward node leaked into the forward graph: it only needs the primals
+    assert [n.name for n in fw.graph.nodes if n.op == "placeholder"] == [f"primals_{i}" for i in range(1, 7)]
+
+
+def test_frontend_normalises_targets_views_and_expands():
+    class M(torch.nn.Module):
+        def forward(self, a, b, v):
+            x = torch.ops.aten.add.Tensor(a, b)
+            d = torch.ops.aten.detach.default(x)
+            e = torch.ops.aten.expand.default(v, [4, 6])
+            y = torch.ops.aten.mul.Tensor(d, e)                      # broadcasts by itself: expand goes
+            e2 = torch.ops.aten.expand.default(v, [4, 6])
+            z = torch.ops.aten.mm.default(e2, torch.ops.aten.t.default(y))   # a GEMM operand keeps its expand
+            return torch.ops.aten.view.default(z, [-1, 2])
+
+    gm = W.trace_module(M(), [torch.empty(4, 6), torch.empty(4, 6), torch.empty(1, 6)])
+    gm, modified = GTLFrontend()(gm)
+    assert modified
+    calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+    assert all(not hasattr(n.target, "overloadpacket") for n in calls)          # suffixes gone
+    assert names_of(gm).count("expand") == 1 and "detach" not in names_of(gm)
+    view = [n for n in calls if target_name(n.target) == "view"][0]
+    assert list(view.args[1]) == [8, 2]
+    a, b, v = torch.randn(4, 6), torch.randn(4, 6), torch.randn(1, 6)
+    assert torch.equal(gm(a, b, v), M()(a, b, v))
+
+
+def test_cse_merges_pure_nodes_only():
+    class M(torch.nn.Module):
+        def forward(self, a):
+            p = aten.permute(a, [1, 0])
+            q = aten.permute(a, [1, 0])
+            r1 = torch.rand_like(a)
+            r2 = torch.rand_like(a)
+            return aten.add(p, q), r1, r2
+
+    gm = W.trace_module(M(), [torch.empty(3, 5)])
+    pass_cse(gm)
+    assert names_of(gm).count("permute") == 1 and names_of(gm).count("rand_like") == 2
+    a = torch.randn(3, 5)
+    assert torch.equal(gm(a)[0], 2 * a.t())
+
+
+def test_permute_pairs_fold():
+    class M(torch.nn.Module):
+        def forward(self, w, x):
+            t1 = aten.t(w)
+            t2 = aten.t(t1)
+            p = aten.permute(aten.permute(x, [2, 0, 1]), [0, 2, 1])
+            return aten.mm(t2, t1), p
+
+    gm = W.trace_module(M(), [torch.empty(4, 4), torch.empty(2, 3, 5)])
+    pass_decomposition(gm)
+    perms = [n for n in gm.graph.nodes if n.op == "call_function" and target_name(n.target) == "permute"]
+    assert sorted(list(n.args[1]) for n in perms) == [[1, 0], [2, 1, 0]]
+    w, x = torch.randn(4, 4), torch.randn(2, 3, 5)
+    out = gm(w, x)
+    assert torch.equal(out[0], w @ w.t()) and torch.equal(out[1], x.permute(2, 0, 1).permute(0, 2, 1))
+
+
+def test_clean_up_and_loss_elimination():
+    class M(torch.nn.Module):
+        def forward(self, x, y):
+            p = aten.permute(x, [1, 0])
+            v = aten.view(aten.clone(p, memory_format=torch.contiguous_format), [-1])
+            return aten.sum(aten.mul(v, y)), v
+
+    gm = W.trace_module(M(), [torch.empty(3, 5), torch.empty(15)])
+
+    class N(torch.nn.Module):
+        def forward(self, x):
+            p = aten.permute(x, [1, 0])
+            return aten.view(p, [15])
+
+    gn = symbolic_trace(N())                               # ShapeProp would already trip over the view
+    pass_clean_up(gn)
+    assert names_of(gn) == ["permute", "clone", "view"]
+    x = torch.randn(3, 5)
+    assert torch.equal(gn(x), x.t().reshape(15))            # a view of a permuted tensor would raise
+
+    pass_loss_elimination(gm)
+    assert "sum" not in names_of(gm) and "mul" not in names_of(gm)
+    loss, v = gm(torch.randn(3, 5), torch.randn(15))
+    assert float(loss) == 1.0 and v.shape == (15,)
+
+
+def test_stable_legalize_moves_only_what_it_must():
+    class M(torch.nn.Module):
+        def forward(self, a, b):
+            f1 = aten.add(a, 1.0)
+            f2 = aten.mul(f1, 2.0)
+            g1 = aten.add(b, 1.0)
+            g2 = aten.mul(g1, f2)
+            return f2, g2
+
+    gm = symbolic_trace(M())
+    nodes = {n.name: n for n in gm.graph.nodes}
+    # make f1 read a node that is defined after it
+    with gm.graph.inserting_after(nodes["mul_1"]):
+        late = gm.graph.call_function(aten.neg, (nodes["a"],))
+    nodes["add"].args = (late, 1.0)
+    with pytest.raises(RuntimeError):
+        gm.graph.lint()
+    legalize_graph(gm)
+    gm.graph.lint()
+    order = [n.name for n in gm.graph.nodes]
+    # the dependants of `late` moved behind it, in their old order; b's chain stayed in front
+    assert order == ["a", "b", "add_1", "neg", "add", "mul", "mul_1", "output"]
+    gm.recompile()
+    a, b = torch.randn(3), torch.randn(3)
+    f2, g2 = gm(a, b)
+    assert torch.equal(f2, (-a + 1) * 2) and torch.equal(g2, (b + 1) * f2)
+
+
+def test_aot_optimize_compiles_here_and_refuses_to_run_without_a_gpu():
+    """Forward and backward graphs go through AOT autograd's own checks (saved
+    activations need fake values on the nodes the passes created); the first
+    fused launch then fails loudly: there is no CPU path."""
+    if torch.cuda.is_available():
+        pytest.skip("covered by the GPU training-step test")
+    from evt_ae_amd.aot_helper import aot_optimize
+    model, (x, y) = W.mlp_classifier()
+    with pytest.raises(RuntimeError, match="HIP device only"):
+        aot_optimize(model)(x, y)
+
+
+def test_torch_compile_backend_traces_here():
+    if torch.cuda.is_available():
+        pytest.skip("covered by the GPU training-step test")
+    from evt_ae_amd.aot_helper import evt_backend
+    model, (x, y) = W.mlp_classifier()
+    with pytest.raises(RuntimeError, match="HIP device only"):
+        torch.compile(model, backend=evt_backend)(x, y)
