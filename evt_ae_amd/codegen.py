@@ -122,6 +122,8 @@ class Codegen:
                     vm, vn = True, True
             elif n.op in ("imm", "rres"):
                 vm, vn = False, False
+            elif n.op == "rowval":      # per-row value an anchor hands over (layer norm: mean, rstd)
+                vm, vn = True, False
             else:
                 vm = any(self.var_m[i] for i in n.inputs)
                 vn = any(self.var_n[i] for i in n.inputs)
@@ -655,5 +657,239 @@ class Codegen:
         return e.text()
 
 
-def generate(ir: EpilogueIR, spec: KernelSpec, module_name: str, clock_probe: bool = False) -> str:
+@dataclass(frozen=True)
+class RowSpec:
+    """Row-wise reduce-apply anchor (csrc/evt_rowwise.hpp): which anchor, how a
+    row is spread over a wave, and the element type of the anchor operands.
+    The analogue of the reference's (rows_per_cta, warp_count, cache_input)
+    tuple (python/gtl/compiler/autotuner/softmax_tuner.py)."""
+    op: str             # "softmax" | "softmax_backward" | "layernorm" | "layernorm_backward"
+    ch: int             # chunks of lpr * 8 columns cached per lane
+    lpr: int            # lanes per row (power of two, <= 64)
+    elt: str            # "f16" | "bf16" | "f32"
+
+    OPS = ("softmax", "softmax_backward", "layernorm", "layernorm_backward")
+
+    def tag(self) -> str:
+        return f"{self.op}_{self.elt}_ch{self.ch}_lpr{self.lpr}"
+
+    @property
+    def max_n(self) -> int:
+        return self.ch * self.lpr * 8
+
+    @staticmethod
+    def for_row_length(op: str, n: int, elt: str) -> "RowSpec":
+        """Smallest lane group that holds the row in at most 16 chunks, widened
+        to a full wave once a row needs 4 or more chunks per lane (one row per
+        wave keeps every 16-byte access of a wave inside one row)."""
+        lpr = 8
+        while lpr < 64 and (n + lpr * 8 - 1) // (lpr * 8) > 2:
+            lpr *= 2
+        ch = (n + lpr * 8 - 1) // (lpr * 8)
+        if ch > 16:
+            raise NotImplementedError(f"rows of {n} elements do not fit the register-cached row kernel (max 8192)")
+        return RowSpec(op, ch, lpr, elt)
+
+
+class RowCodegen(Codegen):
+    """EpilogueIR behind a row-wise anchor -> one kernel module with the same
+    five C entry points as the GEMM modules.  The generated `Epi::row()` walks
+    this lane's chunks of 8 columns; values that do not vary along the row are
+    computed once in front of the chunk loop."""
+
+    def __init__(self, ir: EpilogueIR, spec: RowSpec, module_name: str):
+        super().__init__(ir, None, module_name)
+        self.row_spec = spec
+        for r in ir.reduces.values():
+            raise NotImplementedError(f"reduction {r.name} behind a row-wise anchor")
+        for n in ir.nodes.values():
+            if n.op == "colidx" or (n.op == "load" and ir.slots[n.slot].kind == "rand"):
+                raise NotImplementedError(f"{n.op} behind a row-wise anchor")
+
+    def slot_row_off(self, k: int) -> str:
+        return f"o_{k}"
+
+    def emit_row(self, e: _Emitter):
+        ir = self.ir
+        tile_stores = [s for s in ir.stores if s.domain == "tile"]
+        row_stores = [s for s in ir.stores if s.domain == "row"]
+        if len(tile_stores) + len(row_stores) != len(ir.stores):
+            raise NotImplementedError("per-column outputs behind a row-wise anchor")
+        need = ir.closure([s.input for s in ir.stores])
+        outer = [n for n in need if not self.var_n[n]]
+        inner = [n for n in need if self.var_n[n]]
+        e("template <class Cfg, class Ctx>")
+        e("static EVT_DEV void row(const Params& p, const Ctx& t, const float (&acc)[Cfg::CH][8], const float (&rv)[2]) {")
+        e.indent()
+        for k, s in enumerate(ir.slots):
+            e(f"const int64_t o_{k} = (int64_t)evt::batch_index(t.l, p.t{k}_lm, p.t{k}_ld) * p.t{k}_sl + (int64_t)t.m * p.t{k}_sm;")
+        for name in outer:
+            n = ir.nodes[name]
+            c = _cname(name)
+            if n.op == "imm":
+                e(f"const float {c} = p.s[{n.slot}];")
+            elif n.op == "rowval":
+                e(f"const float {c} = rv[{n.comp}];")
+            elif n.op == "load":
+                e(f"const float {c} = evt::ld_f32(p.t{n.slot}, o_{n.slot});")
+            elif n.op == "accum":
+                raise NotImplementedError("accumulator used as a per-row value")
+            else:
+                e(f"const float {c} = {self.expr(n, 'j')};")
+        e("#pragma unroll")
+        e("for (int c = 0; c < Cfg::CH; ++c) {")
+        e.indent()
+        e("const int nv = t.valid(c);")
+        e("if (nv > 0) {")
+        e.indent()
+        e("const int n0 = t.col0(c);")
+        for name in inner:
+            n = ir.nodes[name]
+            c = _cname(name)
+            e(f"float {c}[8];")
+            if n.op == "accum":
+                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = acc[c][j];")
+            elif n.op == "load":
+                k = n.slot
+                e(f"evt::load8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {c});")
+            else:
+                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = {self.expr(n, 'j')};")
+        for s in tile_stores:
+            k = s.slot
+            src = _cname(s.input)
+            if not self.var_n[s.input]:
+                e(f"float b_{k}[8];\n#pragma unroll\nfor (int j = 0; j < 8; ++j) b_{k}[j] = {src};")
+                src = f"b_{k}"
+            e(f"evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
+        e.dedent()
+        e("}")
+        e.dedent()
+        e("}")
+        if row_stores:
+            e("if (t.sub == 0) {")
+            e.indent()
+            for s in row_stores:
+                if self.var_n[s.input]:
+                    raise NotImplementedError("per-row output of a per-element value")
+                e(f"evt::st_f32(p.t{s.slot}, o_{s.slot}, {_cname(s.input)});")
+            e.dedent()
+            e("}")
+        e("(void)p; (void)t; (void)acc; (void)rv;")
+        e.dedent()
+        e("}")
+
+    def module_spec(self) -> dict:
+        sp = self.row_spec
+        return {
+            "abi": 2,
+            "name": self.name,
+            "anchor": sp.op,
+            "row": {"chunks": sp.ch, "lanes_per_row": sp.lpr, "max_n": sp.max_n},
+            "element": sp.elt,
+            "batched": self.ir.batched,
+            "row_state": 0,
+            "col_state": 0,
+            "tensors": [{"name": s.name, "role": s.role, "dtype": s.dtype, "kind": s.kind,
+                         "domain": s.domain} for s in self.ir.slots],
+            "num_scalars": len(self.ir.scalars),
+            "rng_scalars": None,
+            # scalars[anchor_scalars] = eps of a layer norm anchor
+            "anchor_scalars": self.ir.anchor_scalar,
+            # layer norm backward: tensor slots of the forward pass's mean and rstd
+            "anchor_tensors": list(self.ir.anchor_slots),
+        }
+
+    def source(self) -> str:
+        ir, sp = self.ir, self.row_spec
+        op_id = RowSpec.OPS.index(sp.op)
+        elt_id = {"f16": 0, "bf16": 1, "f32": 2}[sp.elt]
+        two = sp.op in ("softmax_backward", "layernorm_backward")
+        stats = sp.op == "layernorm_backward"
+        e = _Emitter()
+        e("// Generated by evt_ae_amd.codegen -- do not edit.")
+        e(f"// module {self.name}")
+        e('#include "evt_rowwise.hpp"')
+        e('#include "evt_amd.h"')
+        e("")
+        e("namespace {")
+        e("struct Epi {")
+        e.indent()
+        self.emit_params(e)
+        self.emit_row(e)
+        e.dedent()
+        e("};")
+        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}>;")
+        e(f"constexpr int kNumTensors = {len(ir.slots)};")
+        e(f"constexpr int kNumScalars = {len(ir.scalars)};")
+        e(f"constexpr int kEltBytes = {4 if sp.elt == 'f32' else 2};")
+        e("int fill(const EvtArgs* a, evt::RowArgs& g, Epi::Params& p) {")
+        e.indent()
+        e("if (!a || !a->A) return EVT_ERR_BAD_ARGS;")
+        if two:
+            e("if (!a->B) return EVT_ERR_BAD_ARGS;")
+        e("if (a->num_tensors != kNumTensors || a->num_scalars != kNumScalars) return EVT_ERR_BAD_ARGS;")
+        e("if (a->M <= 0 || a->N <= 0 || a->L <= 0) return EVT_ERR_BAD_ARGS;")
+        e("if (a->N > Cfg::CH * Cfg::SPAN) return EVT_ERR_RANGE;       // the row must fit this module's register cache")
+        e("if (((int64_t)a->L * a->M + Cfg::ROWS - 1) / Cfg::ROWS > 0x7fffffffLL) return EVT_ERR_RANGE;")
+        e("g.M = a->M; g.N = a->N; g.L = a->L;")
+        e("g.A = (const char*)a->A; g.lda = a->lda; g.bsA = a->batch_stride_A;")
+        e("g.B = (const char*)a->B; g.ldb = a->ldb; g.bsB = a->batch_stride_B;")
+        e("if (a->lda < a->N) return EVT_ERR_BAD_ARGS;")
+        e("g.vecA = (((uintptr_t)a->A | (uintptr_t)(a->lda * kEltBytes) | (uintptr_t)(a->batch_stride_A * kEltBytes)) & 15) == 0;")
+        e("g.vecB = (((uintptr_t)a->B | (uintptr_t)(a->ldb * kEltBytes) | (uintptr_t)(a->batch_stride_B * kEltBytes)) & 15) == 0;")
+        e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0;")
+        e(f"g.eps = {'a->scalars[%d]' % ir.anchor_scalar if ir.anchor_scalar is not None else '0.f'};")
+        if stats:
+            # the forward statistics are two fp32 load slots with one value per row, contiguous over all rows
+            km, kr = ir.anchor_slots[:2]
+            e(f"if (!a->tensors[{km}].ptr || !a->tensors[{kr}].ptr) return EVT_ERR_BAD_ARGS;")
+            e(f"if (a->tensors[{km}].stride_m != 1 || a->tensors[{kr}].stride_m != 1) return EVT_ERR_BAD_ARGS;")
+            e(f"g.mean = (const float*)a->tensors[{km}].ptr; g.rstd = (const float*)a->tensors[{kr}].ptr;")
+            if len(ir.anchor_slots) > 2:     # the weight, applied to the incoming gradient
+                kg = ir.anchor_slots[2]
+                e(f"if (!a->tensors[{kg}].ptr || a->tensors[{kg}].stride_n != 1) return EVT_ERR_BAD_ARGS;")
+                e(f"g.gamma = (const char*)a->tensors[{kg}].ptr; g.vecG = ((uintptr_t)g.gamma & 15) == 0;")
+        for k, s in enumerate(ir.slots):
+            ct = DTYPE_CTYPES[s.dtype]
+            e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
+            e("  if (!x.ptr || x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
+            e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
+            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div; "
+              f"p.t{k}_lm = (int)x.l_mod;")
+            e(f"  p.t{k}_vec = (x.stride_n == 1 && (((uintptr_t)x.ptr | (uintptr_t)(x.stride_m * (int64_t)sizeof({ct})) | "
+              f"(uintptr_t)(x.stride_l * (int64_t)sizeof({ct}))) & 15) == 0) ? 1 : 0; }}")
+        e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
+        e("p.fast = 0;")
+        e("return EVT_OK;")
+        e.dedent()
+        e("}")
+        e("}  // namespace")
+        e("")
+        e('extern "C" int evt_abi_version(void) { return EVT_ABI_VERSION; }')
+        spec_json = json.dumps(self.module_spec(), sort_keys=True)
+        e(f'extern "C" const char* evt_module_spec(void) {{ return R"evtjson({spec_json})evtjson"; }}')
+        e('extern "C" int64_t evt_workspace_bytes(const EvtArgs* a) {')
+        e("  evt::RowArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  return rc != EVT_OK ? rc : 0;      // row-wise anchors keep everything in registers")
+        e("}")
+        e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
+        e("  (void)ws; (void)bytes; (void)stream;")
+        e("  return EVT_OK;")
+        e("}")
+        e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
+        e("  (void)ws; (void)ws_bytes;")
+        e("  evt::RowArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  const unsigned grid = (unsigned)(((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS);")
+        e("  hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  return (int)hipGetLastError();")
+        e("}")
+        return e.text()
+
+
+def generate(ir: EpilogueIR, spec, module_name: str, clock_probe: bool = False) -> str:
+    if isinstance(spec, RowSpec):
+        return RowCodegen(ir, spec, module_name).source()
     return Codegen(ir, spec, module_name, clock_probe).source()

@@ -1,0 +1,297 @@
+// Row-wise reduce-apply anchors: softmax, softmax backward, layer norm and
+// layer norm backward over the last axis, with the same epilogue visitor tree
+// behind them as the GEMM kernels have.
+//
+// Role in the reference (apuaaChen/EVT_AE): src/cuda/softmax, src/cuda/layernorm
+// and src/cuda/reduce_apply (warp-per-row kernels instantiated by
+// SoftmaxOperation / LayerNormOperation with an epilogue visitor,
+// python/gtl/compiler/passes/evt_fuser.py:700-970).
+//
+// MI355X design: HBM-bound, so the only goals are one read of every input,
+// one write of every output, 16-byte accesses and enough rows in flight.  A
+// row lives in the registers of LPR lanes of one wave64 (LPR = 8 .. 64, a
+// power of two; 64 / LPR rows per wave), 8 consecutive columns per lane and
+// chunk, CH chunks (row length <= CH * LPR * 8).  Reductions are xor-shuffles
+// inside the LPR-lane group; nothing goes through LDS and no workgroup barrier
+// is needed, so a workgroup is just 4 independent waves.  The normalised
+// values stay in registers and are handed to the generated epilogue as the
+// "accumulator".
+#pragma once
+
+#include "evt_epilogue.hpp"
+
+namespace evt {
+
+enum RowOp : int { ROW_SOFTMAX = 0, ROW_SOFTMAX_BWD = 1, ROW_LAYERNORM = 2, ROW_LAYERNORM_BWD = 3 };
+
+struct RowArgs {
+  int M, N, L;               // rows per batch, row length, batches (rows are r = l * M + m)
+  const char* A;             // softmax / layer norm: input; backward kernels: incoming gradient
+  int64_t lda, bsA;          // row and batch stride of A in elements
+  const char* B;             // softmax backward: softmax output; layer norm backward: forward input
+  int64_t ldb, bsB;
+  const float* mean;         // layer norm backward: per-row statistics of the forward pass
+  const float* rstd;
+  const char* gamma;         // layer norm backward: weight [N] in the operands' element type, or null
+  int vecG;
+  float eps;                 // layer norm
+  int vecA, vecB;            // rows of A / B may be read with 16-byte loads
+};
+
+// ELT: 0 = f16, 1 = bf16, 2 = f32 element type of the anchor operands
+template <int OP_, int CH_, int LPR_, int ELT_, int WAVES_ = 4>
+struct RowCfg {
+  static constexpr int OP = OP_, CH = CH_, LPR = LPR_, ELT = ELT_, WAVES = WAVES_;
+  static constexpr int THREADS = WAVES * 64;
+  static constexpr int RPW = 64 / LPR;        // rows per wave
+  static constexpr int ROWS = WAVES * RPW;    // rows per workgroup
+  static constexpr int SPAN = LPR * 8;        // columns per chunk
+  static_assert(LPR >= 1 && LPR <= 64 && (LPR & (LPR - 1)) == 0, "lanes per row: a power of two up to 64");
+  static_assert(CH >= 1 && CH <= 16, "a row is cached in at most 128 registers per lane");
+};
+
+template <int ELT> struct RowElt;
+template <> struct RowElt<0> { using type = f16; };
+template <> struct RowElt<1> { using type = bf16; };
+template <> struct RowElt<2> { using type = float; };
+
+template <class Cfg>
+struct RowCtx {
+  int M, N, L;
+  int64_t r;       // global row (clamped to a valid row for lanes past the end; `ok` says which)
+  int l, m;        // batch and row inside the batch
+  int sub;         // lane inside the row's lane group
+  bool ok;
+  EVT_DEV int col0(int c) const { return c * Cfg::SPAN + sub * 8; }
+  EVT_DEV int valid(int c) const {             // how many of this lane's 8 columns of chunk c exist
+    const int v = N - col0(c);
+    return v < 0 ? 0 : (v > 8 ? 8 : v);
+  }
+};
+
+template <int LPR>
+EVT_DEV float group_sum(float x) {
+#pragma unroll
+  for (int s = 1; s < LPR; s <<= 1) x += __shfl_xor(x, s, 64);
+  return x;
+}
+template <int LPR>
+EVT_DEV float group_max(float x) {
+#pragma unroll
+  for (int s = 1; s < LPR; s <<= 1) x = fmaxf(x, __shfl_xor(x, s, 64));
+  return x;
+}
+
+// 8 consecutive elements starting at p[0] (unit stride), `valid` of them inside the row
+template <class T>
+EVT_DEV void load8(const T* p, bool vec, int valid, float fill, float (&out)[8]) {
+  if (vec && valid == 8) {
+    if constexpr (sizeof(T) == 2) {
+      union { uint4 q; T e[8]; } u;
+      u.q = *reinterpret_cast<const uint4*>(p);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out[j] = (float)u.e[j];
+    } else if constexpr (sizeof(T) == 4 && !std::is_same<T, bool>::value) {
+      union { uint4 q[2]; T e[8]; } u;
+      u.q[0] = reinterpret_cast<const uint4*>(p)[0];
+      u.q[1] = reinterpret_cast<const uint4*>(p)[1];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out[j] = (float)u.e[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out[j] = ld_f32<T>(p, j);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = j < valid ? ld_f32<T>(p, j) : fill;
+  }
+}
+
+// generic strided variant for epilogue tensors (element stride sn)
+template <class T>
+EVT_DEV void load8s(const T* p, int64_t sn, bool vec, int valid, float (&out)[8]) {
+  if (sn == 1) {
+    load8<T>(p, vec, valid, 0.f, out);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = j < valid ? ld_f32<T>(p, (int64_t)j * sn) : 0.f;
+  }
+}
+
+template <class T>
+EVT_DEV void store8s(T* p, int64_t sn, bool vec, int valid, const float (&val)[8]) {
+  if (sn == 1 && vec && valid == 8) {
+    if constexpr (sizeof(T) == 2) {
+      union { uint4 q; T e[8]; } u;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) u.e[j] = (T)val[j];
+      *reinterpret_cast<uint4*>(p) = u.q;
+      return;
+    } else if constexpr (sizeof(T) == 4 && !std::is_same<T, bool>::value) {
+      union { uint4 q[2]; T e[8]; } u;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) u.e[j] = (T)val[j];
+      reinterpret_cast<uint4*>(p)[0] = u.q[0];
+      reinterpret_cast<uint4*>(p)[1] = u.q[1];
+      return;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (j < valid) st_f32<T>(p, (int64_t)j * sn, val[j]);
+}
+
+// ---------------------------------------------------------------------------
+// the four anchors: fill acc[CH][8] (and rv[0..1] = per-row values) for row t
+// ---------------------------------------------------------------------------
+template <class Cfg>
+EVT_DEV void row_read(const char* base, int64_t ld, int64_t bs, int vec, const RowCtx<Cfg>& t, float fill,
+                      float (&x)[Cfg::CH][8]) {
+  using T = typename RowElt<Cfg::ELT>::type;
+  const T* row = reinterpret_cast<const T*>(base) + (int64_t)t.l * bs + (int64_t)t.m * ld;
+#pragma unroll
+  for (int c = 0; c < Cfg::CH; ++c) {
+    const int v = t.valid(c);
+    if (v > 0) {
+      load8<T>(row + t.col0(c), vec != 0, v, fill, x[c]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[c][j] = fill;
+    }
+  }
+}
+
+template <class Cfg>
+EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, float (&acc)[Cfg::CH][8], float (&rv)[2]) {
+  constexpr int CH = Cfg::CH, LPR = Cfg::LPR;
+  const float rn = 1.f / (float)g.N;
+  if constexpr (Cfg::OP == ROW_SOFTMAX) {
+    // aten._softmax over the last axis: exp(x - max) / sum, all in fp32
+    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, -INFINITY, acc);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) mx = fmaxf(mx, acc[c][j]);
+    mx = group_max<LPR>(mx);
+    const float off = (mx == -INFINITY) ? 0.f : mx * kLog2e;    // a row of -inf gives NaN below, as torch does
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        acc[c][j] = __builtin_amdgcn_exp2f(acc[c][j] * kLog2e - off);
+        s += acc[c][j];
+      }
+    s = group_sum<LPR>(s);
+    const float inv = 1.f / s;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[c][j] *= inv;
+    rv[0] = mx; rv[1] = s;
+  } else if constexpr (Cfg::OP == ROW_SOFTMAX_BWD) {
+    // aten._softmax_backward_data: (g - sum(g * y)) * y
+    float y[CH][8];
+    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, 0.f, acc);
+    row_read<Cfg>(g.B, g.ldb, g.bsB, g.vecB, t, 0.f, y);
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += acc[c][j] * y[c][j];
+    s = group_sum<LPR>(s);
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[c][j] = (acc[c][j] - s) * y[c][j];
+    rv[0] = s; rv[1] = 0.f;
+  } else if constexpr (Cfg::OP == ROW_LAYERNORM) {
+    // aten.native_layer_norm without weight and bias: (x - mean) * rstd, mean, rstd;
+    // two passes over the registers (mean first, then centred squares)
+    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, 0.f, acc);
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += acc[c][j];
+    const float mean = group_sum<LPR>(s) * rn;
+    float q = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int v = t.valid(c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float d = acc[c][j] - mean;
+        acc[c][j] = d;
+        q += j < v ? d * d : 0.f;
+      }
+    }
+    const float rstd = rsqrtf(group_sum<LPR>(q) * rn + g.eps);
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[c][j] *= rstd;
+    rv[0] = mean; rv[1] = rstd;
+  } else {
+    // aten.native_layer_norm_backward, input gradient, without weight:
+    //   xh = (x - mean) rstd ;  dx = rstd (g - mean_n(g) - xh mean_n(g xh))
+    //   (g already multiplied by the weight when there is one)
+    float xh[CH][8];
+    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, 0.f, acc);
+    if (g.gamma) {
+      using T = typename RowElt<Cfg::ELT>::type;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int v = t.valid(c);
+        if (v > 0) {
+          float w[8];
+          load8<T>(reinterpret_cast<const T*>(g.gamma) + t.col0(c), g.vecG != 0, v, 0.f, w);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[c][j] *= w[j];
+        }
+      }
+    }
+    row_read<Cfg>(g.B, g.ldb, g.bsB, g.vecB, t, 0.f, xh);
+    const float mean = g.mean[t.r], rstd = g.rstd[t.r];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int v = t.valid(c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        xh[c][j] = j < v ? (xh[c][j] - mean) * rstd : 0.f;
+        s1 += acc[c][j];
+        s2 += acc[c][j] * xh[c][j];
+      }
+    }
+    s1 = group_sum<LPR>(s1) * rn;
+    s2 = group_sum<LPR>(s2) * rn;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[c][j] = rstd * (acc[c][j] - s1 - xh[c][j] * s2);
+    rv[0] = mean; rv[1] = rstd;
+  }
+}
+
+template <class Cfg, class Epi>
+__global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typename Epi::Params p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  RowCtx<Cfg> t;
+  t.M = g.M; t.N = g.N; t.L = g.L;
+  t.sub = lane % Cfg::LPR;
+  const int64_t rows = (int64_t)g.L * g.M;
+  const int64_t r = ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW + lane / Cfg::LPR;
+  t.ok = r < rows;
+  t.r = t.ok ? r : rows - 1;      // lanes past the end recompute the last row and store nothing
+  t.l = (int)(t.r / g.M);
+  t.m = (int)(t.r % g.M);
+  float acc[Cfg::CH][8];
+  float rv[2];
+  row_main<Cfg>(g, t, acc, rv);
+  if (t.ok) Epi::template row<Cfg>(p, t, acc, rv);
+}
+
+}  // namespace evt

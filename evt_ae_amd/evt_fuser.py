@@ -25,7 +25,7 @@ from torch.utils._python_dispatch import _len_torch_dispatch_stack, _pop_mode_te
 from . import jit
 from .autotuner.bmm_tuner import BMMTuner
 from .autotuner.gemm_tuner import MMTuner
-from .codegen import KernelSpec, TileConfig
+from .codegen import KernelSpec, RowSpec, TileConfig
 from .ir import (DTYPE_NAMES, Coord, EpilogueIR, Node as IRNode, Slot, Store, Strides, accum_coord,
                  fit_strides)
 
@@ -153,6 +153,7 @@ class FusedOpBase:
     # -- to be provided by subclasses -----------------------------------------
     module: jit.KernelModule
     problem: Tuple[int, int, int, int]   # M, N, K, L
+    num_anchor_inputs = 2                 # trailing call arguments that belong to the anchor itself
 
     def operands(self, A: torch.Tensor, B: torch.Tensor):
         """-> (A, lda, batch_stride_A, B, ldb, batch_stride_B) ready for the kernel."""
@@ -169,16 +170,24 @@ class FusedOpBase:
         a.M, a.N, a.K, a.L = M, N, K, L
         a.A, a.lda, a.batch_stride_A = A.data_ptr(), lda, bsa
         a.B, a.ldb, a.batch_stride_B = B.data_ptr(), ldb, bsb
+        keep = [A, B]
+        self.fill_epilogue_arguments(a, keep, visitor_args, args)
+        return a, keep
+
+    def fill_epilogue_arguments(self, a: jit.EvtArgs, keep: list, visitor_args: Dict[str, torch.Tensor], args) -> None:
+        """Tensor and scalar slots of the epilogue (shared by every anchor)."""
         a.num_tensors = len(self.ir.slots)
         a.num_scalars = len(self.ir.scalars)
-        keep = [A, B]
         for k, slot in enumerate(self.ir.slots):
             ta = a.tensors[k]
             if slot.kind == "rand":      # generated in the kernel: strides only
                 ta.ptr = None
             else:
                 kind, ref = self.slot_sources[k]
-                t = args[ref] if kind == "input" else visitor_args[ref]
+                if kind == "anchor":
+                    t = args[len(args) - self.num_anchor_inputs + ref]
+                else:
+                    t = args[ref] if kind == "input" else visitor_args[ref]
                 keep.append(t)
                 ta.ptr = t.data_ptr()
             ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
@@ -194,7 +203,6 @@ class FusedOpBase:
             bits[r + 2], bits[r + 3] = self.rand_offset & 0xFFFFFFFF, 0
             self.last_rand_state = (self.rand_seed, self.rand_offset & 0xFFFFFFFF)
             self.rand_offset += 1
-        return a, keep
 
     def workspace_for(self, a: jit.EvtArgs, stream, device) -> Tuple[int, int]:
         """Device workspace for cross-workgroup reductions, one per stream,
@@ -289,7 +297,7 @@ class FusedOpBase:
         relative error and the atol / rtol pass rates.  Returns one record per
         output; nothing is raised (the reference prints and drops into a
         debugger)."""
-        accum = self.anchor_eager(args[-2], args[-1])
+        accum = self.anchor_eager(*args[len(args) - self.num_anchor_inputs:])
         named = dict(zip(self.input_names, args[:len(self.input_names)]))
         inputs = {n.name: named[n.name] for n in self.reference_module.graph.nodes
                   if n.op == "placeholder" and n.name != "accum"}
@@ -492,11 +500,89 @@ def _unsupported_anchor(name: str, where: str):
 
 FusedConvFprop = _unsupported_anchor("FusedConvFprop", "282-365")
 FusedConvDgrad = _unsupported_anchor("FusedConvDgrad", "368-450")
-FusedSoftmax = _unsupported_anchor("FusedSoftmax", "700-762")
-FusedSoftmaxBackward = _unsupported_anchor("FusedSoftmaxBackward", "765-826")
-FusedLayerNorm = _unsupported_anchor("FusedLayerNorm", "829-902")
-FusedLayerNormBackward = _unsupported_anchor("FusedLayerNormBackward", "905-970")
 FusedSpmm = _unsupported_anchor("FusedSpmm", "973-1035")
+
+class FusedRowOp(FusedOpBase):
+    """Common part of the row-wise reduce-apply anchors (softmax, layer norm
+    and their backward passes over the last axis): `fused(*epilogue_inputs,
+    *anchor_operands)`.  The anchor's result takes the place of the GEMM
+    accumulator in front of the same epilogue tree; rows are r = l * M + m of
+    the operand viewed as [L, M, N]."""
+
+    row_op = ""
+
+    def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
+        super().__init__(node, epilogue_visitor)
+        v = epilogue_visitor
+        self.args = list(v.anchor_operands)
+        self.num_anchor_inputs = len(self.args)
+        _, dtype = node_shape_dtype(self.args[0])
+        if dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"{self.row_op} operands of dtype {dtype}")
+        self.problem = (v.M, v.N, 1, v.L)
+        self.row_spec = RowSpec.for_row_length(self.row_op, v.N, DTYPE_NAMES[dtype])
+        self.spec = self.row_spec
+        self.module = jit.load_module(self.ir, self.row_spec)
+
+    def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args) -> Tuple[jit.EvtArgs, list]:
+        M, N, _, L = self.problem
+        ops = [t.contiguous() for t in args[len(args) - self.num_anchor_inputs:]]
+        a = jit.EvtArgs()
+        a.M, a.N, a.K, a.L = M, N, 1, L
+        a.A, a.lda, a.batch_stride_A = ops[0].data_ptr(), N, M * N
+        if len(ops) > 1:
+            a.B, a.ldb, a.batch_stride_B = ops[1].data_ptr(), N, M * N
+        keep = list(ops)
+        self.fill_epilogue_arguments(a, keep, visitor_args, args)
+        return a, keep
+
+
+class FusedSoftmax(FusedRowOp):
+    """aten._softmax over the last axis + epilogue (reference: evt_fuser.py:700-762)."""
+    __name__ = "cutlass_softmax_with_visitor"
+    target = aten._softmax
+    row_op = "softmax"
+
+    def anchor_eager(self, x):
+        return aten._softmax(x, -1, self.node.args[2])
+
+
+class FusedSoftmaxBackward(FusedRowOp):
+    """aten._softmax_backward_data over the last axis + epilogue (reference: evt_fuser.py:765-826)."""
+    __name__ = "cutlass_softmax_backward_with_visitor"
+    target = aten._softmax_backward_data
+    row_op = "softmax_backward"
+
+    def anchor_eager(self, grad, out):
+        return aten._softmax_backward_data(grad, out, -1, self.node.args[3])
+
+
+class FusedLayerNorm(FusedRowOp):
+    """aten.native_layer_norm over the last axis, without weight and bias (they
+    are epilogue nodes), + epilogue; mean and rstd are per-row outputs
+    (reference: evt_fuser.py:829-902)."""
+    __name__ = "cutlass_layernorm_with_visitor"
+    target = aten.native_layer_norm
+    row_op = "layernorm"
+
+    def anchor_eager(self, x):
+        return aten.native_layer_norm(x, list(self.node.args[1]), None, None, self.node.args[4])
+
+
+class FusedLayerNormBackward(FusedRowOp):
+    """Input gradient of aten.native_layer_norm_backward (output mask
+    [True, False, False]) + epilogue; operands: gradient, forward input, mean,
+    rstd and optionally the weight (reference: evt_fuser.py:905-970)."""
+    __name__ = "cutlass_layernorm_backward_with_visitor"
+    target = aten.native_layer_norm_backward
+    row_op = "layernorm_backward"
+
+    def anchor_eager(self, grad, x, mean, rstd, gamma=None):
+        return aten.native_layer_norm_backward(grad, x, list(self.node.args[2]), mean, rstd, gamma, None,
+                                               [True, False, False])
+
+
+
 
 
 # ---------------------------------------------------------------------------
@@ -508,7 +594,10 @@ class EVTFuser:
     """Entry point: `EVTFuser.fusible(partition, gm)` and
     `EVTFuser().trace(gm, partition)` (reference: evt_fuser.py:1038-1235)."""
 
-    supported_targets = [aten.mm, aten.bmm]
+    supported_targets = [aten.mm, aten.bmm, aten._softmax, aten._softmax_backward_data, aten.native_layer_norm,
+                         aten.native_layer_norm_backward]
+    row_targets = {aten._softmax: FusedSoftmax, aten._softmax_backward_data: FusedSoftmaxBackward,
+                   aten.native_layer_norm: FusedLayerNorm, aten.native_layer_norm_backward: FusedLayerNormBackward}
 
     def __init__(self, element_compute=torch.float32, **kwargs):
         self.element_compute = element_compute
@@ -551,6 +640,14 @@ class EVTFuser:
         if anchor is None:
             raise ValueError("partition holds no supported anchor")
         self.anchor = anchor
+        if packet(anchor.target) in (aten.native_layer_norm, aten.native_layer_norm_backward):
+            # a tuple cannot leave the kernel: the getitems of the anchor always belong to its partition
+            extra = [u for u in anchor.users if u not in partition]
+            if any(u.op != "call_function" or u.target is not operator.getitem for u in extra):
+                raise NotImplementedError(f"{anchor.name}: result used other than through getitem")
+            members = set(partition) | set(extra)
+            partition = [n for n in graph_module.graph.nodes if n in members]
+            self.partition_names = [n.name for n in partition]
         epilogue_partition = [n for n in partition if n is not anchor and anchor not in n.users]
         epi_set = set(epilogue_partition)
 
@@ -573,24 +670,33 @@ class EVTFuser:
         self.reference_gm = self._extract_reference(graph_module, anchor, epilogue_partition, inputs, outputs)
 
         # Step 3: build the IR
-        (ashape, adtype) = node_shape_dtype(anchor)
-        batched = packet(anchor.target) == aten.bmm
-        if batched:
-            L, M, N = ashape
+        tgt = packet(anchor.target)
+        self.anchor_operands: List[Node] = []
+        self.pending_multi: Dict[Node, Dict[int, str]] = {}
+        self.pending_coords: Dict[Node, Dict[int, Coord]] = {}
+        self.anchor_slot_nodes: List[Node] = []
+        self.coords: Dict[Node, Coord] = {}
+        self.ir_name: Dict[Node, str] = {}
+        if tgt in self.row_targets:
+            self._begin_row_anchor(anchor, tgt)
         else:
-            L, (M, N) = 1, ashape
-        self.L, self.M, self.N = L, M, N
-        self.ir = EpilogueIR(L, M, N, batched)
-        self.ir.add_node(IRNode("accum", "accum", domain="tile"))
-        self.coords: Dict[Node, Coord] = {anchor: accum_coord(L, M, N, batched)}
-        self.ir_name: Dict[Node, str] = {anchor: "accum"}
+            (ashape, adtype) = node_shape_dtype(anchor)
+            batched = tgt == aten.bmm
+            if batched:
+                L, M, N = ashape
+            else:
+                L, (M, N) = 1, ashape
+            self.L, self.M, self.N = L, M, N
+            self.ir = EpilogueIR(L, M, N, batched)
+            self.ir.add_node(IRNode("accum", "accum", domain="tile"))
+            self.coords[anchor] = accum_coord(L, M, N, batched)
+            self.ir_name[anchor] = "accum"
         self.full = self._accum_dependents(anchor, epi_set)
         self.load_cache: Dict[Tuple[str, Tuple[int, ...]], str] = {}
         self.input_index = {n: i for i, n in enumerate(x for x in inputs if x is not anchor)}
         self.input_names = [n.name for n in inputs if n is not anchor]
         self.input_nodes = [n for n in inputs if n is not anchor]
         self.slot_sources: Dict[int, Tuple[str, Any]] = {}
-        self.pending_multi: Dict[Node, Dict[int, str]] = {}
 
         for node in epilogue_partition:
             if node in self.full:
@@ -640,6 +746,70 @@ class EVTFuser:
         self.fused_kernel = fused_kernel
         return fused_kernel
 
+    def _begin_row_anchor(self, anchor: Node, tgt) -> None:
+        """Geometry, accumulator and anchor operands of a row-wise anchor: the
+        operand is viewed as [L, M, N] with N its last axis (the reference
+        canonicalises these anchors to rank 3, pass_fusion.py:1187-1342)."""
+        x = anchor.args[0] if tgt is not aten.native_layer_norm_backward else anchor.args[1]
+        shape, dtype = node_shape_dtype(x)
+        rank = len(shape)
+        if rank < 2:
+            raise NotImplementedError(f"{anchor.name}: row-wise anchor on a rank-{rank} tensor")
+        if tgt in (aten._softmax, aten._softmax_backward_data):
+            dim = int(anchor.args[1] if tgt is aten._softmax else anchor.args[2])
+            if dim % rank != rank - 1:
+                raise NotImplementedError(f"{anchor.name}: softmax over an axis other than the last")
+        else:
+            nshape = list(anchor.args[1] if tgt is aten.native_layer_norm else anchor.args[2])
+            if [int(d) for d in nshape] != [int(shape[-1])]:
+                raise NotImplementedError(f"{anchor.name}: layer norm over more than the last axis")
+        N = int(shape[-1])
+        M = int(shape[-2])
+        L = 1
+        for d in shape[:-2]:
+            L *= int(d)
+        batched = rank > 2
+        self.L, self.M, self.N = L, M, N
+        self.ir = EpilogueIR(L, M, N, batched)
+        self.ir.add_node(IRNode("accum", "accum", domain="tile"))
+        full = Coord(tuple(shape), lambda l, m, n: (l * M + m) * N + n)
+        self.coords[anchor] = full
+        if tgt is aten._softmax:
+            self.anchor_operands = [anchor.args[0]]
+            self.ir_name[anchor] = "accum"
+        elif tgt is aten._softmax_backward_data:
+            self.anchor_operands = [anchor.args[0], anchor.args[1]]
+            self.ir_name[anchor] = "accum"
+        elif tgt is aten.native_layer_norm:
+            if anchor.args[2] is not None or anchor.args[3] is not None:
+                raise NotImplementedError(f"{anchor.name}: weight and bias belong in the epilogue "
+                                          "(pass_decomposition splits them off)")
+            self.anchor_operands = [anchor.args[0]]
+            self.ir.add_anchor_scalar(float(anchor.args[4]))
+            self.ir.add_node(IRNode("ln_mean", "rowval", domain="row", comp=0))
+            self.ir.add_node(IRNode("ln_rstd", "rowval", domain="row", comp=1))
+            self.pending_multi[anchor] = {0: "accum", 1: "ln_mean", 2: "ln_rstd"}
+            stat = full.reduce([rank - 1], True)
+            self.pending_coords[anchor] = {1: stat, 2: stat}
+        else:
+            grad, xin, _, mean, rstd, gamma, _beta, mask = anchor.args[:8]
+            if [bool(b) for b in mask] != [True, False, False]:
+                raise NotImplementedError(f"{anchor.name}: only the input gradient is computed (mask [True, False, False])")
+            self.anchor_operands = [grad, xin, mean, rstd] + ([gamma] if gamma is not None else [])
+            for node_, st_, dt_, kind_ in ((mean, Strides(M, 1, 0), "f32", "col"), (rstd, Strides(M, 1, 0), "f32", "col")):
+                if node_shape_dtype(node_)[1] != torch.float32:
+                    raise NotImplementedError(f"{anchor.name}: statistics must be fp32")
+                k = self.ir.add_slot(Slot(node_.name, "load", dt_, "tile", kind_, st_, node_shape_dtype(node_)[0]))
+                self.ir.anchor_slots.append(k)
+            if gamma is not None:
+                gshape, gdtype = node_shape_dtype(gamma)
+                if gdtype != dtype or tuple(gshape) != (N,):
+                    raise NotImplementedError(f"{anchor.name}: weight must be an [N] vector of the operands' dtype")
+                k = self.ir.add_slot(Slot(gamma.name, "load", DTYPE_NAMES[gdtype], "tile", "row", Strides(0, 0, 1), (N,)))
+                self.ir.anchor_slots.append(k)
+            self.anchor_slot_nodes = [mean, rstd] + ([gamma] if gamma is not None else [])
+            self.pending_multi[anchor] = {0: "accum"}
+
     @staticmethod
     def _extract_reference(graph_module: GraphModule, anchor: Node, epilogue_partition, inputs, outputs) -> GraphModule:
         """The epilogue as a module of its own: placeholder `accum` for the anchor's
@@ -674,6 +844,9 @@ class EVTFuser:
         for k, slot in enumerate(self.ir.slots):
             if slot.kind == "rand":
                 self.slot_sources[k] = ("rand", None)
+            elif k in self.ir.anchor_slots:
+                j = self.ir.anchor_slots.index(k)
+                self.slot_sources[k] = ("anchor", self.anchor_operands.index(self.anchor_slot_nodes[j]))
             elif slot.role == "load":
                 node = next(n for n in self.input_nodes if n.name == slot.name)
                 self.slot_sources[k] = ("input", self.input_index[node])
@@ -1153,8 +1326,11 @@ class EVTFuser:
         src, idx = node.args
         if src not in self.pending_multi:
             raise NotImplementedError(f"getitem of {src.name}")
+        if int(idx) not in self.pending_multi[src]:
+            raise NotImplementedError(f"getitem {int(idx)} of {src.name}")
         self.ir_name[node] = self.pending_multi[src][int(idx)]
-        self.coords[node] = Coord(node_shape_dtype(node)[0], self.coords[src].fn)
+        own = self.pending_coords.get(src, {}).get(int(idx))
+        self.coords[node] = own if own is not None else Coord(node_shape_dtype(node)[0], self.coords[src].fn)
         return self.ir_name[node]
 
     # -- layout ops: no data movement, only index bookkeeping -----------------------
@@ -1197,4 +1373,6 @@ class EVTFuser:
             return FusedGEMM(node, self)
         if tgt == aten.bmm:
             return FusedBMM(node, self)
+        if tgt in self.row_targets:
+            return self.row_targets[tgt](node, self)
         raise NotImplementedError()

@@ -321,6 +321,8 @@ class EpilogueIR:
         self.stores: List[Store] = []
         self.scalars: List[float] = []
         self.rng_scalar: Optional[int] = None    # first of the four scalars that carry the rand_like seed / offset
+        self.anchor_scalar: Optional[int] = None  # scalar that carries a row-wise anchor's own constant (layer norm eps)
+        self.anchor_slots: List[int] = []         # load slots the anchor itself reads (layer norm backward: mean, rstd)
         self._imm_count = 0
 
     # -- construction -------------------------------------------------------
@@ -353,6 +355,11 @@ class EpilogueIR:
         k = self.add_slot(Slot(name, "load", "f32", "tile", "rand", strides, tuple(shape)))
         self.add_node(Node(name, "load", domain="tile", slot=k))
         return name
+
+    def add_anchor_scalar(self, value: float) -> int:
+        self.anchor_scalar = len(self.scalars)
+        self.scalars.append(float(value))
+        return self.anchor_scalar
 
     def domain_of(self, names: Sequence[str]) -> str:
         """Join of operand domains.
@@ -428,7 +435,7 @@ class EpilogueIR:
         self.row_state, self.col_state = row_off, col_off
         # drop unused slots (e.g. loads that only fed dead nodes), keep order
         used_slots = sorted({n.slot for n in self.nodes.values() if n.op == "load"} |
-                            {s.slot for s in self.stores})
+                            {s.slot for s in self.stores} | set(self.anchor_slots))
         remap = {old: new for new, old in enumerate(used_slots)}
         self.slots = [self.slots[i] for i in used_slots]
         for n in self.nodes.values():
@@ -436,6 +443,7 @@ class EpilogueIR:
                 n.slot = remap[n.slot]
         for s in self.stores:
             s.slot = remap[s.slot]
+        self.anchor_slots = [remap[k] for k in self.anchor_slots]
         # validation
         for n in self.nodes.values():
             if n.domain == "bad":
@@ -483,6 +491,8 @@ class EpilogueIR:
             "reduces": [[r.name, r.kind, r.axis, r.input, r.state_offset, r.fold] for r in self.reduces.values()],
             "stores": [[s.slot, s.input, s.domain] for s in self.stores],
             "rng_scalar": self.rng_scalar,
+            **({"anchor_scalar": self.anchor_scalar, "anchor_slots": self.anchor_slots}
+               if self.anchor_scalar is not None or self.anchor_slots else {}),
         }
 
     def key(self) -> str:

@@ -13,6 +13,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import json
+import re
 import os
 import sqlite3
 import subprocess
@@ -123,12 +124,27 @@ def _db() -> sqlite3.Connection:
     return con
 
 
+def _included_headers(text: str, seen: Dict[str, bytes]) -> None:
+    for name in re.findall(r'#include\s+"([^"]+)"', text):
+        if name in seen:
+            continue
+        path = next((d / name for d in (CSRC_DIR, INCLUDE_DIR) if (d / name).exists()), None)
+        if path is None:
+            continue
+        seen[name] = path.read_bytes()
+        _included_headers(seen[name].decode(), seen)
+
+
 def module_hash(source: str) -> str:
+    """Digest of everything the binary depends on: the generated source, the
+    compiler flags and the headers it includes (transitively)."""
     h = hashlib.sha256()
     h.update(source.encode())
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for hdr in sorted(CSRC_DIR.glob("*.hpp")) + [INCLUDE_DIR / "evt_amd.h"]:
-        h.update(hdr.read_bytes())
+    seen: Dict[str, bytes] = {}
+    _included_headers(source, seen)
+    for name in sorted(seen):
+        h.update(seen[name])
     return h.hexdigest()[:20]
 
 
@@ -159,11 +175,16 @@ class LazyModule:
     use, so that tracing a graph never needs hipcc or a GPU.  Modules built
     ahead of time (evt_ae_amd.prebuild) are found by their hash."""
 
-    def __init__(self, ir: EpilogueIR, spec: KernelSpec, clock_probe: bool = False):
-        from .codegen import Codegen
+    def __init__(self, ir: EpilogueIR, spec, clock_probe: bool = False):
+        from .codegen import Codegen, RowCodegen, RowSpec
         self.ir, self.kernel_spec = ir, spec
-        self.name = f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}" + ("_probe" if clock_probe else "")
-        cg = Codegen(ir, spec, self.name, clock_probe)
+        if isinstance(spec, RowSpec):
+            self.name = f"evt_row_{ir.key()}_{spec.tag()}"
+            cg = RowCodegen(ir, spec, self.name)
+        else:
+            self.name = (f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}"
+                         + ("_probe" if clock_probe else ""))
+            cg = Codegen(ir, spec, self.name, clock_probe)
         self.source = cg.source()
         self.spec_json = json.dumps(cg.module_spec(), sort_keys=True)
         self.hash = module_hash(self.source)

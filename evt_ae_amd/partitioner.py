@@ -81,6 +81,15 @@ def _volume_bits_meta(tm) -> int:
     return n * _DTYPE_BITS.get(tm.dtype, 32)
 
 
+def same_phase(node: Node, anchor: Node) -> bool:
+    """In a joint forward/backward graph a kernel belongs to one side: a
+    forward anchor that took a backward node into its epilogue would make the
+    forward results wait for the incoming gradients.  AOT autograd tags every
+    node of a joint graph; graphs without tags have one phase."""
+    a, b = node.meta.get("partitioner_tag"), anchor.meta.get("partitioner_tag")
+    return a is None or b is None or a == b
+
+
 class PartitionCache:
     """Solved instances keyed by a digest of the program, in sqlite when
     `EVT_PARTITION_CACHE` names a file (the reference keeps its solutions in the
@@ -161,7 +170,7 @@ class AnchorPartitionILP:
         for j in self.nodes:                      # graph order is topological
             if j not in desc or j in self.anchor_set or j in self.reserved or not self.fusible(j):
                 continue
-            if (j, s) in self.banned:
+            if (j, s) in self.banned or not same_phase(j, s):
                 continue
             ins = j.all_input_nodes
             if not any(i in inside for i in ins):

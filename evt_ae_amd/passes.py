@@ -21,6 +21,7 @@ import torch
 from torch.fx import Graph, GraphModule, Node
 
 from .evt_fuser import EVTFuser, legalize_graph, packet, target_name
+from .partitioner import same_phase
 from .frontend_passes import (GTLFrontend, inherit_meta, pass_clean_up, pass_cse,  # noqa: F401  (one namespace,
                               pass_loss_elimination)                                # as gtl.compiler.passes)
 
@@ -92,7 +93,7 @@ def _grow(anchor: Node, taken: Set[Node]) -> List[Node]:
         if node is anchor:
             after = True
             continue
-        if not after or node in taken or node not in desc or not _fusible(node):
+        if not after or node in taken or node not in desc or not _fusible(node) or not same_phase(node, anchor):
             continue
         ins = node.all_input_nodes
         if not any(i in inside for i in ins):

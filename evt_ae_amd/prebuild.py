@@ -54,6 +54,8 @@ def register_all() -> List[jit.LazyModule]:
     W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
     for name, (cls, _) in W.MULTI_ANCHOR_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    for name, (cls, _) in W.ROW_ANCHOR_PATTERNS.items():
+        W.fuse(cls(), _meta(W.pattern_inputs(name)))
     from .aot_helper import aot_capture, evt_backend
     aot_capture(*W.mlp_classifier())
     # the same step through torch.compile: Dynamo's graph differs slightly, so

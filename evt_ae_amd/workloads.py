@@ -601,6 +601,114 @@ def mlp_classifier(seed: int = 0, device: str = "cpu", dtype=torch.float16):
     return model, (x, y)
 
 
+# ---------------------------------------------------------------------------
+# row-wise anchors: the patterns of the reference's softmax / layer norm fuser
+# tests (unittest/evt_fuser/softmax.py:30-105, softmax_backward.py:30-41,
+# layernorm.py:31-78, layernorm_backward.py:31-55)
+# ---------------------------------------------------------------------------
+
+class SoftmaxAuxStore(torch.nn.Module):      # softmax.py:30-41
+    def forward(self, input):
+        _softmax = aten._softmax(input, -1, False)
+        return aten.view(_softmax, [16384, 512])
+
+
+class SoftmaxAuxLoad(torch.nn.Module):       # softmax.py:43-55
+    def forward(self, input, aux):
+        return aten.add(aten._softmax(input, -1, False), aux)
+
+
+class SoftmaxRowBroadcast(torch.nn.Module):  # softmax.py:57-69
+    def forward(self, input, row):
+        return aten.add(aten._softmax(input, -1, False), row)
+
+
+class SoftmaxScalar(torch.nn.Module):        # softmax.py:71-82
+    def forward(self, input):
+        return aten.mul(aten._softmax(input, -1, False), 2.)
+
+
+class SoftmaxColumnBroadcast(torch.nn.Module):   # softmax.py:99-111
+    def forward(self, input, col):
+        return aten.add(aten._softmax(input, -1, False), col)
+
+
+class SoftmaxRagged(torch.nn.Module):
+    """Rank 4, a row length that is no multiple of 8, fp32 result of fp16 logits, two results."""
+    def forward(self, input, mask):
+        s = aten._softmax(input, -1, True)
+        return s, aten.mul(s, mask)
+
+
+class SoftmaxBackward(torch.nn.Module):      # softmax_backward.py:30-41
+    def forward(self, grad, out):
+        return aten._softmax_backward_data(grad, out, -1, torch.float16)
+
+
+class LayerNormPattern1(torch.nn.Module):    # layernorm.py:31-52
+    def forward(self, add_4, primals_18, primals_19):
+        ln = aten.native_layer_norm(add_4, [1024], None, None, 1e-12)
+        getitem_46 = operator.getitem(ln, 0)
+        getitem_47 = operator.getitem(ln, 1)
+        getitem_48 = operator.getitem(ln, 2)
+        mul_2 = aten.mul(getitem_46, primals_18)
+        add_32 = aten.add(mul_2, primals_19)
+        view_11 = aten.view(add_32, [1024, 1024])
+        return getitem_47, getitem_48, add_32, view_11
+
+
+class LayerNormPattern2(torch.nn.Module):    # layernorm.py:54-78  (permuted result)
+    def forward(self, add_8, primals_36, primals_37):
+        ln = aten.native_layer_norm(add_8, [1024], None, None, 1e-12)
+        getitem_55 = operator.getitem(ln, 0)
+        getitem_56 = operator.getitem(ln, 1)
+        getitem_57 = operator.getitem(ln, 2)
+        mul_5 = aten.mul(getitem_55, primals_36)
+        add_35 = aten.add(mul_5, primals_37)
+        permute_141 = aten.permute(add_35, [1, 0, 2])
+        clone_5 = aten.clone(permute_141, memory_format=torch.contiguous_format)
+        view_33 = aten.view(clone_5, [1024, 1024])
+        return getitem_56, getitem_57, clone_5, view_33
+
+
+class LayerNormBackwardMasked(torch.nn.Module):   # layernorm_backward.py:31-44 without its column sum
+    def forward(self, grad, input, mean, invstd, gamma, beta, ge_1):
+        ln = aten.native_layer_norm_backward(grad, input, [1024], mean, invstd, gamma, beta, [True, False, False])
+        getitem = operator.getitem(ln, 0)
+        mul_42 = aten.mul(getitem, ge_1)
+        mul_43 = aten.mul(mul_42, 1.0)
+        view_282 = aten.view(mul_43, [2048, 1024])
+        return getitem, view_282
+
+
+def _softmax_out(g, shape):
+    return torch.softmax(_h(g, shape).float(), -1).half()
+
+
+def _ln_backward_inputs(g):
+    grad, x = _h(g, (512, 4, 1024)), _h(g, (512, 4, 1024))
+    mean = x.float().mean(-1, keepdim=True)
+    rstd = torch.rsqrt(x.float().var(-1, unbiased=False, keepdim=True) + 1e-5)
+    gamma, beta = _h(g, (1024,)), _h(g, (1024,))
+    keep = torch.rand(x.shape, generator=g) >= 0.5
+    return [grad, x, mean, rstd, gamma, beta, keep]
+
+
+ROW_ANCHOR_PATTERNS = {
+    "softmax_aux_store": (SoftmaxAuxStore, lambda g: [_h(g, (16384, 512))]),
+    "softmax_aux_load": (SoftmaxAuxLoad, lambda g: [_h(g, (16384, 512)), _h(g, (16384, 512))]),
+    "softmax_row_broadcast": (SoftmaxRowBroadcast, lambda g: [_h(g, (16384, 512)), _h(g, (512,))]),
+    "softmax_scalar": (SoftmaxScalar, lambda g: [_h(g, (16384, 512))]),
+    "softmax_column_broadcast": (SoftmaxColumnBroadcast, lambda g: [_h(g, (16384, 512)), _h(g, (16384, 1))]),
+    "softmax_ragged": (SoftmaxRagged, lambda g: [_h(g, (3, 5, 37, 203), 3.0), _h(g, (37, 1))]),
+    "softmax_backward": (SoftmaxBackward, lambda g: [_h(g, (4, 16, 512, 512)), _softmax_out(g, (4, 16, 512, 512))]),
+    "layernorm1": (LayerNormPattern1, lambda g: [_h(g, (512, 2, 1024)) + 1., _h(g, (1024,)), _h(g, (1024,))]),
+    "layernorm2": (LayerNormPattern2, lambda g: [_h(g, (512, 2, 1024)) + 1., _h(g, (1024,)), _h(g, (1024,))]),
+    "layernorm_backward": (LayerNormBackwardMasked, _ln_backward_inputs),
+}
+
+
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
-    return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS[name])[1](g)
+    return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS.get(name)
+            or ROW_ANCHOR_PATTERNS[name])[1](g)

@@ -73,10 +73,25 @@ def philox_rand_like(seed: int, offset: int, salt: int):
         torch.rand_like = orig
 
 
+class _Fp32DtypeFlags(torch.overrides.TorchFunctionMode):
+    """`aten._softmax(x, dim, half_to_float)` and `aten._softmax_backward_data(g, y,
+    dim, input_dtype)` name the fp16 storage type of the graph; on the widened
+    fp32 inputs of the oracle the flags have to say fp32."""
+
+    def __torch_function__(self, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        pk = getattr(func, "overloadpacket", func)
+        if pk is torch.ops.aten._softmax and args[0].dtype == torch.float32:
+            args = (args[0], args[1], False)
+        elif pk is torch.ops.aten._softmax_backward_data and args[0].dtype == torch.float32:
+            args = (args[0], args[1], args[2], torch.float32)
+        return func(*args, **kwargs)
+
+
 def eval_fp32(module: torch.nn.Module, inputs: Sequence[torch.Tensor], rand=None) -> List[torch.Tensor]:
     """Eager fp32 evaluation on CPU of `module` on the (already fp16-rounded) inputs.
     rand = (seed, offset, salt): replay the kernels' random stream for rand_like."""
-    with torch.no_grad(), (philox_rand_like(*rand) if rand is not None else contextlib.nullcontext()):
+    with torch.no_grad(), _Fp32DtypeFlags(), (philox_rand_like(*rand) if rand is not None else contextlib.nullcontext()):
         out = module(*[widen(t.cpu() if isinstance(t, torch.Tensor) else t) for t in inputs])
     if isinstance(out, torch.Tensor):
         out = [out]

@@ -46,7 +46,12 @@ def test_every_built_module_exports_the_abi():
         assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 2
         lib.evt_module_spec.restype = ctypes.c_char_p
         spec = json.loads(lib.evt_module_spec().decode())
-        assert spec["abi"] == 2 and spec["element"] in ("f16", "bf16") and "tile" in spec
+        assert spec["abi"] == 2
+        if "anchor" in spec:      # row-wise reduce-apply module
+            assert spec["anchor"] in ("softmax", "softmax_backward", "layernorm", "layernorm_backward")
+            assert spec["element"] in ("f16", "bf16", "f32") and spec["row"]["max_n"] >= 1
+        else:
+            assert spec["element"] in ("f16", "bf16") and "tile" in spec
 
 
 def test_struct_layout_matches_header():

@@ -240,6 +240,6 @@ def test_unsupported_ops_raise():
 
 def test_stubbed_anchors():
     from evt_ae_amd import evt_fuser
-    for name in ("FusedSoftmax", "FusedLayerNorm", "FusedConvFprop", "FusedSpmm"):
+    for name in ("FusedConvFprop", "FusedConvDgrad", "FusedSpmm"):
         with pytest.raises(NotImplementedError):
             getattr(evt_fuser, name)(None, None)

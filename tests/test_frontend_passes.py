@@ -62,15 +62,19 @@ def test_decomposed_joint_graph_matches_autograd(reduction):
 
 
 def test_joint_graph_is_fused_and_split():
-    """Five GEMMs in the training step of the classifier: two in the forward
-    graph (bias + GELU with the pre-activation saved; bias + cast), three in
-    the backward graph (data gradient with GELU' and the bias gradient fused,
-    two weight gradients)."""
+    """Five GEMMs and a softmax in the training step of the classifier: in the
+    forward graph bias + GELU with the pre-activation saved, bias + cast, and
+    softmax + log (both results leave: one for the loss, one for backward);
+    in the backward graph the data gradient with GELU' and the bias gradient
+    in one launch and two weight gradients.  No kernel mixes forward and
+    backward nodes."""
     model, inputs = W.mlp_classifier()
     box = aot_capture(model, inputs)
-    assert len(fused_nodes(box["joint"])) == 5
+    assert len(fused_nodes(box["joint"])) == 6
     fw, bw = box["fw"], box["bw"]
-    assert len(fused_nodes(fw)) == 2 and len(fused_nodes(bw)) == 3
+    assert len(fused_nodes(fw)) == 3 and len(fused_nodes(bw)) == 3
+    softmax = fused_nodes(fw)[2].target
+    assert type(softmax).__name__ == "FusedSoftmax" and softmax.partition_names == ["_softmax", "log"]
     assert "mm" not in names_of(fw) + names_of(bw) and "addmm" not in names_of(fw)
     first = fused_nodes(fw)[0].target
     assert first.ir.epilogue_counts()[1] == 1                       # the bias, broadcast along rows

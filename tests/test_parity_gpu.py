@@ -14,6 +14,8 @@ from evt_ae_amd.autotuner.tuner_base import force_tile
 from oracle import evt_oracle
 from tests.util import fused_nodes, rand_slot
 
+aten = torch.ops.aten
+
 pytestmark = pytest.mark.gpu
 
 FP16_TOL = 2e-2
@@ -342,3 +344,37 @@ def test_aot_training_step(entry):
             assert err <= 1e-2, f"step {step} {name}: norm-wise error {err:.3e}"
             close = torch.isclose(p.grad, pe.grad, rtol=1e-1).float().mean().item()
             assert close > 0.9, f"step {step} {name}: {close:.3f} of the elements agree with eager fp16"
+
+
+ROW_ATOL = {"softmax": 3e-3, "layernorm": 3e-2}   # the reference's criteria (softmax.py:28, layernorm.py:29)
+
+
+@pytest.mark.parametrize("name", list(W.ROW_ANCHOR_PATTERNS))
+def test_row_anchor_patterns(name):
+    """Softmax / layer norm (forward and backward) as anchors with an epilogue
+    behind them: the patterns of the reference's fuser tests
+    (unittest/evt_fuser/softmax.py, softmax_backward.py, layernorm.py,
+    layernorm_backward.py), one launch each, checked with the reference's
+    absolute tolerance against the module run eagerly and with the parity
+    contract's relative tolerance against the fp32 oracle."""
+    cls, _ = W.ROW_ANCHOR_PATTERNS[name]
+    inputs = W.pattern_inputs(name)
+    dev = [t.cuda() for t in inputs]
+    gm = W.fuse(cls(), inputs)
+    assert len(fused_nodes(gm)) == 1
+    assert not [n for n in gm.graph.nodes if n.op == "call_function"
+                and n.target in (aten._softmax, aten._softmax_backward_data, aten.native_layer_norm,
+                                 aten.native_layer_norm_backward)]
+    outs = gm(*dev)
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    eager = cls()(*dev)
+    eager = list(eager) if isinstance(eager, (tuple, list)) else [eager]
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(cls(), inputs)
+    atol = ROW_ATOL["softmax" if name.startswith("softmax") else "layernorm"]
+    for k, (o, e, r) in enumerate(zip(outs, eager, refs)):
+        assert tuple(o.shape) == tuple(e.shape) and o.dtype == e.dtype, f"{name} output {k}"
+        assert torch.allclose(o.float(), e.float(), atol=atol, rtol=1e-2), f"{name} output {k} vs eager"
+        stat = o.dtype == torch.float32 and o.numel() * 8 <= inputs[0].numel()      # per-row mean / rstd
+        err = evt_oracle.max_rel_err(o, r)
+        assert err <= (REDUCTION_TOL if stat else FP16_TOL), f"{name} output {k}: max rel err {err:.3e}"
