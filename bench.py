@@ -182,6 +182,55 @@ def time_graph(torch, fn, steps, warmup, span):
         return None
 
 
+def bench_row_anchors(torch, W, steps, warmup):
+    """The row-wise anchors (softmax / layer norm, forward and backward) on
+    HBM-sized inputs: microseconds per launch from a HIP graph of rotating
+    buffer sets, algorithmic bytes per second against the 8 TB/s HBM peak, and
+    the same module run eagerly."""
+    out = {}
+    g = torch.Generator(device="cuda").manual_seed(0x50F7)
+    for name, (cls, shapes, nbytes) in W.ROW_BENCH.items():
+        nsets = max(3, -(-(1 << 30) // nbytes))        # more than 1 GiB in rotation: past the 256 MB cache
+        sets = []
+        for _ in range(nsets):
+            ins = []
+            for sh, dt in shapes:
+                t = torch.randn(sh, generator=g, device="cuda", dtype=torch.float32)
+                ins.append(t.to(dt))
+            if name == "softmax_backward":
+                ins[1] = torch.softmax(ins[1].float(), -1).half()
+            if name == "layernorm_backward":
+                x = ins[1].float()
+                ins[2] = x.mean(-1, keepdim=True)
+                ins[3] = torch.rsqrt(x.var(-1, unbiased=False, keepdim=True) + 1e-5)
+                del x
+            sets.append(ins)
+        gm = W.fuse(cls(), sets[0])
+        (node,) = W.fused_nodes(gm)
+        eager = cls()
+        fused_out = gm(*sets[0])
+        eager_out = eager(*sets[0])
+        fo = list(fused_out) if isinstance(fused_out, (tuple, list)) else [fused_out]
+        eo = list(eager_out) if isinstance(eager_out, (tuple, list)) else [eager_out]
+        err = max(float((a.float() - b.float()).abs().max() / b.float().abs().max().clamp_min(1e-30)) for a, b in zip(fo, eo))
+        if not err <= 2e-2:
+            sys.exit(f"bench.py: row anchor {name} disagrees with the eager module (norm-wise error {err:.3e})")
+        del fused_out, eager_out, fo, eo
+        ms = time_graph(torch, lambda i: gm(*sets[i % nsets]), steps, warmup, span=nsets * 2) or \
+            time_loop(torch, lambda i: gm(*sets[i % nsets]), steps, warmup)
+        ms_eager = time_loop(torch, lambda i: eager(*sets[i % nsets]), max(10, steps // 4), 3)
+        out[name] = {"kernel": node.target.module.name, "rows_x_cols": [shapes[0][0][0] * (shapes[0][0][1] if len(shapes[0][0]) == 3 else 1),
+                                                                     shapes[0][0][-1]],
+                     "us": round(ms * 1e3, 2), "alg_bytes": nbytes, "alg_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                     "eager_us": round(ms_eager * 1e3, 2), "speedup_vs_eager": round(ms_eager / ms, 3),
+                     "normwise_err_vs_eager": err, "buffer_sets": nsets}
+        log(f"[bench] row anchor {name}: {out[name]}")
+        del sets, gm
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(torch, W, evt_oracle, cfgs, reps=3):
     """PyTorch fp32 eager evaluation of the same subgraphs on the host cores."""
     torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
@@ -225,6 +274,8 @@ def main():
                     help="timed regions of --steps launches per config; the median is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-row-anchors", dest="row_anchors", action="store_false",
+                    help="skip the bandwidth measurement of the softmax / layer norm anchors (row_anchors in the output)")
     ap.add_argument("--configs", default="1,2,3,4,5")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB streaming kernel (torch.neg, known traffic) so HBM counters can be scaled")
@@ -356,6 +407,7 @@ def main():
                      "us": details[dom]["us"], **clock, "mfma_only": mfma_only},
         "cpu_baseline": cpu,
         "per_config": details,
+        "row_anchors": bench_row_anchors(torch, W, max(20, args.steps // 4), 5) if args.row_anchors else None,
     }
     print(json.dumps(line), flush=True)
 

@@ -705,6 +705,9 @@ class RowCodegen(Codegen):
         for n in ir.nodes.values():
             if n.op == "colidx" or (n.op == "load" and ir.slots[n.slot].kind == "rand"):
                 raise NotImplementedError(f"{n.op} behind a row-wise anchor")
+        # [N] vectors shared by every row (weight, bias, ...): read once per wave, not once per row
+        self.hoisted = [n.name for n in ir.nodes.values() if n.op == "load" and ir.slots[n.slot].kind == "row"
+                        and ir.slots[n.slot].strides.stride_l == 0 and n.slot not in ir.anchor_slots]
 
     def slot_row_off(self, k: int) -> str:
         return f"o_{k}"
@@ -718,8 +721,33 @@ class RowCodegen(Codegen):
         need = ir.closure([s.input for s in ir.stores])
         outer = [n for n in need if not self.var_n[n]]
         inner = [n for n in need if self.var_n[n]]
-        e("template <class Cfg, class Ctx>")
-        e("static EVT_DEV void row(const Params& p, const Ctx& t, const float (&acc)[Cfg::CH][8], const float (&rv)[2]) {")
+        nh = len(self.hoisted)
+        e(f"static constexpr int NH = {nh};   // row vectors kept in registers across the rows of a wave")
+        e("template <class Cfg, bool FAST, class Ctx>")
+        e(f"static EVT_DEV void hoist(const Params& p, const Ctx& t, float (&hz)[{max(nh, 1)}][Cfg::CH][8]) {{")
+        e.indent()
+        if nh:
+            e("#pragma unroll")
+            e("for (int c = 0; c < Cfg::CH; ++c) {")
+            e.indent()
+            e("const int nv = t.valid(c);")
+            e("const int n0 = t.col0(c);")
+            for i, name in enumerate(self.hoisted):
+                k = ir.nodes[name].slot
+                e("if (nv > 0) {")
+                e(f"  if constexpr (FAST) evt::load8v(p.t{k} + n0, hz[{i}][c]);")
+                e(f"  else evt::load8s(p.t{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, hz[{i}][c]);")
+                e("} else {")
+                e(f"  #pragma unroll\n  for (int j = 0; j < 8; ++j) hz[{i}][c][j] = 0.f;")
+                e("}")
+            e.dedent()
+            e("}")
+        e("(void)p; (void)t; (void)hz;")
+        e.dedent()
+        e("}")
+        e("template <class Cfg, bool FAST, class Ctx>")
+        e(f"static EVT_DEV void row(const Params& p, const Ctx& t, const float (&acc)[Cfg::CH][8], const float (&rv)[2], "
+          f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8]) {{")
         e.indent()
         for k, s in enumerate(ir.slots):
             e(f"const int64_t o_{k} = (int64_t)evt::batch_index(t.l, p.t{k}_lm, p.t{k}_ld) * p.t{k}_sl + (int64_t)t.m * p.t{k}_sm;")
@@ -749,9 +777,12 @@ class RowCodegen(Codegen):
             e(f"float {c}[8];")
             if n.op == "accum":
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = acc[c][j];")
+            elif n.op == "load" and name in self.hoisted:
+                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
             elif n.op == "load":
                 k = n.slot
-                e(f"evt::load8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {c});")
+                e(f"if constexpr (FAST) evt::load8v(p.t{k} + o_{k} + n0, {c});")
+                e(f"else evt::load8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {c});")
             else:
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = {self.expr(n, 'j')};")
         for s in tile_stores:
@@ -760,7 +791,8 @@ class RowCodegen(Codegen):
             if not self.var_n[s.input]:
                 e(f"float b_{k}[8];\n#pragma unroll\nfor (int j = 0; j < 8; ++j) b_{k}[j] = {src};")
                 src = f"b_{k}"
-            e(f"evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
+            e(f"if constexpr (FAST) evt::store8v(p.t{k} + o_{k} + n0, {src});")
+            e(f"else evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
         e.dedent()
         e("}")
         e.dedent()
@@ -774,7 +806,7 @@ class RowCodegen(Codegen):
                 e(f"evt::st_f32(p.t{s.slot}, o_{s.slot}, {_cname(s.input)});")
             e.dedent()
             e("}")
-        e("(void)p; (void)t; (void)acc; (void)rv;")
+        e("(void)p; (void)t; (void)acc; (void)rv; (void)hz;")
         e.dedent()
         e("}")
 
@@ -810,6 +842,7 @@ class RowCodegen(Codegen):
         e(f"// module {self.name}")
         e('#include "evt_rowwise.hpp"')
         e('#include "evt_amd.h"')
+        e("#include <stdlib.h>")
         e("")
         e("namespace {")
         e("struct Epi {")
@@ -838,6 +871,7 @@ class RowCodegen(Codegen):
         e("g.vecA = (((uintptr_t)a->A | (uintptr_t)(a->lda * kEltBytes) | (uintptr_t)(a->batch_stride_A * kEltBytes)) & 15) == 0;")
         e("g.vecB = (((uintptr_t)a->B | (uintptr_t)(a->ldb * kEltBytes) | (uintptr_t)(a->batch_stride_B * kEltBytes)) & 15) == 0;")
         e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0;")
+        e(f"g.fast = (g.vecA && {'g.vecB && ' if two else ''}(a->N & 7) == 0) ? 1 : 0;")
         e(f"g.eps = {'a->scalars[%d]' % ir.anchor_scalar if ir.anchor_scalar is not None else '0.f'};")
         if stats:
             # the forward statistics are two fp32 load slots with one value per row, contiguous over all rows
@@ -858,8 +892,15 @@ class RowCodegen(Codegen):
               f"p.t{k}_lm = (int)x.l_mod;")
             e(f"  p.t{k}_vec = (x.stride_n == 1 && (((uintptr_t)x.ptr | (uintptr_t)(x.stride_m * (int64_t)sizeof({ct})) | "
               f"(uintptr_t)(x.stride_l * (int64_t)sizeof({ct}))) & 15) == 0) ? 1 : 0; }}")
+        for name in self.hoisted:
+            k = ir.nodes[name].slot
+            e(f"if (a->tensors[{k}].stride_l != 0 || a->tensors[{k}].stride_m != 0) return EVT_ERR_BAD_ARGS;   // read once per wave")
         e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
-        e("p.fast = 0;")
+        # slots read or written per element (their kind says they vary along the row; strides are run-time values)
+        vec_slots = [k for k, sl in enumerate(ir.slots) if k not in ir.anchor_slots and
+                     ((sl.role == "load" and sl.kind in ("aux", "row")) or (sl.role == "store" and sl.domain == "tile"))]
+        cond = " && ".join(f"p.t{k}_vec" for k in vec_slots) or "1"
+        e(f"p.fast = (g.fast && {cond}) ? 1 : 0;   // every per-element tensor of the epilogue is unit-stride and 16-byte aligned too")
         e("return EVT_OK;")
         e.dedent()
         e("}")
@@ -882,8 +923,15 @@ class RowCodegen(Codegen):
         e("  evt::RowArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  const unsigned grid = (unsigned)(((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS);")
-        e("  hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  // workgroups per CU before waves start walking over several rows (0: one pass, a workgroup per Cfg::ROWS rows);")
+        e("  // walking pays when row vectors are kept in registers across the rows of a wave")
+        e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); return s ? atoi(s) : {16 if (self.hoisted or len(ir.anchor_slots) > 2) else 0}; }}();")
+        e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
+          "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
+        e("  const int64_t want = ((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS;")
+        e("  const unsigned grid = (unsigned)((per_cu <= 0 || want < (int64_t)cus * per_cu) ? want : (int64_t)cus * per_cu);")
+        e("  if (p.fast) hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, true>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  else hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, false>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  return (int)hipGetLastError();")
         e("}")
         return e.text()

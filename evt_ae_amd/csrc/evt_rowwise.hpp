@@ -11,9 +11,10 @@
 // one write of every output, 16-byte accesses and enough rows in flight.  A
 // row lives in the registers of LPR lanes of one wave64 (LPR = 8 .. 64, a
 // power of two; 64 / LPR rows per wave), 8 consecutive columns per lane and
-// chunk, CH chunks (row length <= CH * LPR * 8).  Reductions are xor-shuffles
-// inside the LPR-lane group; nothing goes through LDS and no workgroup barrier
-// is needed, so a workgroup is just 4 independent waves.  The normalised
+// chunk, CH chunks (row length <= CH * LPR * 8).  Reductions run over DPP
+// operands and scalar lane reads inside the LPR-lane group; nothing goes
+// through LDS and no workgroup barrier is needed, so a workgroup is just 4
+// independent waves.  The normalised
 // values stay in registers and are handed to the generated epilogue as the
 // "accumulator".
 #pragma once
@@ -36,6 +37,7 @@ struct RowArgs {
   int vecG;
   float eps;                 // layer norm
   int vecA, vecB;            // rows of A / B may be read with 16-byte loads
+  int fast;                  // N % 8 == 0 and every anchor operand is 16-byte aligned: whole 8-column groups only
 };
 
 // ELT: 0 = f16, 1 = bf16, 2 = f32 element type of the anchor operands
@@ -69,18 +71,42 @@ struct RowCtx {
   }
 };
 
-template <int LPR>
-EVT_DEV float group_sum(float x) {
-#pragma unroll
-  for (int s = 1; s < LPR; s <<= 1) x += __shfl_xor(x, s, 64);
+// All-reduce over the LPR lanes of a row.  Inside a row of 16 lanes the partner
+// values come through DPP operands (quad permutes for lane ^ 1 and lane ^ 2,
+// then the mirrored half row and the mirrored row: by then all lanes of a quad
+// / of 8 hold the same value, so a mirror reaches the other half just as an
+// xor would); the four rows of 16 are combined from scalar lane reads.  No
+// LDS-crossbar shuffle is involved: a reduction costs a few dozen cycles.
+template <int CTRL>
+EVT_DEV float dpp_move(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+EVT_DEV float lane_read(float x, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+struct OpSum { static EVT_DEV float f(float a, float b) { return a + b; } };
+struct OpMax { static EVT_DEV float f(float a, float b) { return fmaxf(a, b); } };
+
+template <int LPR, class Op>
+EVT_DEV float group_reduce(float x) {
+  if constexpr (LPR >= 2) x = Op::f(x, dpp_move<0xB1>(x));     // quad_perm [1,0,3,2]
+  if constexpr (LPR >= 4) x = Op::f(x, dpp_move<0x4E>(x));     // quad_perm [2,3,0,1]
+  if constexpr (LPR >= 8) x = Op::f(x, dpp_move<0x141>(x));    // row_half_mirror
+  if constexpr (LPR >= 16) x = Op::f(x, dpp_move<0x140>(x));   // row_mirror
+  if constexpr (LPR == 32) {
+    const float lo = Op::f(lane_read(x, 0), lane_read(x, 16));
+    const float hi = Op::f(lane_read(x, 32), lane_read(x, 48));
+    x = (threadIdx.x & 32) ? hi : lo;
+  }
+  if constexpr (LPR == 64) {
+    x = Op::f(Op::f(lane_read(x, 0), lane_read(x, 16)), Op::f(lane_read(x, 32), lane_read(x, 48)));
+  }
   return x;
 }
 template <int LPR>
-EVT_DEV float group_max(float x) {
-#pragma unroll
-  for (int s = 1; s < LPR; s <<= 1) x = fmaxf(x, __shfl_xor(x, s, 64));
-  return x;
-}
+EVT_DEV float group_sum(float x) { return group_reduce<LPR, OpSum>(x); }
+template <int LPR>
+EVT_DEV float group_max(float x) { return group_reduce<LPR, OpMax>(x); }
 
 // 8 consecutive elements starting at p[0] (unit stride), `valid` of them inside the row
 template <class T>
@@ -141,33 +167,126 @@ EVT_DEV void store8s(T* p, int64_t sn, bool vec, int valid, const float (&val)[8
     if (j < valid) st_f32<T>(p, (int64_t)j * sn, val[j]);
 }
 
+// whole, aligned 8-column groups (the check-free epilogue path)
+template <class T>
+EVT_DEV void load8v(const T* p, float (&out)[8]) {
+  constexpr int Q = (sizeof(T) * 8 + 15) / 16;
+  union { uint4 q[Q]; T e[8]; } u;
+  if constexpr (sizeof(T) * 8 >= 16) {
+#pragma unroll
+    for (int i = 0; i < Q; ++i) u.q[i] = reinterpret_cast<const uint4*>(p)[i];
+  } else {   // 1-byte elements: one 8-byte load
+    *reinterpret_cast<uint2*>(&u) = *reinterpret_cast<const uint2*>(p);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if constexpr (std::is_same<T, bool>::value) out[j] = u.e[j] ? 1.f : 0.f;
+    else out[j] = (float)u.e[j];
+  }
+}
+template <class T>
+EVT_DEV void store8v(T* p, const float (&val)[8]) {
+  constexpr int Q = (sizeof(T) * 8 + 15) / 16;
+  union { uint4 q[Q]; T e[8]; } u;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if constexpr (std::is_same<T, bool>::value) u.e[j] = val[j] != 0.f;
+    else u.e[j] = (T)val[j];
+  }
+  if constexpr (sizeof(T) * 8 >= 16) {
+#pragma unroll
+    for (int i = 0; i < Q; ++i) reinterpret_cast<uint4*>(p)[i] = u.q[i];
+  } else {
+    *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(&u);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // the four anchors: fill acc[CH][8] (and rv[0..1] = per-row values) for row t
 // ---------------------------------------------------------------------------
+// A row as it comes from memory, still in the operands' element type: fetched one
+// row ahead of the arithmetic, so the conversion (which would wait for the
+// load) happens only when the row is consumed.
 template <class Cfg>
-EVT_DEV void row_read(const char* base, int64_t ld, int64_t bs, int vec, const RowCtx<Cfg>& t, float fill,
-                      float (&x)[Cfg::CH][8]) {
+struct RowRaw {
+  using T = typename RowElt<Cfg::ELT>::type;
+  static constexpr bool TWO = Cfg::OP == ROW_SOFTMAX_BWD || Cfg::OP == ROW_LAYERNORM_BWD;
+  T a[Cfg::CH][8];
+  T b[TWO ? Cfg::CH : 1][8];
+  float mean, rstd;
+};
+
+template <class T>
+EVT_DEV void load8_raw(const T* p, bool vec, int valid, T fill, T (&out)[8]) {
+  if (vec && valid == 8) {
+    constexpr int Q = sizeof(T) * 8 / 16;
+    union { uint4 q[Q]; T e[8]; } u;
+#pragma unroll
+    for (int i = 0; i < Q; ++i) u.q[i] = reinterpret_cast<const uint4*>(p)[i];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = u.e[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = j < valid ? p[j] : fill;
+  }
+}
+
+template <class Cfg, bool FAST>
+EVT_DEV void row_fetch_one(const char* base, int64_t ld, int64_t bs, int vec, const RowCtx<Cfg>& t, float fill,
+                           typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8]) {
   using T = typename RowElt<Cfg::ELT>::type;
   const T* row = reinterpret_cast<const T*>(base) + (int64_t)t.l * bs + (int64_t)t.m * ld;
+  if constexpr (FAST) {
+    // every lane loads 16-byte groups; a lane whose group lies past the row end reads the row's first group
+    // instead (always there) and the value is replaced afterwards: no branch, no partial group
+    constexpr int Q = sizeof(T) * 8 / 16;
+#pragma unroll
+    for (int c = 0; c < Cfg::CH; ++c) {
+      const bool in = t.col0(c) < t.N;
+      union { uint4 q[Q]; T e[8]; } u;
+      const uint4* src = reinterpret_cast<const uint4*>(row + (in ? t.col0(c) : 0));
+#pragma unroll
+      for (int i = 0; i < Q; ++i) u.q[i] = src[i];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[c][j] = in ? u.e[j] : (T)fill;
+    }
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < Cfg::CH; ++c) {
     const int v = t.valid(c);
     if (v > 0) {
-      load8<T>(row + t.col0(c), vec != 0, v, fill, x[c]);
+      load8_raw<T>(row + t.col0(c), vec != 0, v, (T)fill, x[c]);
     } else {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[c][j] = fill;
+      for (int j = 0; j < 8; ++j) x[c][j] = (T)fill;
     }
   }
 }
 
+template <class Cfg, bool FAST>
+EVT_DEV void row_fetch(const RowArgs& g, const RowCtx<Cfg>& t, RowRaw<Cfg>& raw) {
+  row_fetch_one<Cfg, FAST>(g.A, g.lda, g.bsA, g.vecA, t, Cfg::OP == ROW_SOFTMAX ? -INFINITY : 0.f, raw.a);
+  if constexpr (RowRaw<Cfg>::TWO) row_fetch_one<Cfg, FAST>(g.B, g.ldb, g.bsB, g.vecB, t, 0.f, raw.b);
+  if constexpr (Cfg::OP == ROW_LAYERNORM_BWD) { raw.mean = g.mean[t.r]; raw.rstd = g.rstd[t.r]; }
+}
+
 template <class Cfg>
-EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, float (&acc)[Cfg::CH][8], float (&rv)[2]) {
+EVT_DEV void row_widen(const typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8], float (&y)[Cfg::CH][8]) {
+#pragma unroll
+  for (int c = 0; c < Cfg::CH; ++c)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[c][j] = (float)x[c][j];
+}
+
+template <class Cfg>
+EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>& raw, const float (&gz)[Cfg::CH][8],
+                      float (&acc)[Cfg::CH][8], float (&rv)[2]) {
   constexpr int CH = Cfg::CH, LPR = Cfg::LPR;
   const float rn = 1.f / (float)g.N;
   if constexpr (Cfg::OP == ROW_SOFTMAX) {
     // aten._softmax over the last axis: exp(x - max) / sum, all in fp32
-    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, -INFINITY, acc);
+    row_widen<Cfg>(raw.a, acc);
     float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -193,8 +312,8 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, float (&acc)[Cfg::
   } else if constexpr (Cfg::OP == ROW_SOFTMAX_BWD) {
     // aten._softmax_backward_data: (g - sum(g * y)) * y
     float y[CH][8];
-    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, 0.f, acc);
-    row_read<Cfg>(g.B, g.ldb, g.bsB, g.vecB, t, 0.f, y);
+    row_widen<Cfg>(raw.a, acc);
+    row_widen<Cfg>(raw.b, y);
     float s = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -209,7 +328,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, float (&acc)[Cfg::
   } else if constexpr (Cfg::OP == ROW_LAYERNORM) {
     // aten.native_layer_norm without weight and bias: (x - mean) * rstd, mean, rstd;
     // two passes over the registers (mean first, then centred squares)
-    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, 0.f, acc);
+    row_widen<Cfg>(raw.a, acc);
     float s = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -238,22 +357,15 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, float (&acc)[Cfg::
     //   xh = (x - mean) rstd ;  dx = rstd (g - mean_n(g) - xh mean_n(g xh))
     //   (g already multiplied by the weight when there is one)
     float xh[CH][8];
-    row_read<Cfg>(g.A, g.lda, g.bsA, g.vecA, t, 0.f, acc);
+    row_widen<Cfg>(raw.a, acc);
     if (g.gamma) {
-      using T = typename RowElt<Cfg::ELT>::type;
 #pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int v = t.valid(c);
-        if (v > 0) {
-          float w[8];
-          load8<T>(reinterpret_cast<const T*>(g.gamma) + t.col0(c), g.vecG != 0, v, 0.f, w);
+      for (int c = 0; c < CH; ++c)
 #pragma unroll
-          for (int j = 0; j < 8; ++j) acc[c][j] *= w[j];
-        }
-      }
+        for (int j = 0; j < 8; ++j) acc[c][j] *= gz[c][j];
     }
-    row_read<Cfg>(g.B, g.ldb, g.bsB, g.vecB, t, 0.f, xh);
-    const float mean = g.mean[t.r], rstd = g.rstd[t.r];
+    row_widen<Cfg>(raw.b, xh);
+    const float mean = raw.mean, rstd = raw.rstd;
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -275,23 +387,66 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, float (&acc)[Cfg::
   }
 }
 
-template <class Cfg, class Epi>
+// Each wave walks rows first, first + stride, ... (stride = all waves of the
+// grid x rows per wave) and fetches the next row before it reduces the present
+// one, so a wave always has a row's worth of loads in flight; the grid is sized
+// to fill the chip once instead of one workgroup per handful of rows.
+template <class Cfg, class Epi, bool FAST>
 __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typename Epi::Params p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t rows = (int64_t)g.L * g.M;
+  const int64_t stride = (int64_t)gridDim.x * Cfg::ROWS;
   RowCtx<Cfg> t;
   t.M = g.M; t.N = g.N; t.L = g.L;
   t.sub = lane % Cfg::LPR;
-  const int64_t rows = (int64_t)g.L * g.M;
-  const int64_t r = ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW + lane / Cfg::LPR;
-  t.ok = r < rows;
-  t.r = t.ok ? r : rows - 1;      // lanes past the end recompute the last row and store nothing
-  t.l = (int)(t.r / g.M);
-  t.m = (int)(t.r % g.M);
-  float acc[Cfg::CH][8];
-  float rv[2];
-  row_main<Cfg>(g, t, acc, rv);
-  if (t.ok) Epi::template row<Cfg>(p, t, acc, rv);
+  auto locate = [&](int64_t base) {
+    const int64_t r = base + lane / Cfg::LPR;
+    t.ok = r < rows;
+    t.r = t.ok ? r : rows - 1;      // lanes past the end recompute the last row and store nothing
+    t.l = (int)(t.r / g.M);
+    t.m = (int)(t.r % g.M);
+  };
+  int64_t base = ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW;    // wave-uniform
+  if (base >= rows) return;
+  RowRaw<Cfg> cur;
+  locate(base);
+  row_fetch<Cfg, FAST>(g, t, cur);
+  float hz[Epi::NH > 0 ? Epi::NH : 1][Cfg::CH][8];
+  Epi::template hoist<Cfg, FAST>(p, t, hz);
+  float gz[Cfg::CH][8];          // layer norm backward: this lane's columns of the weight, read once
+  if constexpr (Cfg::OP == ROW_LAYERNORM_BWD) {
+    using T = typename RowElt<Cfg::ELT>::type;
+    if (g.gamma) {
+#pragma unroll
+      for (int c = 0; c < Cfg::CH; ++c) {
+        const int v = t.valid(c);
+        if (v > 0) {
+          load8<T>(reinterpret_cast<const T*>(g.gamma) + t.col0(c), g.vecG != 0, v, 0.f, gz[c]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) gz[c][j] = 0.f;
+        }
+      }
+    }
+  }
+  while (true) {
+    const RowCtx<Cfg> here = t;
+    const int64_t next = base + stride;
+    const bool more = next < rows;                                         // wave-uniform
+    RowRaw<Cfg> ahead;
+    if (more) {
+      locate(next);
+      row_fetch<Cfg, FAST>(g, t, ahead);
+    }
+    float acc[Cfg::CH][8];
+    float rv[2];
+    row_main<Cfg>(g, here, cur, gz, acc, rv);
+    if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, hz);
+    if (!more) break;
+    cur = ahead;
+    base = next;
+  }
 }
 
 }  // namespace evt

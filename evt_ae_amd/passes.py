@@ -321,6 +321,8 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                                      -> mul(mul(neg(one_hot(target)), tangent),
                                             unsqueeze(ne(target, ignore_index), 1)) [/ batch]   (:294-348;
                                         the reference compares with -1 instead of ignore_index)
+      native_layer_norm(x, s, w, b, eps)
+                                     -> add(mul(native_layer_norm(x, s, None, None, eps)[0], w), b)   (:504-544)
     and permute(permute(x)) folded into one permute or none.  The reference's
     other decompositions (layer / batch norm, convolution, pooling, spmm)
     belong to anchors this backend does not provide and are left untouched."""
@@ -386,6 +388,24 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                     new = mk(aten.mul, (grad, keep))
                     if reduction == 1:       # mean over the batch (labels equal to ignore_index are
                         new = mk(aten.div, (new, int(shape[0])))     # not discounted, as in the reference)
+            elif name == "native_layer_norm" and len(node.args) == 5 and (node.args[2] is not None or node.args[3] is not None):
+                # weight and bias become epilogue nodes of the normalisation (:504-544)
+                x, shape, w, b, eps = node.args
+                plain = mk(aten.native_layer_norm, (x, shape, None, None, eps))
+                items = {i: mk(operator.getitem, (plain, i)) for i in range(3)}
+                y = items[0]
+                if w is not None:
+                    y = mk(aten.mul, (y, w))
+                if b is not None:
+                    y = mk(aten.add, (y, b))
+                for user in list(node.users):
+                    if user.op == "call_function" and user.target is operator.getitem:
+                        user.replace_all_uses_with(y if user.args[1] == 0 else items[int(user.args[1])])
+                        graph.erase_node(user)
+                if not node.users:
+                    graph.erase_node(node)
+                    changed = True
+                continue
             elif name == "native_dropout" and len(node.args) == 3 and node.args[2] is True:
                 x, p = node.args[0], node.args[1]
                 mask = mk(aten.ge, (mk(torch.rand_like, (x,)), p))

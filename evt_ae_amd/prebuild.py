@@ -56,6 +56,8 @@ def register_all() -> List[jit.LazyModule]:
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
     for name, (cls, _) in W.ROW_ANCHOR_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    for name, (cls, shapes, _) in W.ROW_BENCH.items():
+        W.fuse(cls(), [torch.empty(sh, dtype=dt, device="meta") for sh, dt in shapes])
     from .aot_helper import aot_capture, evt_backend
     aot_capture(*W.mlp_classifier())
     # the same step through torch.compile: Dynamo's graph differs slightly, so

@@ -708,6 +708,49 @@ ROW_ANCHOR_PATTERNS = {
 }
 
 
+# bandwidth cases for the row-wise anchors (bench.py): attention probabilities of 256 x 512 x 512 and
+# 131072 rows of a 1024-wide layer norm, fp16, sized so that a few rotating buffer sets exceed the 256 MB cache
+
+class RowBenchSoftmax(torch.nn.Module):
+    def forward(self, x):
+        return aten._softmax(x, -1, False)
+
+
+class RowBenchSoftmaxBackward(torch.nn.Module):
+    def forward(self, g, y):
+        return aten._softmax_backward_data(g, y, -1, torch.float16)
+
+
+class RowBenchLayerNorm(torch.nn.Module):
+    def forward(self, x, w, b):
+        ln = aten.native_layer_norm(x, [1024], None, None, 1e-5)
+        y = aten.add(aten.mul(operator.getitem(ln, 0), w), b)
+        return y, operator.getitem(ln, 1), operator.getitem(ln, 2)
+
+
+class RowBenchLayerNormBackward(torch.nn.Module):
+    def forward(self, g, x, mean, rstd, w):
+        ln = aten.native_layer_norm_backward(g, x, [1024], mean, rstd, w, None, [True, False, False])
+        return operator.getitem(ln, 0)
+
+
+def _row_bench_shapes():
+    sm, ln = (256, 512, 512), (131072, 1024)
+    h, f = torch.float16, torch.float32
+    return {
+        # name: (module, [(shape, dtype), ...] inputs, algorithmic bytes per launch)
+        "softmax": (RowBenchSoftmax, [(sm, h)], 2 * 2 * 256 * 512 * 512),
+        "softmax_backward": (RowBenchSoftmaxBackward, [(sm, h), (sm, h)], 3 * 2 * 256 * 512 * 512),
+        "layernorm": (RowBenchLayerNorm, [(ln, h), ((1024,), h), ((1024,), h)], 2 * 2 * 131072 * 1024 + 8 * 131072),
+        "layernorm_backward": (RowBenchLayerNormBackward,
+                               [(ln, h), (ln, h), ((131072, 1), f), ((131072, 1), f), ((1024,), h)],
+                               3 * 2 * 131072 * 1024 + 8 * 131072),
+    }
+
+
+ROW_BENCH = _row_bench_shapes()
+
+
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
     return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS.get(name)

@@ -72,6 +72,20 @@ typedef struct EvtTensorArg {
  * module (see evt_module_spec).  `lda`/`ldb` are the strides, in elements, of
  * the non-contiguous dimension; batch strides are in elements and may be 0.
  * Replaces GemmArguments / BmmArguments2x (evt_fuser.py:539-544, bmm.py:23-64).
+ *
+ * Row-wise modules (module spec has "anchor": softmax, softmax_backward,
+ * layernorm, layernorm_backward; they replace SoftmaxArguments /
+ * SoftmaxBackwardArguments / LayerNormArguments / LayerNormBackwardArguments,
+ * evt_fuser.py:755-760, :818-824, :893-900, :960-968) use the same block: the
+ * operand is viewed as [L, M, N] with rows of N contiguous elements; A is the
+ * input (backward modules: the incoming gradient) and B the second operand of
+ * the backward modules (softmax output / forward input), `lda`/`ldb` their row
+ * strides and the batch strides their strides between batches, in elements;
+ * K is ignored.  N may not exceed the module's "row"."max_n".  A layer norm's
+ * eps is scalars["anchor_scalars"]; layer norm backward reads the forward
+ * pass's mean and rstd (fp32, one per row, contiguous) and optionally the
+ * weight from the tensor slots listed under "anchor_tensors".  These modules
+ * need no workspace (evt_workspace_bytes returns 0).
  */
 typedef struct EvtArgs {
   int32_t M, N, K, L;

@@ -2,11 +2,13 @@
 subgraphs and the reference's fuser-test patterns (unittest/evt_fuser/mm.py,
 bmm.py) to an IR whose CPU interpretation equals PyTorch's fp32 eager
 evaluation of the original module."""
+import operator
+
 import pytest
 import torch
 
 from evt_ae_amd import workloads as W
-from evt_ae_amd.evt_fuser import EVTFuser, FusedBMM, FusedGEMM
+from evt_ae_amd.evt_fuser import EVTFuser, FusedBMM, FusedGEMM, target_name
 from oracle import evt_oracle
 from tests.util import fused_nodes, rand_slot, run_emulated
 
@@ -243,3 +245,76 @@ def test_stubbed_anchors():
     for name in ("FusedConvFprop", "FusedConvDgrad", "FusedSpmm"):
         with pytest.raises(NotImplementedError):
             getattr(evt_fuser, name)(None, None)
+
+
+# ---------------------------------------------------------------------------
+# row-wise anchors (softmax / layer norm, forward and backward)
+# ---------------------------------------------------------------------------
+
+ROW_CLASSES = {"softmax": "FusedSoftmax", "softmax_backward": "FusedSoftmaxBackward",
+               "layernorm": "FusedLayerNorm", "layernorm_backward": "FusedLayerNormBackward"}
+
+
+@pytest.mark.parametrize("name", list(W.ROW_ANCHOR_PATTERNS))
+def test_row_anchor_patterns_trace(name):
+    """Every pattern of the reference's softmax / layer norm fuser tests becomes
+    one fused node of the matching class whose module describes a row kernel
+    (reference: FusedSoftmax ... FusedLayerNormBackward, evt_fuser.py:700-970)."""
+    from evt_ae_amd.codegen import RowSpec
+    cls, _ = W.ROW_ANCHOR_PATTERNS[name]
+    inputs = W.pattern_inputs(name)
+    gm = W.fuse(cls(), [t.to("meta") for t in inputs])
+    (node,) = fused_nodes(gm)
+    op = node.target
+    kind = op.row_spec.op
+    assert type(op).__name__ == ROW_CLASSES[kind] and isinstance(op.row_spec, RowSpec)
+    M, N, K, L = op.problem
+    assert K == 1 and N == inputs[0].shape[-1] and L * M * N == inputs[0].numel()
+    assert op.row_spec.max_n >= N and op.row_spec.lpr in (8, 16, 32, 64) and 1 <= op.row_spec.ch <= 16
+    spec = op.module.spec
+    assert spec["abi"] == 2 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
+    assert op.num_anchor_inputs == {"softmax": 1, "softmax_backward": 2, "layernorm": 1, "layernorm_backward": 5}[kind]
+    if kind == "layernorm":
+        # eps travels as a scalar; mean and rstd are per-row stores
+        assert op.ir.scalars[spec["anchor_scalars"]] == pytest.approx(1e-12)
+        assert sum(1 for s in op.ir.slots if s.role == "store" and s.domain == "row") == 2
+    if kind == "layernorm_backward":
+        assert [op.ir.slots[k].name for k in spec["anchor_tensors"]] == ["mean", "invstd", "gamma"]
+
+
+def test_row_anchor_limits():
+    from evt_ae_amd.codegen import RowSpec
+    aten = torch.ops.aten
+
+    class SoftmaxOverRows(torch.nn.Module):
+        def forward(self, x):
+            return aten._softmax(x, 0, False)
+
+    class LayerNormWithWeight(torch.nn.Module):
+        def forward(self, x, w, b):
+            return operator.getitem(aten.native_layer_norm(x, [64], w, b, 1e-5), 0)
+
+    class SoftmaxThenColumnSum(torch.nn.Module):
+        def forward(self, x):
+            y = aten.mul(aten._softmax(x, -1, False), 2.)
+            return y, aten.sum(y, [0], True)
+
+    x = torch.empty(32, 64, dtype=torch.float16, device="meta")
+    for mod, ins in ((SoftmaxOverRows(), [x]), (LayerNormWithWeight(), [x, x[0], x[0]])):
+        gm = W.trace_module(mod, ins)
+        names = [n.name for n in gm.graph.nodes if n.op == "call_function"]
+        with pytest.raises(NotImplementedError):
+            EVTFuser().trace(gm, names)
+        assert not fused_nodes(W.fuse(mod, ins))                 # pass_fusion leaves such an anchor to eager
+    # a reduction behind a row-wise anchor is not fused: the partition is cut in front of it
+    gm = W.fuse(SoftmaxThenColumnSum(), [x])
+    (node,) = fused_nodes(gm)
+    assert node.target.partition_names == ["_softmax", "mul"]
+    assert [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"].count("sum") == 1
+    # row length -> lanes per row and chunks
+    assert RowSpec.for_row_length("softmax", 64, "f16") == RowSpec("softmax", 1, 8, "f16")
+    assert RowSpec.for_row_length("softmax", 512, "f16") == RowSpec("softmax", 2, 32, "f16")
+    assert RowSpec.for_row_length("layernorm", 1024, "f16") == RowSpec("layernorm", 2, 64, "f16")
+    assert RowSpec.for_row_length("layernorm", 8192, "bf16") == RowSpec("layernorm", 16, 64, "bf16")
+    with pytest.raises(NotImplementedError):
+        RowSpec.for_row_length("softmax", 8200, "f16")

@@ -214,3 +214,23 @@ def test_torch_compile_backend_traces_here():
     model, (x, y) = W.mlp_classifier()
     with pytest.raises(RuntimeError, match="HIP device only"):
         torch.compile(model, backend=evt_backend)(x, y)
+
+
+def test_layer_norm_weight_and_bias_are_split_off():
+    class M(torch.nn.Module):
+        def forward(self, x, w, b):
+            ln = aten.native_layer_norm(x, [64], w, b, 1e-5)
+            return operator.getitem(ln, 0), operator.getitem(ln, 1), operator.getitem(ln, 2)
+
+    x, w, b = torch.randn(6, 5, 64), torch.randn(64), torch.randn(64)
+    gm = W.trace_module(M(), [x, w, b])
+    pass_decomposition(gm)
+    ln = [n for n in gm.graph.nodes if n.op == "call_function" and target_name(n.target) == "native_layer_norm"]
+    assert len(ln) == 1 and ln[0].args[2] is None and ln[0].args[3] is None
+    for got, ref in zip(gm(x, w, b), M()(x, w, b)):
+        assert torch.allclose(got, ref, rtol=1e-5, atol=1e-6)
+    # after the split the normalisation is a row-wise anchor with weight and bias in its epilogue
+    from evt_ae_amd.passes import pass_fusion
+    pass_fusion(gm, gm.graph)
+    (node,) = fused_nodes(gm)
+    assert type(node.target).__name__ == "FusedLayerNorm" and {"mul", "add"} <= set(node.target.partition_names)
