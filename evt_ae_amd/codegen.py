@@ -925,7 +925,7 @@ class RowCodegen(Codegen):
         e("  if (rc != EVT_OK) return rc;")
         e("  // workgroups per CU before waves start walking over several rows (0: one pass, a workgroup per Cfg::ROWS rows);")
         e("  // walking pays when row vectors are kept in registers across the rows of a wave")
-        e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); return s ? atoi(s) : {16 if (self.hoisted or len(ir.anchor_slots) > 2) else 0}; }}();")
+        e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); return s ? atoi(s) : {16 if self.hoisted else 0}; }}();")
         e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
           "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
         e("  const int64_t want = ((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS;")

@@ -56,6 +56,11 @@ def register_all() -> List[jit.LazyModule]:
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
     for name, (cls, _) in W.ROW_ANCHOR_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    for anchor in ("softmax", "softmax_backward", "layernorm", "layernorm_backward"):
+        for n in W.ROW_EDGE_LENGTHS:
+            for dt in W.ROW_EDGE_DTYPES:
+                mod, ins = W.row_edge_case(anchor, n, dt)
+                W.fuse(mod, _meta(ins))
     for name, (cls, shapes, _) in W.ROW_BENCH.items():
         W.fuse(cls(), [torch.empty(sh, dtype=dt, device="meta") for sh, dt in shapes])
     from .aot_helper import aot_capture, evt_backend

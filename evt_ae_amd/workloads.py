@@ -751,6 +751,66 @@ def _row_bench_shapes():
 ROW_BENCH = _row_bench_shapes()
 
 
+# row lengths and element types of the row-wise anchors beyond the reference's patterns: the shortest and the
+# longest supported rows, lengths that are no multiple of 8 (generic path), bf16 and fp32 operands
+
+class _BareSoftmax(torch.nn.Module):
+    def forward(self, x):
+        return aten._softmax(x, -1, False)
+
+
+class _BareSoftmaxBackward(torch.nn.Module):
+    def __init__(self, dtype):
+        super().__init__()
+        self.dtype = dtype
+
+    def forward(self, g, y):
+        return aten._softmax_backward_data(g, y, -1, self.dtype)
+
+
+class _BareLayerNorm(torch.nn.Module):
+    def __init__(self, n):
+        super().__init__()
+        self.n = n
+
+    def forward(self, x):
+        ln = aten.native_layer_norm(x, [self.n], None, None, 1e-5)
+        return operator.getitem(ln, 0), operator.getitem(ln, 1), operator.getitem(ln, 2)
+
+
+class _BareLayerNormBackward(torch.nn.Module):
+    def __init__(self, n):
+        super().__init__()
+        self.n = n
+
+    def forward(self, g, x, mean, rstd):
+        ln = aten.native_layer_norm_backward(g, x, [self.n], mean, rstd, None, None, [True, False, False])
+        return operator.getitem(ln, 0)
+
+
+ROW_EDGE_LENGTHS = (8, 24, 1000, 8192)
+ROW_EDGE_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
+
+
+def row_edge_case(anchor: str, n: int, dtype, seed: int = 0):
+    """(module, CPU inputs) for a bare anchor on 3 x 7 rows of length n."""
+    g = torch.Generator(device="cpu").manual_seed(0xED6E + 31 * n + seed)
+    shape = (3, 7, n)
+    x = (torch.randn(shape, generator=g) * 2 + 0.5).to(dtype)
+    if anchor == "softmax":
+        return _BareSoftmax(), [x]
+    if anchor == "softmax_backward":
+        y = torch.softmax(torch.randn(shape, generator=g), -1).to(dtype)
+        return _BareSoftmaxBackward(dtype), [x, y]
+    if anchor == "layernorm":
+        return _BareLayerNorm(n), [x]
+    grad = torch.randn(shape, generator=g).to(dtype)
+    xf = x.float()
+    mean = xf.mean(-1, keepdim=True)
+    rstd = torch.rsqrt(xf.var(-1, unbiased=False, keepdim=True) + 1e-5)
+    return _BareLayerNormBackward(n), [grad, x, mean, rstd]
+
+
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
     return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS.get(name)

@@ -378,3 +378,26 @@ def test_row_anchor_patterns(name):
         stat = o.dtype == torch.float32 and o.numel() * 8 <= inputs[0].numel()      # per-row mean / rstd
         err = evt_oracle.max_rel_err(o, r)
         assert err <= (REDUCTION_TOL if stat else FP16_TOL), f"{name} output {k}: max rel err {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", W.ROW_EDGE_DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("n", W.ROW_EDGE_LENGTHS)
+@pytest.mark.parametrize("anchor", ["softmax", "softmax_backward", "layernorm", "layernorm_backward"])
+def test_row_anchor_lengths_and_dtypes(anchor, n, dtype):
+    """Bare row-wise anchors at the shortest (8) and longest (8192) supported row,
+    at lengths that are no multiple of 8 or of the 16-byte access (24, 1000: the
+    generic path), in fp16, bf16 and fp32, against the fp32 oracle."""
+    mod, inputs = W.row_edge_case(anchor, n, dtype)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    assert node.target.row_spec.max_n >= n
+    outs = gm(*[t.cuda() for t in inputs])
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    tol = {torch.float16: FP16_TOL, torch.bfloat16: FP16_TOL, torch.float32: REDUCTION_TOL}[dtype]
+    for k, (o, r) in enumerate(zip(outs, refs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        stat = k > 0                                  # layer norm's mean and rstd (fp32)
+        err = evt_oracle.max_rel_err(o, r)
+        assert err <= (REDUCTION_TOL if stat else tol), f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
