@@ -205,18 +205,17 @@ def test_philox_known_answers():
 # ---------------------------------------------------------------------------
 
 def test_row_anchor_oracle_against_definitions():
-    from evt_ae_amd import workloads as W
     g = torch.Generator().manual_seed(11)
     for n in (8, 24, 1000):
         # softmax: closed form; rows sum to one; shift invariance
         mod, (x,) = W.row_edge_case("softmax", n, torch.float16)
-        (y,) = evt_oracle.eval_fp32(mod, [x])
+        (y,) = O.eval_fp32(mod, [x])
         xd = x.double()
         e = np.exp(xd.numpy() - xd.numpy().max(-1, keepdims=True))
         assert np.allclose(y.numpy(), e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-7)
         # softmax backward = vector-Jacobian product of softmax
         mod, (gr, ys) = W.row_edge_case("softmax_backward", n, torch.float16)
-        (dx,) = evt_oracle.eval_fp32(mod, [gr, ys])
+        (dx,) = O.eval_fp32(mod, [gr, ys])
         z = torch.randn(3, 7, n, dtype=torch.float64, generator=g).requires_grad_()
         sm = torch.softmax(z, -1)
         (auto,) = torch.autograd.grad(sm, z, gr.double())
@@ -226,7 +225,7 @@ def test_row_anchor_oracle_against_definitions():
         assert torch.allclose(dx.double(), (gr.double() - (gr.double() * yd).sum(-1, keepdim=True)) * yd, rtol=1e-4, atol=1e-6)
         # layer norm: closed form of y, mean, rstd
         mod, (x,) = W.row_edge_case("layernorm", n, torch.float16)
-        yv, mean, rstd = evt_oracle.eval_fp32(mod, [x])
+        yv, mean, rstd = O.eval_fp32(mod, [x])
         xd = x.double().numpy()
         mu, var = xd.mean(-1, keepdims=True), xd.var(-1, keepdims=True)
         assert np.allclose(mean.numpy(), mu, rtol=1e-5, atol=1e-6)
@@ -234,7 +233,7 @@ def test_row_anchor_oracle_against_definitions():
         assert np.allclose(yv.numpy(), (xd - mu) / np.sqrt(var + 1e-5), rtol=1e-4, atol=1e-5)
         # layer norm backward = vector-Jacobian product of layer norm (no weight)
         mod, (gr, x, mean, rstd) = W.row_edge_case("layernorm_backward", n, torch.float16)
-        (dx,) = evt_oracle.eval_fp32(mod, [gr, x, mean, rstd])
+        (dx,) = O.eval_fp32(mod, [gr, x, mean, rstd])
         z = x.double().clone().requires_grad_()
         out = torch.nn.functional.layer_norm(z, (n,), eps=1e-5)
         (auto,) = torch.autograd.grad(out, z, gr.double())
