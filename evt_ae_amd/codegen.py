@@ -701,7 +701,13 @@ class RowCodegen(Codegen):
         super().__init__(ir, None, module_name)
         self.row_spec = spec
         for r in ir.reduces.values():
-            raise NotImplementedError(f"reduction {r.name} behind a row-wise anchor")
+            # a sum / max over all rows is carried in registers and combined in two phases; a reduction along
+            # the row would be a second pass over the anchor's own axis
+            if r.axis != "col" or r.kind not in ("sum", "max"):
+                raise NotImplementedError(f"per-row reduction {r.name} behind a row-wise anchor")
+        if ir.col_state and (ir.L != 1 or 4 * ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536):
+            raise NotImplementedError("per-column reduction behind a row-wise anchor: one batch and rows of at most "
+                                      f"{65536 // (16 * max(ir.col_state, 1))} elements")
         for n in ir.nodes.values():
             if n.op == "colidx" or (n.op == "load" and ir.slots[n.slot].kind == "rand"):
                 raise NotImplementedError(f"{n.op} behind a row-wise anchor")
@@ -716,9 +722,8 @@ class RowCodegen(Codegen):
         ir = self.ir
         tile_stores = [s for s in ir.stores if s.domain == "tile"]
         row_stores = [s for s in ir.stores if s.domain == "row"]
-        if len(tile_stores) + len(row_stores) != len(ir.stores):
-            raise NotImplementedError("per-column outputs behind a row-wise anchor")
-        need = ir.closure([s.input for s in ir.stores])
+        col_reds = list(ir.reduces.values())
+        need = ir.closure([s.input for s in tile_stores + row_stores] + [r.input for r in col_reds])
         outer = [n for n in need if not self.var_n[n]]
         inner = [n for n in need if self.var_n[n]]
         nh = len(self.hoisted)
@@ -747,7 +752,7 @@ class RowCodegen(Codegen):
         e("}")
         e("template <class Cfg, bool FAST, class Ctx>")
         e(f"static EVT_DEV void row(const Params& p, const Ctx& t, const float (&acc)[Cfg::CH][8], const float (&rv)[2], "
-          f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8]) {{")
+          f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8], float (&cst)[{max(ir.col_state, 1)}][Cfg::CH][8]) {{")
         e.indent()
         for k, s in enumerate(ir.slots):
             e(f"const int64_t o_{k} = (int64_t)evt::batch_index(t.l, p.t{k}_lm, p.t{k}_ld) * p.t{k}_sl + (int64_t)t.m * p.t{k}_sm;")
@@ -793,6 +798,14 @@ class RowCodegen(Codegen):
                 src = f"b_{k}"
             e(f"if constexpr (FAST) evt::store8v(p.t{k} + o_{k} + n0, {src});")
             e(f"else evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
+        for r in col_reds:
+            x = f"{_cname(r.input)}[j]" if self.var_n[r.input] else _cname(r.input)
+            o = r.state_offset
+            e("#pragma unroll")
+            if r.kind == "sum":
+                e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] += j < nv ? {x} : 0.f;")
+            else:
+                e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] = j < nv ? fmaxf(cst[{o}][c][j], {x}) : cst[{o}][c][j];")
         e.dedent()
         e("}")
         e.dedent()
@@ -806,7 +819,7 @@ class RowCodegen(Codegen):
                 e(f"evt::st_f32(p.t{s.slot}, o_{s.slot}, {_cname(s.input)});")
             e.dedent()
             e("}")
-        e("(void)p; (void)t; (void)acc; (void)rv; (void)hz;")
+        e("(void)p; (void)t; (void)acc; (void)rv; (void)hz; (void)cst;")
         e.dedent()
         e("}")
 
@@ -820,7 +833,7 @@ class RowCodegen(Codegen):
             "element": sp.elt,
             "batched": self.ir.batched,
             "row_state": 0,
-            "col_state": 0,
+            "col_state": self.ir.col_state,
             "tensors": [{"name": s.name, "role": s.role, "dtype": s.dtype, "kind": s.kind,
                          "domain": s.domain} for s in self.ir.slots],
             "num_scalars": len(self.ir.scalars),
@@ -847,7 +860,11 @@ class RowCodegen(Codegen):
         e("namespace {")
         e("struct Epi {")
         e.indent()
+        e(f"static constexpr int COL_STATE = {ir.col_state};")
         self.emit_params(e)
+        self.emit_combine(e, "col")
+        self.emit_identity(e, "col")
+        self.emit_finalize(e, "col")
         self.emit_row(e)
         e.dedent()
         e("};")
@@ -870,7 +887,9 @@ class RowCodegen(Codegen):
         e("if (a->lda < a->N) return EVT_ERR_BAD_ARGS;")
         e("g.vecA = (((uintptr_t)a->A | (uintptr_t)(a->lda * kEltBytes) | (uintptr_t)(a->batch_stride_A * kEltBytes)) & 15) == 0;")
         e("g.vecB = (((uintptr_t)a->B | (uintptr_t)(a->ldb * kEltBytes) | (uintptr_t)(a->batch_stride_B * kEltBytes)) & 15) == 0;")
-        e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0;")
+        e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0; g.colws = nullptr;")
+        if ir.col_state:
+            e("if (a->L != 1) return EVT_ERR_BAD_ARGS;      // the per-column reductions run over every row")
         e(f"g.fast = (g.vecA && {'g.vecB && ' if two else ''}(a->N & 7) == 0) ? 1 : 0;")
         e(f"g.eps = {'a->scalars[%d]' % ir.anchor_scalar if ir.anchor_scalar is not None else '0.f'};")
         if stats:
@@ -909,29 +928,42 @@ class RowCodegen(Codegen):
         e('extern "C" int evt_abi_version(void) { return EVT_ABI_VERSION; }')
         spec_json = json.dumps(self.module_spec(), sort_keys=True)
         e(f'extern "C" const char* evt_module_spec(void) {{ return R"evtjson({spec_json})evtjson"; }}')
-        e('extern "C" int64_t evt_workspace_bytes(const EvtArgs* a) {')
-        e("  evt::RowArgs g; Epi::Params p;")
-        e("  const int rc = fill(a, g, p);")
-        e("  return rc != EVT_OK ? rc : 0;      // row-wise anchors keep everything in registers")
-        e("}")
-        e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
-        e("  (void)ws; (void)bytes; (void)stream;")
-        e("  return EVT_OK;")
-        e("}")
-        e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
-        e("  (void)ws; (void)ws_bytes;")
-        e("  evt::RowArgs g; Epi::Params p;")
-        e("  const int rc = fill(a, g, p);")
-        e("  if (rc != EVT_OK) return rc;")
-        e("  // workgroups per CU before waves start walking over several rows (0: one pass, a workgroup per Cfg::ROWS rows);")
-        e("  // walking pays when row vectors are kept in registers across the rows of a wave")
-        e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); return s ? atoi(s) : {16 if self.hoisted else 0}; }}();")
+        e("// workgroups per CU before waves start walking over several rows (0: one pass, a workgroup per Cfg::ROWS rows);")
+        e("// walking pays when row vectors are kept in registers across the rows of a wave, and bounds the number of")
+        e("// partials of a per-column reduction")
+        default_cap = 8 if ir.col_state else (16 if self.hoisted else 0)
+        e("static unsigned grid_for(const evt::RowArgs& g) {")
+        e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); int v = s ? atoi(s) : {default_cap}; "
+          f"return {'v > 0 ? v : 8' if ir.col_state else 'v'}; }}();")
         e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
           "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
         e("  const int64_t want = ((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS;")
-        e("  const unsigned grid = (unsigned)((per_cu <= 0 || want < (int64_t)cus * per_cu) ? want : (int64_t)cus * per_cu);")
+        e("  return (unsigned)((per_cu <= 0 || want < (int64_t)cus * per_cu) ? want : (int64_t)cus * per_cu);")
+        e("}")
+        e('extern "C" int64_t evt_workspace_bytes(const EvtArgs* a) {')
+        e("  evt::RowArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  // partials of the per-column reductions, one per (workgroup, state word, column); nothing else is staged")
+        e("  return (int64_t)grid_for(g) * Epi::COL_STATE * g.N * 4;")
+        e("}")
+        e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
+        e("  (void)ws; (void)bytes; (void)stream;      // no counters: every partial is written before it is read")
+        e("  return EVT_OK;")
+        e("}")
+        e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
+        e("  evt::RowArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  const unsigned grid = grid_for(g);")
+        e("  const int64_t need = (int64_t)grid * Epi::COL_STATE * g.N * 4;")
+        e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
+        e("  g.colws = (float*)ws;")
         e("  if (p.fast) hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, true>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  else hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, false>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  int err = (int)hipGetLastError();")
+        e("  if (err != 0 || Epi::COL_STATE == 0) return err;")
+        e("  hipLaunchKernelGGL((evt::evt_row_col_finalize_kernel<Epi>), dim3((g.N + 255) / 256), dim3(256), 0, (hipStream_t)stream, g, p, (int)grid);")
         e("  return (int)hipGetLastError();")
         e("}")
         return e.text()

@@ -37,6 +37,7 @@ struct RowArgs {
   int vecG;
   float eps;                 // layer norm
   int vecA, vecB;            // rows of A / B may be read with 16-byte loads
+  float* colws;              // per-column reductions of the epilogue: [workgroups][COL_STATE][N] partials
   int fast;                  // N % 8 == 0 and every anchor operand is 16-byte aligned: whole 8-column groups only
 };
 
@@ -393,6 +394,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
 // to fill the chip once instead of one workgroup per handful of rows.
 template <class Cfg, class Epi, bool FAST>
 __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typename Epi::Params p) {
+  constexpr int CS = Epi::COL_STATE;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t rows = (int64_t)g.L * g.M;
@@ -407,46 +409,116 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
     t.l = (int)(t.r / g.M);
     t.m = (int)(t.r % g.M);
   };
+  // this lane's share of the epilogue's per-column reductions, carried over all rows the wave visits
+  float cst[CS > 0 ? CS : 1][Cfg::CH][8];
+  if constexpr (CS > 0) {
+#pragma unroll
+    for (int c = 0; c < Cfg::CH; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float id[CS];
+        Epi::col_identity(id);
+#pragma unroll
+        for (int k = 0; k < CS; ++k) cst[k][c][j] = id[k];
+      }
+  }
   int64_t base = ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW;    // wave-uniform
-  if (base >= rows) return;
-  RowRaw<Cfg> cur;
-  locate(base);
-  row_fetch<Cfg, FAST>(g, t, cur);
-  float hz[Epi::NH > 0 ? Epi::NH : 1][Cfg::CH][8];
-  Epi::template hoist<Cfg, FAST>(p, t, hz);
-  float gz[Cfg::CH][8];          // layer norm backward: this lane's columns of the weight, read once
-  if constexpr (Cfg::OP == ROW_LAYERNORM_BWD) {
-    using T = typename RowElt<Cfg::ELT>::type;
-    if (g.gamma) {
+  if (base < rows) {
+    RowRaw<Cfg> cur;
+    locate(base);
+    row_fetch<Cfg, FAST>(g, t, cur);
+    float hz[Epi::NH > 0 ? Epi::NH : 1][Cfg::CH][8];
+    Epi::template hoist<Cfg, FAST>(p, t, hz);
+    float gz[Cfg::CH][8];          // layer norm backward: this lane's columns of the weight, read once
+    if constexpr (Cfg::OP == ROW_LAYERNORM_BWD) {
+      using T = typename RowElt<Cfg::ELT>::type;
+      if (g.gamma) {
 #pragma unroll
-      for (int c = 0; c < Cfg::CH; ++c) {
-        const int v = t.valid(c);
-        if (v > 0) {
-          load8<T>(reinterpret_cast<const T*>(g.gamma) + t.col0(c), g.vecG != 0, v, 0.f, gz[c]);
-        } else {
+        for (int c = 0; c < Cfg::CH; ++c) {
+          const int v = t.valid(c);
+          if (v > 0) {
+            load8<T>(reinterpret_cast<const T*>(g.gamma) + t.col0(c), g.vecG != 0, v, 0.f, gz[c]);
+          } else {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) gz[c][j] = 0.f;
+            for (int j = 0; j < 8; ++j) gz[c][j] = 0.f;
+          }
         }
       }
     }
-  }
-  while (true) {
-    const RowCtx<Cfg> here = t;
-    const int64_t next = base + stride;
-    const bool more = next < rows;                                         // wave-uniform
-    RowRaw<Cfg> ahead;
-    if (more) {
-      locate(next);
-      row_fetch<Cfg, FAST>(g, t, ahead);
+    while (true) {
+      const RowCtx<Cfg> here = t;
+      const int64_t next = base + stride;
+      const bool more = next < rows;                                         // wave-uniform
+      RowRaw<Cfg> ahead;
+      if (more) {
+        locate(next);
+        row_fetch<Cfg, FAST>(g, t, ahead);
+      }
+      float acc[Cfg::CH][8];
+      float rv[2];
+      row_main<Cfg>(g, here, cur, gz, acc, rv);
+      if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, hz, cst);
+      if (!more) break;
+      cur = ahead;
+      base = next;
     }
-    float acc[Cfg::CH][8];
-    float rv[2];
-    row_main<Cfg>(g, here, cur, gz, acc, rv);
-    if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, hz);
-    if (!more) break;
-    cur = ahead;
-    base = next;
   }
+  if constexpr (CS > 0) {
+    // Column partials of the workgroup: first across the row groups of a wave (lanes that hold the same
+    // columns of different rows), then across the waves through LDS; one partial per (workgroup, column)
+    // goes to the workspace and a second kernel adds the workgroups up in a fixed order.
+    __shared__ float red[Cfg::WAVES][CS][Cfg::CH * Cfg::SPAN];
+#pragma unroll
+    for (int k = 0; k < CS; ++k)
+#pragma unroll
+      for (int c = 0; c < Cfg::CH; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float x = cst[k][c][j];
+#pragma unroll
+          for (int m = Cfg::LPR; m < 64; m <<= 1) {
+            float a[CS], b[CS];
+            Epi::col_identity(a); Epi::col_identity(b);
+            a[k] = x; b[k] = __shfl_xor(x, m, 64);
+            Epi::col_combine(a, b);
+            x = a[k];
+          }
+          if (lane < Cfg::LPR) red[wave][k][c * Cfg::SPAN + t.sub * 8 + j] = x;
+        }
+    __syncthreads();
+    for (int n = threadIdx.x; n < g.N; n += Cfg::THREADS) {
+      float a[CS];
+#pragma unroll
+      for (int k = 0; k < CS; ++k) a[k] = red[0][k][n];
+#pragma unroll
+      for (int w = 1; w < Cfg::WAVES; ++w) {
+        float b[CS];
+#pragma unroll
+        for (int k = 0; k < CS; ++k) b[k] = red[w][k][n];
+        Epi::col_combine(a, b);
+      }
+#pragma unroll
+      for (int k = 0; k < CS; ++k) g.colws[((int64_t)blockIdx.x * CS + k) * g.N + n] = a[k];
+    }
+  }
+}
+
+// second phase of the per-column reductions: one thread per column adds the workgroups' partials in
+// workgroup order and evaluates the per-column output expressions
+template <class Epi>
+__global__ __launch_bounds__(256) void evt_row_col_finalize_kernel(RowArgs g, typename Epi::Params p, int blocks) {
+  constexpr int CS = Epi::COL_STATE > 0 ? Epi::COL_STATE : 1;
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= g.N) return;
+  float a[CS];
+  Epi::col_identity(a);
+  for (int b = 0; b < blocks; ++b) {
+    float x[CS];
+#pragma unroll
+    for (int k = 0; k < CS; ++k) x[k] = g.colws[((int64_t)b * CS + k) * g.N + n];
+    Epi::col_combine(a, x);
+  }
+  Epi::col_finalize(p, 0, n, a);
 }
 
 }  // namespace evt

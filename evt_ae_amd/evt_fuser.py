@@ -669,6 +669,48 @@ class EVTFuser:
         self.outputs_subgraph = set(outputs)
         self.reference_gm = self._extract_reference(graph_module, anchor, epilogue_partition, inputs, outputs)
 
+        # Steps 3 and 4: the epilogue IR and its stores.  A row-wise anchor on a tensor of rank 3 or more is
+        # first viewed as [L, M, N] (what broadcasts along a middle axis need); if the epilogue cannot be
+        # expressed that way (a reduction over every row, say), as one batch of L * M rows
+        try:
+            fused_kernel = self._lower(anchor, epilogue_partition, epi_set, inputs, outputs, flatten=False)
+        except NotImplementedError:
+            if packet(anchor.target) not in self.row_targets or getattr(self, "L", 1) == 1:
+                raise
+            fused_kernel = self._lower(anchor, epilogue_partition, epi_set, inputs, outputs, flatten=True)
+
+        # Step 5: compose the fused kernel and rewire the graph
+        if dry_run:
+            return fused_kernel
+        args = [i for i in inputs if i is not anchor] + fused_kernel.args
+        graph_module.graph.inserting_after(anchor)
+        fused_node = graph_module.graph.call_function(fused_kernel, args=tuple(args))
+        # the forward/backward split of AOT autograd reads these tags and wants
+        # tensor metadata on every tensor-valued node
+        carried = {k: anchor.meta[k] for k in ("partitioner_tag", "seq_nr", "autograd_backward") if k in anchor.meta}
+        fused_node.meta = {"evt": True, **carried}
+        graph_module.graph.inserting_after(fused_node)
+        for idx, output_node in enumerate(outputs):
+            get_item_node = graph_module.graph.call_function(operator.getitem, args=(fused_node, idx))
+            graph_module.graph.inserting_after(get_item_node)
+            shape, dtype = node_shape_dtype(output_node)
+            get_item_node.meta = {"tensor_meta": _tensor_meta(shape, dtype), **carried}
+            view_node = graph_module.graph.call_function(aten.view, args=(get_item_node, list(shape)))
+            view_node.meta = {k: v for k, v in output_node.meta.items()
+                              if k in ("tensor_meta", "val", "partitioner_tag", "seq_nr", "autograd_backward")}
+            if output_node is anchor:
+                for user in list(anchor.users):
+                    if user not in epi_set and user is not fused_node:
+                        user.replace_input_with(anchor, view_node)
+            else:
+                output_node.replace_all_uses_with(view_node)
+            graph_module.graph.inserting_after(view_node)
+        self.fused_kernel = fused_kernel
+        return fused_kernel
+
+    def _lower(self, anchor: Node, epilogue_partition, epi_set, inputs, outputs, flatten: bool):
+        """Steps 3 and 4 of `trace`: the epilogue IR and its stores for one
+        choice of the (L, M) split of a row-wise anchor's rows."""
         # Step 3: build the IR
         tgt = packet(anchor.target)
         self.anchor_operands: List[Node] = []
@@ -678,7 +720,7 @@ class EVTFuser:
         self.coords: Dict[Node, Coord] = {}
         self.ir_name: Dict[Node, str] = {}
         if tgt in self.row_targets:
-            self._begin_row_anchor(anchor, tgt)
+            self._begin_row_anchor(anchor, tgt, flatten)
         else:
             (ashape, adtype) = node_shape_dtype(anchor)
             batched = tgt == aten.bmm
@@ -716,37 +758,9 @@ class EVTFuser:
         self.reduction_names = [s.name for s in self.ir.slots if s.role == "store" and s.domain != "tile"]
         self.transposed = False
 
-        # Step 5: compose the fused kernel and rewire the graph
-        fused_kernel = self.get_fused_node(anchor)
-        if dry_run:
-            return fused_kernel
-        args = [i for i in inputs if i is not anchor] + fused_kernel.args
-        graph_module.graph.inserting_after(anchor)
-        fused_node = graph_module.graph.call_function(fused_kernel, args=tuple(args))
-        # the forward/backward split of AOT autograd reads these tags and wants
-        # tensor metadata on every tensor-valued node
-        carried = {k: anchor.meta[k] for k in ("partitioner_tag", "seq_nr", "autograd_backward") if k in anchor.meta}
-        fused_node.meta = {"evt": True, **carried}
-        graph_module.graph.inserting_after(fused_node)
-        for idx, output_node in enumerate(outputs):
-            get_item_node = graph_module.graph.call_function(operator.getitem, args=(fused_node, idx))
-            graph_module.graph.inserting_after(get_item_node)
-            shape, dtype = node_shape_dtype(output_node)
-            get_item_node.meta = {"tensor_meta": _tensor_meta(shape, dtype), **carried}
-            view_node = graph_module.graph.call_function(aten.view, args=(get_item_node, list(shape)))
-            view_node.meta = {k: v for k, v in output_node.meta.items()
-                              if k in ("tensor_meta", "val", "partitioner_tag", "seq_nr", "autograd_backward")}
-            if output_node is anchor:
-                for user in list(anchor.users):
-                    if user not in epi_set and user is not fused_node:
-                        user.replace_input_with(anchor, view_node)
-            else:
-                output_node.replace_all_uses_with(view_node)
-            graph_module.graph.inserting_after(view_node)
-        self.fused_kernel = fused_kernel
-        return fused_kernel
+        return self.get_fused_node(anchor)
 
-    def _begin_row_anchor(self, anchor: Node, tgt) -> None:
+    def _begin_row_anchor(self, anchor: Node, tgt, flatten: bool = False) -> None:
         """Geometry, accumulator and anchor operands of a row-wise anchor: the
         operand is viewed as [L, M, N] with N its last axis (the reference
         canonicalises these anchors to rank 3, pass_fusion.py:1187-1342)."""
@@ -768,7 +782,9 @@ class EVTFuser:
         L = 1
         for d in shape[:-2]:
             L *= int(d)
-        batched = rank > 2
+        if flatten:          # all rows as one batch: what a reduction over every row needs
+            L, M = 1, L * M
+        batched = L > 1
         self.L, self.M, self.N = L, M, N
         self.ir = EpilogueIR(L, M, N, batched)
         self.ir.add_node(IRNode("accum", "accum", domain="tile"))

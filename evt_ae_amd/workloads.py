@@ -633,6 +633,12 @@ class SoftmaxColumnBroadcast(torch.nn.Module):   # softmax.py:99-111
         return aten.add(aten._softmax(input, -1, False), col)
 
 
+class SoftmaxColumnReduce(torch.nn.Module):   # softmax.py:84-97
+    def forward(self, input):
+        out = aten.mul(aten._softmax(input, -1, False), 2.)
+        return out, aten.sum(out, [0], True)
+
+
 class SoftmaxRagged(torch.nn.Module):
     """Rank 4, a row length that is no multiple of 8, fp32 result of fp16 logits, two results."""
     def forward(self, input, mask):
@@ -681,6 +687,17 @@ class LayerNormBackwardMasked(torch.nn.Module):   # layernorm_backward.py:31-44 
         return getitem, view_282
 
 
+class LayerNormBackwardColumnSum(torch.nn.Module):   # layernorm_backward.py:31-44 as written there
+    def forward(self, grad, input, mean, invstd, gamma, beta, ge_1):
+        ln = aten.native_layer_norm_backward(grad, input, [1024], mean, invstd, gamma, beta, [True, False, False])
+        getitem = operator.getitem(ln, 0)
+        mul_42 = aten.mul(getitem, ge_1)
+        mul_43 = aten.mul(mul_42, 1.0)
+        view_282 = aten.view(mul_43, [2048, 1024])
+        sum_13 = aten.sum(view_282, [0], True)
+        return getitem, view_282, sum_13
+
+
 def _softmax_out(g, shape):
     return torch.softmax(_h(g, shape).float(), -1).half()
 
@@ -700,11 +717,14 @@ ROW_ANCHOR_PATTERNS = {
     "softmax_row_broadcast": (SoftmaxRowBroadcast, lambda g: [_h(g, (16384, 512)), _h(g, (512,))]),
     "softmax_scalar": (SoftmaxScalar, lambda g: [_h(g, (16384, 512))]),
     "softmax_column_broadcast": (SoftmaxColumnBroadcast, lambda g: [_h(g, (16384, 512)), _h(g, (16384, 1))]),
+    "softmax_column_reduce": (SoftmaxColumnReduce, lambda g: [_h(g, (16, 512))]),
+    "softmax_column_reduce_tall": (SoftmaxColumnReduce, lambda g: [_h(g, (40000, 512))]),
     "softmax_ragged": (SoftmaxRagged, lambda g: [_h(g, (3, 5, 37, 203), 3.0), _h(g, (37, 1))]),
     "softmax_backward": (SoftmaxBackward, lambda g: [_h(g, (4, 16, 512, 512)), _softmax_out(g, (4, 16, 512, 512))]),
     "layernorm1": (LayerNormPattern1, lambda g: [_h(g, (512, 2, 1024)) + 1., _h(g, (1024,)), _h(g, (1024,))]),
     "layernorm2": (LayerNormPattern2, lambda g: [_h(g, (512, 2, 1024)) + 1., _h(g, (1024,)), _h(g, (1024,))]),
     "layernorm_backward": (LayerNormBackwardMasked, _ln_backward_inputs),
+    "layernorm_backward_column_sum": (LayerNormBackwardColumnSum, _ln_backward_inputs),
 }
 
 

@@ -85,7 +85,9 @@ typedef struct EvtTensorArg {
  * eps is scalars["anchor_scalars"]; layer norm backward reads the forward
  * pass's mean and rstd (fp32, one per row, contiguous) and optionally the
  * weight from the tensor slots listed under "anchor_tensors".  These modules
- * need no workspace (evt_workspace_bytes returns 0).
+ * need a workspace only when the epilogue reduces over the rows (per-column
+ * sum / max: one partial per workgroup and column; L must then be 1); it holds
+ * no counters, so evt_workspace_init has nothing to do.
  */
 typedef struct EvtArgs {
   int32_t M, N, K, L;
