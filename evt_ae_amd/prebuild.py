@@ -65,6 +65,7 @@ def register_all() -> List[jit.LazyModule]:
         W.fuse(cls(), [torch.empty(sh, dtype=dt, device="meta") for sh, dt in shapes])
     from .aot_helper import aot_capture, evt_backend
     aot_capture(*W.mlp_classifier())
+    aot_capture(*W.encoder_layer())
     # the same step through torch.compile: Dynamo's graph differs slightly, so
     # its kernels are registered as well (tracing stops at the first launch
     # when there is no GPU)

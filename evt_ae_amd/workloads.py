@@ -831,6 +831,52 @@ def row_edge_case(anchor: str, n: int, dtype, seed: int = 0):
     return _BareLayerNormBackward(n), [grad, x, mean, rstd]
 
 
+class EncoderLayer(torch.nn.Module):
+    """fp16 post-LN transformer encoder layer with a squared-error loss: QKV
+    projection, batched QK^T and PV products, softmax, output projection,
+    two layer norms and the GELU feed-forward block (the shape of the
+    reference's BERT test, unittest/fx_passes/bert.py, at a small size)."""
+    def __init__(self, d: int = 256, heads: int = 4, ffn: int = 1024) -> None:
+        super().__init__()
+        self.heads = heads
+        self.qkv = torch.nn.Linear(d, 3 * d)
+        self.out = torch.nn.Linear(d, d)
+        self.ln1 = torch.nn.LayerNorm(d)
+        self.ln2 = torch.nn.LayerNorm(d)
+        self.ffn1 = torch.nn.Linear(d, ffn)
+        self.ffn2 = torch.nn.Linear(ffn, d)
+
+    def forward(self, x, target):
+        B, S, D = x.shape
+        H = self.heads
+        dh = D // H
+        qkv = self.qkv(x).view(B, S, 3, H, dh).permute(2, 0, 3, 1, 4)
+        q, k, v = qkv[0], qkv[1], qkv[2]
+        att = torch.softmax((q @ k.transpose(-1, -2)) / (dh ** 0.5), -1)
+        ctx = (att @ v).permute(0, 2, 1, 3).reshape(B, S, D)
+        x = self.ln1(x + self.out(ctx))
+        x = self.ln2(x + self.ffn2(torch.nn.functional.gelu(self.ffn1(x), approximate="tanh")))
+        return ((x.float() - target) ** 2).sum()
+
+
+def encoder_layer(seed: int = 0, device: str = "cpu", dtype=torch.float16):
+    """(model, (x, target)) with seeded parameters and inputs: batch 8, sequence 128, width 256."""
+    g = torch.Generator(device="cpu").manual_seed(0xE9C + seed)
+    model = EncoderLayer()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() == 2:
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+            elif "ln" in name and name.endswith("weight"):
+                p.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+            else:
+                p.copy_(0.02 * torch.randn(p.shape, generator=g))
+    model = model.to(dtype).to(device)
+    x = torch.randn(8, 128, 256, generator=g).to(dtype).to(device)
+    target = torch.randn(8, 128, 256, generator=g).to(device)
+    return model, (x, target)
+
+
 def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
     return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS.get(name)

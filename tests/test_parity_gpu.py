@@ -401,3 +401,36 @@ def test_row_anchor_lengths_and_dtypes(anchor, n, dtype):
         stat = k > 0                                  # layer norm's mean and rstd (fp32)
         err = evt_oracle.max_rel_err(o, r)
         assert err <= (REDUCTION_TOL if stat else tol), f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
+
+
+def test_aot_encoder_layer_training_step():
+    """A transformer encoder layer, forward and backward, through AOT autograd
+    with the joint pipeline (the reference's BERT flow, unittest/fx_passes/bert.py:
+    frontend, decomposition, CSE, fusion, default_partition): projections with
+    bias / residual / GELU epilogues, batched QK^T and PV products with their
+    permutes and the 1/sqrt(d) scale, softmax and softmax backward, both layer
+    norms with weight and bias, all as fused launches.  Loss and gradients
+    against the same model in fp32."""
+    import copy
+    from evt_ae_amd.aot_helper import aot_capture, aot_optimize
+    model, (x, target) = W.encoder_layer(device="cuda")
+    box = aot_capture(copy.deepcopy(model), (x, target))
+    kinds = [type(n.target).__name__ for n in fused_nodes(box["fw"])] + [type(n.target).__name__ for n in fused_nodes(box["bw"])]
+    assert kinds.count("FusedGEMM") >= 10 and kinds.count("FusedBMM") >= 6
+    assert {"FusedSoftmax", "FusedSoftmaxBackward", "FusedLayerNorm"} <= set(kinds)
+    master = copy.deepcopy(model).float()
+    ref_loss = master(x.float(), target)
+    ref_grads = torch.autograd.grad(ref_loss, list(master.parameters()))
+    eager = copy.deepcopy(model)
+    eager(x, target).backward()
+    compiled = aot_optimize(model)
+    loss = compiled(x, target)
+    loss.backward()
+    torch.cuda.synchronize()
+    assert abs(float(loss) - float(ref_loss)) <= 5e-3 * abs(float(ref_loss)), (float(loss), float(ref_loss))
+    for (name, p), g32, pe in zip(model.named_parameters(), ref_grads, eager.parameters()):
+        assert p.grad is not None and p.grad.shape == g32.shape
+        err = float((p.grad.float() - g32).norm() / g32.norm())
+        err_eager = float((pe.grad.float() - g32).norm() / g32.norm())
+        # no worse than the fp16 eager run of the same model (whose own rounding sets the scale), within 2e-2
+        assert err <= max(2e-2, 2.0 * err_eager), f"{name}: norm-wise error {err:.3e} (eager fp16: {err_eager:.3e})"
