@@ -124,6 +124,8 @@ class Codegen:
                 vm, vn = False, False
             elif n.op == "rowval":      # per-row value an anchor hands over (layer norm: mean, rstd)
                 vm, vn = True, False
+            elif n.op == "anchorval":   # further per-element value of a row-wise anchor (layer norm backward: g, xhat)
+                vm, vn = True, True
             else:
                 vm = any(self.var_m[i] for i in n.inputs)
                 vn = any(self.var_n[i] for i in n.inputs)
@@ -711,6 +713,7 @@ class RowCodegen(Codegen):
         for n in ir.nodes.values():
             if n.op == "colidx" or (n.op == "load" and ir.slots[n.slot].kind == "rand"):
                 raise NotImplementedError(f"{n.op} behind a row-wise anchor")
+        self.anchor_values = 1 + max([n.comp for n in ir.nodes.values() if n.op == "anchorval"], default=-1)
         # [N] vectors shared by every row (weight, bias, ...): read once per wave, not once per row
         self.hoisted = [n.name for n in ir.nodes.values() if n.op == "load" and ir.slots[n.slot].kind == "row"
                         and ir.slots[n.slot].strides.stride_l == 0 and n.slot not in ir.anchor_slots]
@@ -752,6 +755,7 @@ class RowCodegen(Codegen):
         e("}")
         e("template <class Cfg, bool FAST, class Ctx>")
         e(f"static EVT_DEV void row(const Params& p, const Ctx& t, const float (&acc)[Cfg::CH][8], const float (&rv)[2], "
+          f"const float (&av)[{max(self.anchor_values, 1)}][Cfg::CH][8], "
           f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8], float (&cst)[{max(ir.col_state, 1)}][Cfg::CH][8]) {{")
         e.indent()
         for k, s in enumerate(ir.slots):
@@ -782,6 +786,8 @@ class RowCodegen(Codegen):
             e(f"float {c}[8];")
             if n.op == "accum":
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = acc[c][j];")
+            elif n.op == "anchorval":
+                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = av[{n.comp}][c][j];")
             elif n.op == "load" and name in self.hoisted:
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
             elif n.op == "load":
@@ -819,7 +825,7 @@ class RowCodegen(Codegen):
                 e(f"evt::st_f32(p.t{s.slot}, o_{s.slot}, {_cname(s.input)});")
             e.dedent()
             e("}")
-        e("(void)p; (void)t; (void)acc; (void)rv; (void)hz; (void)cst;")
+        e("(void)p; (void)t; (void)acc; (void)rv; (void)av; (void)hz; (void)cst;")
         e.dedent()
         e("}")
 
@@ -868,7 +874,7 @@ class RowCodegen(Codegen):
         self.emit_row(e)
         e.dedent()
         e("};")
-        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}>;")
+        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}, {self.anchor_values}>;")
         e(f"constexpr int kNumTensors = {len(ir.slots)};")
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
         e(f"constexpr int kEltBytes = {4 if sp.elt == 'f32' else 2};")

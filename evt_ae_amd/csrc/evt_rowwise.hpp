@@ -42,9 +42,11 @@ struct RowArgs {
 };
 
 // ELT: 0 = f16, 1 = bf16, 2 = f32 element type of the anchor operands
-template <int OP_, int CH_, int LPR_, int ELT_, int WAVES_ = 4>
+// AV: per-element values besides the result that the anchor hands to the epilogue (layer norm backward with
+// weight / bias gradients: the incoming gradient and the normalised input)
+template <int OP_, int CH_, int LPR_, int ELT_, int AV_ = 0, int WAVES_ = 4>
 struct RowCfg {
-  static constexpr int OP = OP_, CH = CH_, LPR = LPR_, ELT = ELT_, WAVES = WAVES_;
+  static constexpr int OP = OP_, CH = CH_, LPR = LPR_, ELT = ELT_, AV = AV_, WAVES = WAVES_;
   static constexpr int THREADS = WAVES * 64;
   static constexpr int RPW = 64 / LPR;        // rows per wave
   static constexpr int ROWS = WAVES * RPW;    // rows per workgroup
@@ -282,7 +284,7 @@ EVT_DEV void row_widen(const typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8], f
 
 template <class Cfg>
 EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>& raw, const float (&gz)[Cfg::CH][8],
-                      float (&acc)[Cfg::CH][8], float (&rv)[2]) {
+                      float (&acc)[Cfg::CH][8], float (&rv)[2], float (&av)[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8]) {
   constexpr int CH = Cfg::CH, LPR = Cfg::LPR;
   const float rn = 1.f / (float)g.N;
   if constexpr (Cfg::OP == ROW_SOFTMAX) {
@@ -359,6 +361,12 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
     //   (g already multiplied by the weight when there is one)
     float xh[CH][8];
     row_widen<Cfg>(raw.a, acc);
+    if constexpr (Cfg::AV >= 1) {      // the weight / bias gradients are column sums of g * xhat and of g
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) av[0][c][j] = acc[c][j];
+    }
     if (g.gamma) {
 #pragma unroll
       for (int c = 0; c < CH; ++c)
@@ -384,8 +392,15 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
     for (int c = 0; c < CH; ++c)
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[c][j] = rstd * (acc[c][j] - s1 - xh[c][j] * s2);
+    if constexpr (Cfg::AV >= 2) {
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) av[1][c][j] = xh[c][j];
+    }
     rv[0] = mean; rv[1] = rstd;
   }
+  (void)av;
 }
 
 // Each wave walks rows first, first + stride, ... (stride = all waves of the
@@ -456,8 +471,9 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
       }
       float acc[Cfg::CH][8];
       float rv[2];
-      row_main<Cfg>(g, here, cur, gz, acc, rv);
-      if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, hz, cst);
+      float av[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8];
+      row_main<Cfg>(g, here, cur, gz, acc, rv, av);
+      if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, av, hz, cst);
       if (!more) break;
       cur = ahead;
       base = next;

@@ -570,16 +570,18 @@ class FusedLayerNorm(FusedRowOp):
 
 
 class FusedLayerNormBackward(FusedRowOp):
-    """Input gradient of aten.native_layer_norm_backward (output mask
-    [True, False, False]) + epilogue; operands: gradient, forward input, mean,
-    rstd and optionally the weight (reference: evt_fuser.py:905-970)."""
+    """aten.native_layer_norm_backward + epilogue: the input gradient and, when
+    the output mask asks for them, the weight and bias gradients as per-column
+    sums of the same pass; operands: gradient, forward input, mean, rstd and
+    optionally the weight (reference: evt_fuser.py:905-970, input gradient only)."""
     __name__ = "cutlass_layernorm_backward_with_visitor"
     target = aten.native_layer_norm_backward
     row_op = "layernorm_backward"
 
     def anchor_eager(self, grad, x, mean, rstd, gamma=None):
-        return aten.native_layer_norm_backward(grad, x, list(self.node.args[2]), mean, rstd, gamma, None,
-                                               [True, False, False])
+        mask = [bool(b) for b in self.node.args[7]]
+        bias = torch.zeros_like(gamma) if (gamma is not None and mask[2]) else None
+        return aten.native_layer_norm_backward(grad, x, list(self.node.args[2]), mean, rstd, gamma, bias, mask)
 
 
 
@@ -809,8 +811,12 @@ class EVTFuser:
             self.pending_coords[anchor] = {1: stat, 2: stat}
         else:
             grad, xin, _, mean, rstd, gamma, _beta, mask = anchor.args[:8]
-            if [bool(b) for b in mask] != [True, False, False]:
-                raise NotImplementedError(f"{anchor.name}: only the input gradient is computed (mask [True, False, False])")
+            mask = [bool(b) for b in mask]
+            if not mask[0]:
+                raise NotImplementedError(f"{anchor.name}: the input gradient is always computed")
+            if (mask[1] or mask[2]) and L != 1:
+                # weight / bias gradients are sums over every row: one batch of rows
+                raise NotImplementedError(f"{anchor.name}: weight / bias gradients need the rows as one batch")
             self.anchor_operands = [grad, xin, mean, rstd] + ([gamma] if gamma is not None else [])
             for node_, st_, dt_, kind_ in ((mean, Strides(M, 1, 0), "f32", "col"), (rstd, Strides(M, 1, 0), "f32", "col")):
                 if node_shape_dtype(node_)[1] != torch.float32:
@@ -825,6 +831,24 @@ class EVTFuser:
                 self.ir.anchor_slots.append(k)
             self.anchor_slot_nodes = [mean, rstd] + ([gamma] if gamma is not None else [])
             self.pending_multi[anchor] = {0: "accum"}
+            if mask[1] or mask[2]:
+                # dweight = sum_rows g * xhat, dbias = sum_rows g: per-column reductions of two more per-element
+                # values the anchor hands to the epilogue (the incoming gradient and the normalised input)
+                self.ir.add_node(IRNode("ln_g", "anchorval", domain="tile", comp=0))
+                self.ir.add_node(IRNode("ln_xhat", "anchorval", domain="tile", comp=1))
+                per_column = full.reduce(list(range(rank - 1)), False)
+                self.pending_coords[anchor] = {}
+                if mask[1]:
+                    self.ir.add_compute("ln_gx", "mul", ["ln_g", "ln_xhat"])
+                    self.ir.add_reduce("ln_dw_red", "sum", "col", "ln_gx")
+                    self.ir.add_node(IRNode("ln_dw", "rres", domain="col", reduce="ln_dw_red", comp=0))
+                    self.pending_multi[anchor][1] = "ln_dw"
+                    self.pending_coords[anchor][1] = per_column
+                if mask[2]:
+                    self.ir.add_reduce("ln_db_red", "sum", "col", "ln_g")
+                    self.ir.add_node(IRNode("ln_db", "rres", domain="col", reduce="ln_db_red", comp=0))
+                    self.pending_multi[anchor][2] = "ln_db"
+                    self.pending_coords[anchor][2] = per_column
 
     @staticmethod
     def _extract_reference(graph_module: GraphModule, anchor: Node, epilogue_partition, inputs, outputs) -> GraphModule:

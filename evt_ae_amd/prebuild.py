@@ -64,8 +64,11 @@ def register_all() -> List[jit.LazyModule]:
     for name, (cls, shapes, _) in W.ROW_BENCH.items():
         W.fuse(cls(), [torch.empty(sh, dtype=dt, device="meta") for sh, dt in shapes])
     from .aot_helper import aot_capture, evt_backend
+    # traced on the meta device: its dtype rules are the GPU's (fp32 layer norm statistics for fp16 inputs), so the
+    # modules registered here are the ones a GPU run asks for
+    aot_capture(*W.mlp_classifier(device="meta"))
     aot_capture(*W.mlp_classifier())
-    aot_capture(*W.encoder_layer())
+    aot_capture(*W.encoder_layer(device="meta"))
     # the same step through torch.compile: Dynamo's graph differs slightly, so
     # its kernels are registered as well (tracing stops at the first launch
     # when there is no GPU)

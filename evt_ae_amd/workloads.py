@@ -698,6 +698,15 @@ class LayerNormBackwardColumnSum(torch.nn.Module):   # layernorm_backward.py:31-
         return getitem, view_282, sum_13
 
 
+class LayerNormBackwardFull(torch.nn.Module):
+    """Input, weight and bias gradients of a layer norm in one pass (the
+    reference computes the input gradient only, evt_fuser.py:905-970)."""
+    def forward(self, grad, input, mean, invstd, gamma, beta, ge_1):
+        ln = aten.native_layer_norm_backward(grad, input, [1024], mean, invstd, gamma, beta, [True, True, True])
+        dx = aten.mul(operator.getitem(ln, 0), ge_1)
+        return dx, operator.getitem(ln, 1), operator.getitem(ln, 2)
+
+
 def _softmax_out(g, shape):
     return torch.softmax(_h(g, shape).float(), -1).half()
 
@@ -725,6 +734,7 @@ ROW_ANCHOR_PATTERNS = {
     "layernorm2": (LayerNormPattern2, lambda g: [_h(g, (512, 2, 1024)) + 1., _h(g, (1024,)), _h(g, (1024,))]),
     "layernorm_backward": (LayerNormBackwardMasked, _ln_backward_inputs),
     "layernorm_backward_column_sum": (LayerNormBackwardColumnSum, _ln_backward_inputs),
+    "layernorm_backward_full": (LayerNormBackwardFull, _ln_backward_inputs),
 }
 
 
