@@ -231,6 +231,73 @@ def bench_row_anchors(torch, W, steps, warmup):
     return out
 
 
+def bench_encoder_step(torch, W, iters=20):
+    """One training step (forward + backward) of a BERT-large encoder layer in
+    fp16, through AOT autograd with every GEMM / BMM / softmax / layer norm
+    fused, against the same model run eagerly; both also replayed from a HIP
+    graph, which removes the host-side launch cost of either."""
+    import copy
+    from evt_ae_amd.aot_helper import aot_optimize
+    model, (x, target) = W.encoder_layer(device="cuda", **W.ENCODER_BENCH)
+    eager = copy.deepcopy(model)
+    fused = aot_optimize(model)
+
+    def run(fn, params):
+        def step():
+            for p in params:
+                p.grad = None
+            fn(x, target).backward()
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        loop_ms = e0.elapsed_time(e1) / iters
+        graph_ms = None
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            for p in params:
+                p.grad = None
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn(x, target).backward()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(iters):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            graph_ms = e0.elapsed_time(e1) / iters
+        except Exception as exc:
+            log(f"[bench] encoder step: graph capture unavailable: {exc!r}")
+            torch.cuda.synchronize()
+        return loop_ms, graph_ms
+
+    e_loop, e_graph = run(eager, list(eager.parameters()))
+    f_loop, f_graph = run(fused, list(model.parameters()))
+    ref = [p.grad.float() for p in eager.parameters()]
+    got = [p.grad.float() for p in model.parameters()]
+    err = max(float((a - b).norm() / b.norm().clamp_min(1e-30)) for a, b in zip(got, ref))
+    best_e = min(t for t in (e_loop, e_graph) if t)
+    best_f = min(t for t in (f_loop, f_graph) if t)
+    out = {"model": "post-LN encoder layer", **W.ENCODER_BENCH, "dtype": "f16",
+           "fused_ms": round(f_loop, 4), "fused_graph_ms": None if f_graph is None else round(f_graph, 4),
+           "eager_ms": round(e_loop, 4), "eager_graph_ms": None if e_graph is None else round(e_graph, 4),
+           "speedup_vs_eager": round(best_e / best_f, 3), "max_grad_normwise_diff_vs_eager": err}
+    log(f"[bench] encoder layer training step: {out}")
+    return out
+
+
 def cpu_baseline(torch, W, evt_oracle, cfgs, reps=3):
     """PyTorch fp32 eager evaluation of the same subgraphs on the host cores."""
     torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
@@ -274,6 +341,8 @@ def main():
                     help="timed regions of --steps launches per config; the median is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-encoder-step", dest="encoder_step", action="store_false",
+                    help="skip the fused-vs-eager training step of an encoder layer (encoder_layer_step in the output)")
     ap.add_argument("--no-row-anchors", dest="row_anchors", action="store_false",
                     help="skip the bandwidth measurement of the softmax / layer norm anchors (row_anchors in the output)")
     ap.add_argument("--configs", default="1,2,3,4,5")
@@ -408,6 +477,7 @@ def main():
         "cpu_baseline": cpu,
         "per_config": details,
         "row_anchors": bench_row_anchors(torch, W, max(20, args.steps // 4), 5) if args.row_anchors else None,
+        "encoder_layer_step": bench_encoder_step(torch, W) if args.encoder_step else None,
     }
     print(json.dumps(line), flush=True)
 

@@ -519,22 +519,39 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
   }
 }
 
-// second phase of the per-column reductions: one thread per column adds the workgroups' partials in
-// workgroup order and evaluates the per-column output expressions
+// Second phase of the per-column reductions.  A workgroup owns 64 columns; its 16 waves each add every 16th
+// workgroup partial of those columns (coalesced 256-byte reads, independent loads), then one wave adds the 16
+// sub-sums in wave order and evaluates the per-column output expressions.  The order of the additions is fixed
+// by (partial index mod 16, then wave), so results do not depend on timing.
 template <class Epi>
-__global__ __launch_bounds__(256) void evt_row_col_finalize_kernel(RowArgs g, typename Epi::Params p, int blocks) {
+__global__ __launch_bounds__(1024) void evt_row_col_finalize_kernel(RowArgs g, typename Epi::Params p, int blocks) {
   constexpr int CS = Epi::COL_STATE > 0 ? Epi::COL_STATE : 1;
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= g.N) return;
+  __shared__ float part[16][CS][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * 64 + lane;
   float a[CS];
   Epi::col_identity(a);
-  for (int b = 0; b < blocks; ++b) {
-    float x[CS];
+  if (n < g.N) {
+    for (int b = wave; b < blocks; b += 16) {
+      float x[CS];
 #pragma unroll
-    for (int k = 0; k < CS; ++k) x[k] = g.colws[((int64_t)b * CS + k) * g.N + n];
-    Epi::col_combine(a, x);
+      for (int k = 0; k < CS; ++k) x[k] = g.colws[((int64_t)b * CS + k) * g.N + n];
+      Epi::col_combine(a, x);
+    }
   }
-  Epi::col_finalize(p, 0, n, a);
+#pragma unroll
+  for (int k = 0; k < CS; ++k) part[wave][k][lane] = a[k];
+  __syncthreads();
+  if (wave == 0 && n < g.N) {
+#pragma unroll
+    for (int w = 1; w < 16; ++w) {
+      float x[CS];
+#pragma unroll
+      for (int k = 0; k < CS; ++k) x[k] = part[w][k][lane];
+      Epi::col_combine(a, x);
+    }
+    Epi::col_finalize(p, 0, n, a);
+  }
 }
 
 }  // namespace evt

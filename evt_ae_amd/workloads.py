@@ -869,10 +869,14 @@ class EncoderLayer(torch.nn.Module):
         return ((x.float() - target) ** 2).sum()
 
 
-def encoder_layer(seed: int = 0, device: str = "cpu", dtype=torch.float16):
-    """(model, (x, target)) with seeded parameters and inputs: batch 8, sequence 128, width 256."""
+ENCODER_BENCH = dict(d=1024, heads=16, ffn=4096, batch=8, seq=512)     # a BERT-large layer
+
+
+def encoder_layer(seed: int = 0, device: str = "cpu", dtype=torch.float16, d: int = 256, heads: int = 4,
+                  ffn: int = 1024, batch: int = 8, seq: int = 128):
+    """(model, (x, target)) with seeded parameters and inputs (default: batch 8, sequence 128, width 256)."""
     g = torch.Generator(device="cpu").manual_seed(0xE9C + seed)
-    model = EncoderLayer()
+    model = EncoderLayer(d, heads, ffn)
     with torch.no_grad():
         for name, p in model.named_parameters():
             if p.dim() == 2:
@@ -882,8 +886,8 @@ def encoder_layer(seed: int = 0, device: str = "cpu", dtype=torch.float16):
             else:
                 p.copy_(0.02 * torch.randn(p.shape, generator=g))
     model = model.to(dtype).to(device)
-    x = torch.randn(8, 128, 256, generator=g).to(dtype).to(device)
-    target = torch.randn(8, 128, 256, generator=g).to(device)
+    x = torch.randn(batch, seq, d, generator=g).to(dtype).to(device)
+    target = torch.randn(batch, seq, d, generator=g).to(device)
     return model, (x, target)
 
 
