@@ -576,7 +576,27 @@ class Codegen:
         e("// few partials: the last workgroup to arrive combines them; many: a finalize kernel does")
         e("g.row_inkernel = (g.tiles_n * g.row_fold_count <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
         e("g.col_inkernel = (g.tiles_m <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
-        e("if ((int64_t)g.tiles_m * g.tiles_n * a->L > 0x7fffffffLL) return EVT_ERR_RANGE;")
+        e("// Split-K: when the output tiles cannot fill the chip and K is long, several workgroups share a tile")
+        e("// (EVT_SPLIT_K=1 turns this off, EVT_SPLIT_K=n asks for n splits)")
+        e("g.splits = 1; g.k_chunk = (a->K + Cfg::BK - 1) / Cfg::BK * Cfg::BK;")
+        if t.stages > 1:
+            e("{")
+            e("  const char* env = getenv(\"EVT_SPLIT_K\");      // read per call: a caller may switch it between launches")
+            e("  const int want = env ? atoi(env) : 0;")
+            e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
+              "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
+            e("  const int kt = (a->K + Cfg::BK - 1) / Cfg::BK;")
+            e("  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * a->L;")
+            e("  int s = 1;")
+            e("  if (want > 1) s = want < kt ? want : kt;")
+            e("  else if (want == 0 && tiles * 2 <= cus && kt >= 8) { s = (int)(cus / tiles); if (s > 8) s = 8; if (s > kt / 4) s = kt / 4; }")
+            e("  if (s >= 2) {")
+            e("    const int chunk = (kt + s - 1) / s;")
+            e("    g.splits = (kt + chunk - 1) / chunk;      // every split has work")
+            e("    g.k_chunk = chunk * Cfg::BK;")
+            e("  }")
+            e("}")
+        e("if ((int64_t)g.tiles_m * g.tiles_n * a->L * g.splits > 0x7fffffffLL) return EVT_ERR_RANGE;")
         e("if (a->N > (1 << 24)) return EVT_ERR_RANGE;   // column indices are carried as fp32")
         if t.stages == 1:
             e("if (a->K > Cfg::BK) return EVT_ERR_RANGE;   // single-stage variant: K must fit one tile")
@@ -628,7 +648,7 @@ class Codegen:
         e("  evt::GemmArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  return evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
+        e("  return evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
         e("}")
         e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
         e("  if (bytes <= 0) return EVT_OK;")
@@ -641,10 +661,10 @@ class Codegen:
         e("  evt::GemmArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  const int64_t need = evt::ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
+        e("  const int64_t need = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
         e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
         e("  g.workspace = (char*)ws;")
-        e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L);")
+        e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L * g.splits);")
         e("  hipLaunchKernelGGL((evt::evt_gemm_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  const int err = (int)hipGetLastError();")
         e("  if (err != 0) return err;")

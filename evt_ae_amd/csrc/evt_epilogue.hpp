@@ -340,7 +340,8 @@ constexpr int kMaxInKernelPartials = 64;
 
 struct WsLayout {
   int64_t counter_bytes, row_bytes, col_bytes;
-  __host__ __device__ int64_t total() const { return counter_bytes + row_bytes + col_bytes; }
+  int64_t split_counter_bytes, split_bytes;     // split-K: one arrival counter per tile, one accumulator tile per split
+  __host__ __device__ int64_t total() const { return counter_bytes + row_bytes + col_bytes + split_counter_bytes + split_bytes; }
 };
 
 // a per-row reduction goes through the workspace when several tiles span the
@@ -356,6 +357,18 @@ __host__ __device__ inline WsLayout ws_layout(const GemmArgs& g) {
   w.counter_bytes = (ncnt * 4 + 255) / 256 * 256;
   w.row_bytes = row ? ((int64_t)g.L * g.tiles_n * g.M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
   w.col_bytes = col ? ((int64_t)g.L * g.tiles_m * g.N * COL_STATE * 4 + 255) / 256 * 256 : 0;
+  w.split_counter_bytes = w.split_bytes = 0;
+  return w;
+}
+// with the split-K regions, which need the tile size
+template <class Cfg, int ROW_STATE, int COL_STATE>
+__host__ __device__ inline WsLayout ws_layout_split(const GemmArgs& g) {
+  WsLayout w = ws_layout<ROW_STATE, COL_STATE>(g);
+  if (g.splits > 1) {
+    const int64_t tiles = (int64_t)g.L * g.tiles_m * g.tiles_n;
+    w.split_counter_bytes = (tiles * 4 + 255) / 256 * 256;
+    w.split_bytes = tiles * g.splits * Cfg::BM * Cfg::BN * 4;
+  }
   return w;
 }
 
@@ -716,12 +729,51 @@ template <class Cfg, class Epi>
 __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
   __shared__ __attribute__((aligned(1024))) char smem[Cfg::LDS_BYTES];
   int batch, tm, tn;
-  tile_coords<Cfg::GROUP_M>(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
+  const int split = g.splits > 1 ? (int)(blockIdx.x % (unsigned)g.splits) : 0;
+  const unsigned tile_id = g.splits > 1 ? blockIdx.x / (unsigned)g.splits : blockIdx.x;
+  tile_coords<Cfg::GROUP_M>(tile_id, g.splits > 1 ? gridDim.x / (unsigned)g.splits : gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
   f32x16 acc[Cfg::MI][Cfg::NI];
 #ifdef EVT_CLOCK_PROBE
   const uint64_t probe_c0 = __builtin_amdgcn_s_memtime(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
-  Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, smem, acc);
+  Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, split, smem, acc);
+  if (g.splits > 1) {
+    // Split-K exchange.  Every workgroup of the tile leaves its accumulators in the workspace in register
+    // order (consecutive lanes write consecutive words); the one whose ticket is the last reads all of them
+    // back in split order -- its own included, so the sum does not depend on who arrived last -- and goes on
+    // to the epilogue; the others are done.
+    const WsLayout wl = ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g);
+    char* region = g.workspace + wl.counter_bytes + wl.row_bytes + wl.col_bytes;
+    int* counter = (int*)region + tile_id;
+    constexpr int REGS = Cfg::MI * Cfg::NI * 16;
+    float* part = (float*)(region + wl.split_counter_bytes) + (int64_t)tile_id * g.splits * REGS * Cfg::THREADS;
+    float* mine = part + (int64_t)split * REGS * Cfg::THREADS + threadIdx.x;
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st_device(mine + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS, acc[mi][ni][v]);
+    __syncthreads();                 // nobody still reads operand tiles from the LDS the flag lives in
+    if (!arrive_last(counter, g.splits, (int*)smem)) return;
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
+    for (int sp = 0; sp < g.splits; ++sp) {
+      const float* src = part + (int64_t)sp * REGS * Cfg::THREADS + threadIdx.x;
+#pragma unroll
+      for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[mi][ni][v] += ld_device(src + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch
+  }
 #ifdef EVT_CLOCK_PROBE
   const uint64_t probe_c1 = __builtin_amdgcn_s_memtime(), probe_r1 = __builtin_amdgcn_s_memrealtime();
 #endif

@@ -61,6 +61,10 @@ struct GemmArgs {
   // (result keyed by l % row_fold_step), otherwise row_fold_count consecutive
   // ones (keyed by l / row_fold_count).  (0, 1, 1): every batch on its own.
   int row_fold_mod, row_fold_step, row_fold_count;
+  // Split-K: `splits` workgroups share an output tile, each over `k_chunk` (a multiple of BK) of the K extent;
+  // they leave their accumulators in the workspace and the last one to arrive adds them up in split order and
+  // runs the epilogue.  splits == 1: one workgroup per tile, nothing goes through the workspace.
+  int splits, k_chunk;
 };
 
 // Compile-time description of one kernel variant.
@@ -714,7 +718,7 @@ struct Mainloop {
     wait_vmcnt<0>();                // the zero-fill transfers past the last tile have landed
   }
 
-  static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, char* smem,
+  static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, int split, char* smem,
                           f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -724,11 +728,15 @@ struct Mainloop {
     OpA a;
     OpB b;
     {
-      const char* pa = g.A + ((int64_t)batch * g.bsA + (Cfg::A_KC ? (int64_t)m0 * g.lda : (int64_t)m0)) * 2;
-      const char* pb = g.B + ((int64_t)batch * g.bsB + (Cfg::B_KC ? (int64_t)n0 * g.ldb : (int64_t)n0)) * 2;
-      a.init(pa, g.lda, g.M - m0, g.K, tid);
-      b.init(pb, g.ldb, g.N - n0, g.K, tid);
+      // this workgroup's share of K: [k_lo, k_lo + Kw)
+      const int k_lo = split * g.k_chunk;
+      const int Kw_ = g.K - k_lo < g.k_chunk ? g.K - k_lo : g.k_chunk;
+      const char* pa = g.A + ((int64_t)batch * g.bsA + (Cfg::A_KC ? (int64_t)m0 * g.lda + k_lo : (int64_t)m0 + (int64_t)k_lo * g.lda)) * 2;
+      const char* pb = g.B + ((int64_t)batch * g.bsB + (Cfg::B_KC ? (int64_t)n0 * g.ldb + k_lo : (int64_t)n0 + (int64_t)k_lo * g.ldb)) * 2;
+      a.init(pa, g.lda, g.M - m0, Kw_, tid);
+      b.init(pb, g.ldb, g.N - n0, Kw_, tid);
     }
+    const int Kw = (g.K - split * g.k_chunk < g.k_chunk) ? g.K - split * g.k_chunk : g.k_chunk;
     RdA ra;
     RdB rb;
     ra.init(wm * Cfg::TM, lane);
@@ -741,7 +749,7 @@ struct Mainloop {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
 
-    const int KT = (g.K + Cfg::BK - 1) / Cfg::BK;
+    const int KT = (Kw + Cfg::BK - 1) / Cfg::BK;
 
     if constexpr (Cfg::PIPE == 1) {
       run_lookahead(a, b, ra, rb, smem, wave, KT, acc);

@@ -167,6 +167,14 @@ GOLDEN_SHAPES = {
 }
 # several workgroup tiles in M and N, several k-tiles with a K tail: the shapes
 # the main-loop pipeline variants (PIPELINE_TILES) are checked on
+# few output tiles and a long K: the kernels split K over several workgroups per tile (K tail included)
+SPLIT_K_SHAPES = {
+    1: dict(M=264, N=200, K=2120),
+    3: dict(M=136, N=520, K=4168),
+    4: dict(M=520, N=136, K=3080),
+    5: dict(M=72, N=1032, K=2056),
+}
+
 PIPELINE_SHAPES = {
     1: dict(M=300, N=264, K=200),
     2: dict(L=2, S=200, D=72),

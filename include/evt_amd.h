@@ -118,7 +118,9 @@ const char* evt_module_spec(void);
 /* Bytes of device workspace `evt_launch` needs for these arguments (0 when the
  * epilogue has no reduction that spans several workgroup tiles).  It holds the
  * per-tile partial results of the two-phase reduction and one arrival counter
- * per row / column block.  The counters must be zero before the first launch
+ * per row / column block; when the module splits K over several workgroups per
+ * output tile (few tiles, long K) also one fp32 accumulator tile per split and
+ * one counter per tile.  The counters must be zero before the first launch
  * (evt_workspace_init) and every launch leaves them zero; launches that share
  * a workspace must not overlap in time.  Takes the place of the host-side
  * pre-zeroing of reduction outputs (evt_fuser.py:217-225). */

@@ -435,3 +435,46 @@ def test_aot_encoder_layer_training_step():
         err_eager = float((pe.grad.float() - g32).norm() / g32.norm())
         # no worse than the fp16 eager run of the same model (whose own rounding sets the scale), within 2e-2
         assert err <= max(2e-2, 2.0 * err_eager), f"{name}: norm-wise error {err:.3e} (eager fp16: {err_eager:.3e})"
+
+
+@pytest.mark.parametrize("cfg", list(W.SPLIT_K_SHAPES))
+def test_split_k(cfg, monkeypatch):
+    """Few output tiles and a long K: several workgroups share a tile, leave their
+    accumulators in the workspace and the last to arrive adds them in split order
+    and runs the epilogue (with its own per-row / per-column reductions).  Checked
+    against the oracle with the automatic split, with a forced odd split and with
+    splitting off; repeated launches are bit-identical (the order of the sum is
+    fixed), and the automatic choice really splits."""
+    shapes = W.SPLIT_K_SHAPES[cfg]
+    wl = W.CONFIGS[cfg]
+    inputs = W.make_inputs(cfg, shapes)
+    refs = evt_oracle.eval_fp32(wl.module(), inputs)
+    dev = [t.cuda() for t in inputs]
+    gm = W.fuse(wl.module(), inputs)
+    (node,) = fused_nodes(gm)
+    op = node.target
+    results = {}
+    for mode in ("auto", "3", "1"):
+        if mode == "auto":
+            monkeypatch.delenv("EVT_SPLIT_K", raising=False)
+        else:
+            monkeypatch.setenv("EVT_SPLIT_K", mode)
+        op._workspace.clear()                       # sized for the split in force
+        outs = gm(*dev)
+        outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+        torch.cuda.synchronize()
+        _compare(wl, outs, refs)
+        again = gm(*dev)
+        again = list(again) if isinstance(again, (tuple, list)) else [again]
+        torch.cuda.synchronize()
+        for a, b in zip(outs, again):
+            assert torch.equal(a, b), f"config {cfg} split {mode}: launches differ"
+        results[mode] = [o.clone() for o in outs]
+        if cfg == 1:        # no reduction in this epilogue: a workspace exists exactly when K is split
+            assert bool(op._workspace) == (mode != "1"), mode
+    monkeypatch.delenv("EVT_SPLIT_K", raising=False)
+    tile = op.tile
+    tiles = -(-op.problem[0] // tile.bm) * -(-op.problem[1] // tile.bn)
+    assert tiles * 2 <= 256 and op.problem[2] >= 8 * tile.bk
+    for o_auto, o_off in zip(results["auto"], results["1"]):
+        assert evt_oracle.max_rel_err(o_auto, o_off.float()) <= 1e-2
