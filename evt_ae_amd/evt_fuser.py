@@ -988,12 +988,8 @@ class EVTFuser:
             sshape, _ = node_shape_dtype(src)
             return self._materialize(src, coord.inverse_permute([int(i) for i in node.args[1]], sshape))
         # elementwise on small tensors: evaluate per element from its operands
-        saved = (self.coords.get(node), )
         self.coords[node] = coord
-        try:
-            self.visit(node)
-        finally:
-            pass
+        self.visit(node)
         return self.ir_name[node]
 
     # -- node visitors (reference vocabulary: evt_fuser.py:1308-1485) ----------------
