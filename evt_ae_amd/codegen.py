@@ -589,7 +589,10 @@ class Codegen:
             e("  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * a->L;")
             e("  int s = 1;")
             e("  if (want > 1) s = want < kt ? want : kt;")
-            e("  else if (want == 0 && tiles * 2 <= cus && kt >= 8) { s = (int)(cus / tiles); if (s > 8) s = 8; if (s > kt / 4) s = kt / 4; }")
+            e("  // automatic: only small outputs -- every split writes and the last arriver reads a whole fp32 tile, which")
+            e("  // costs more than the idle CUs once the output runs to megabytes")
+            e("  else if (want == 0 && tiles * 2 <= cus && kt >= 8 && (int64_t)a->M * a->N * a->L <= (1 << 20)) "
+              "{ s = (int)(cus / tiles); if (s > 8) s = 8; if (s > kt / 4) s = kt / 4; }")
             e("  if (s >= 2) {")
             e("    const int chunk = (kt + s - 1) / s;")
             e("    g.splits = (kt + chunk - 1) / chunk;      // every split has work")
