@@ -4,6 +4,7 @@ ships next to its benchmarks, e.g. benchmark/bert/tuner_cache.db).
 
     python -m evt_ae_amd.autotuner.tune_workloads --build-only   # compile every candidate (no GPU needed)
     python -m evt_ae_amd.autotuner.tune_workloads [--cache FILE]  # time them on the GPU, store the best
+    ... --encoder [--short-list]   # also the GEMMs / batched products of the BERT-large encoder layer step
 """
 from __future__ import annotations
 
@@ -30,15 +31,50 @@ def _tuners():
     return out
 
 
+def _encoder_tuners():
+    """One tuner per distinct fused GEMM / BMM of the encoder layer's training
+    step at the benchmark's size (traced on the meta device: the GPU's dtypes)."""
+    from .. import workloads as W
+    from ..aot_helper import aot_capture
+    from ..autotuner.bmm_tuner import BMMTuner
+    from ..autotuner.gemm_tuner import MMTuner
+    from ..evt_fuser import FusedBMM, FusedGEMM
+    box = aot_capture(*W.encoder_layer(device="meta", **W.ENCODER_BENCH))
+    out, seen = [], set()
+    for node in W.fused_nodes(box["joint"]):
+        op = node.target
+        if not isinstance(op, (FusedGEMM, FusedBMM)):
+            continue
+        cls = BMMTuner if isinstance(op, FusedBMM) else MMTuner
+        t = cls(op.problem, op.a_kc, op.b_kc, op.spec.bf16, op.tile.dma, op.ir)
+        if t.key() not in seen:
+            seen.add(t.key())
+            out.append((f"encoder {op.problem}", t))
+    return out
+
+
+# the tiles that have won somewhere so far: a short list keeps the compile time of a new model's problems bounded
+SHORT_LIST = [(256, 256, 64, 4, 2, 2, 2), (256, 256, 64, 2, 4, 2, 3), (256, 256, 64, 4, 2, 2, 0), (256, 128, 64, 4, 2, 3, 3),
+              (256, 128, 64, 4, 2, 3, 2), (128, 256, 64, 2, 4, 3, 3), (128, 256, 64, 2, 4, 3, 2), (128, 128, 64, 2, 4, 4, 2),
+              (128, 128, 64, 4, 2, 2, 2), (128, 128, 64, 2, 4, 2, 3), (128, 128, 64, 2, 2, 2, 0), (64, 64, 64, 2, 2, 2, 0)]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--build-only", action="store_true")
+    ap.add_argument("--encoder", action="store_true", help="tune the encoder layer's problems instead of the five configs")
+    ap.add_argument("--short-list", action="store_true", help="only the tiles of SHORT_LIST")
     ap.add_argument("--cache", default=None, help="tuner cache file to write (default: the package's)")
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     args = ap.parse_args()
     # candidates must be enumerated without consulting an existing cache
     os.environ["EVT_TUNER_CACHE"] = "/nonexistent/tuner_cache.db"
-    tuners = _tuners()
+    tuners = _encoder_tuners() if args.encoder else _tuners()
+    if args.short_list:
+        for _, t in tuners:
+            full = t.candidates()
+            short = [c for c in full if (c.bm, c.bn, c.bk, c.wm, c.wn, c.stages, c.pipe) in SHORT_LIST]
+            t.candidates = (lambda s=short: s)
     from .. import jit
     from ..codegen import KernelSpec
     mods = []
