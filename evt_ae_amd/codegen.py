@@ -730,9 +730,13 @@ class RowCodegen(Codegen):
             # the row would be a second pass over the anchor's own axis
             if r.axis != "col" or r.kind not in ("sum", "max"):
                 raise NotImplementedError(f"per-row reduction {r.name} behind a row-wise anchor")
-        if ir.col_state and (ir.L != 1 or 4 * ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536):
+        if ir.col_state and (ir.L != 1 or ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536):
             raise NotImplementedError("per-column reduction behind a row-wise anchor: one batch and rows of at most "
-                                      f"{65536 // (16 * max(ir.col_state, 1))} elements")
+                                      f"{65536 // (4 * max(ir.col_state, 1))} elements")
+        # a kernel that reduces over the rows runs 8 waves per workgroup: as many rows in flight per CU from half
+        # the workgroups, so half the partials for the second phase (16 waves would cap a wave at 128 registers,
+        # which spills the layer norm backward kernel)
+        self.waves = 8 if ir.col_state else 4
         for n in ir.nodes.values():
             if n.op == "colidx" or (n.op == "load" and ir.slots[n.slot].kind == "rand"):
                 raise NotImplementedError(f"{n.op} behind a row-wise anchor")
@@ -897,7 +901,7 @@ class RowCodegen(Codegen):
         self.emit_row(e)
         e.dedent()
         e("};")
-        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}, {self.anchor_values}>;")
+        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}, {self.anchor_values}, {self.waves}>;")
         e(f"constexpr int kNumTensors = {len(ir.slots)};")
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
         e(f"constexpr int kEltBytes = {4 if sp.elt == 'f32' else 2};")
@@ -960,10 +964,10 @@ class RowCodegen(Codegen):
         e("// workgroups per CU before waves start walking over several rows (0: one pass, a workgroup per Cfg::ROWS rows);")
         e("// walking pays when row vectors are kept in registers across the rows of a wave, and bounds the number of")
         e("// partials of a per-column reduction")
-        default_cap = 8 if ir.col_state else (16 if self.hoisted else 0)
+        default_cap = 4 if ir.col_state else (16 if self.hoisted else 0)
         e("static unsigned grid_for(const evt::RowArgs& g) {")
         e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); int v = s ? atoi(s) : {default_cap}; "
-          f"return {'v > 0 ? v : 8' if ir.col_state else 'v'}; }}();")
+          f"return {'v > 0 ? v : 4' if ir.col_state else 'v'}; }}();")
         e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
           "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
         e("  const int64_t want = ((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS;")

@@ -481,9 +481,10 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
   }
   if constexpr (CS > 0) {
     // Column partials of the workgroup: first across the row groups of a wave (lanes that hold the same
-    // columns of different rows), then across the waves through LDS; one partial per (workgroup, column)
-    // goes to the workspace and a second kernel adds the workgroups up in a fixed order.
-    __shared__ float red[Cfg::WAVES][CS][Cfg::CH * Cfg::SPAN];
+    // columns of different rows), then across the waves, which add their share into one LDS copy one after
+    // the other in wave order; one partial per (workgroup, column) goes to the workspace and a second kernel
+    // adds the workgroups up in a fixed order.
+    __shared__ float red[CS][Cfg::CH * Cfg::SPAN];
 #pragma unroll
     for (int k = 0; k < CS; ++k)
 #pragma unroll
@@ -499,22 +500,33 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
             Epi::col_combine(a, b);
             x = a[k];
           }
-          if (lane < Cfg::LPR) red[wave][k][c * Cfg::SPAN + t.sub * 8 + j] = x;
+          cst[k][c][j] = x;
         }
-    __syncthreads();
-    for (int n = threadIdx.x; n < g.N; n += Cfg::THREADS) {
-      float a[CS];
+    for (int w = 0; w < Cfg::WAVES; ++w) {
+      if (wave == w && lane < Cfg::LPR) {
 #pragma unroll
-      for (int k = 0; k < CS; ++k) a[k] = red[0][k][n];
+        for (int c = 0; c < Cfg::CH; ++c)
 #pragma unroll
-      for (int w = 1; w < Cfg::WAVES; ++w) {
-        float b[CS];
+          for (int j = 0; j < 8; ++j) {
+            const int n = c * Cfg::SPAN + t.sub * 8 + j;
+            float a[CS], b[CS];
 #pragma unroll
-        for (int k = 0; k < CS; ++k) b[k] = red[w][k][n];
-        Epi::col_combine(a, b);
+            for (int k = 0; k < CS; ++k) { a[k] = red[k][n]; b[k] = cst[k][c][j]; }
+            if (w == 0) {
+#pragma unroll
+              for (int k = 0; k < CS; ++k) a[k] = b[k];
+            } else {
+              Epi::col_combine(a, b);
+            }
+#pragma unroll
+            for (int k = 0; k < CS; ++k) red[k][n] = a[k];
+          }
       }
+      __syncthreads();
+    }
+    for (int n = threadIdx.x; n < g.N; n += Cfg::THREADS) {
 #pragma unroll
-      for (int k = 0; k < CS; ++k) g.colws[((int64_t)blockIdx.x * CS + k) * g.N + n] = a[k];
+      for (int k = 0; k < CS; ++k) g.colws[((int64_t)blockIdx.x * CS + k) * g.N + n] = red[k][n];
     }
   }
 }

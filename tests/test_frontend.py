@@ -281,7 +281,7 @@ def test_row_anchor_patterns_trace(name):
     if kind == "layernorm_backward":
         assert [op.ir.slots[k].name for k in spec["anchor_tensors"]] == ["mean", "invstd", "gamma"]
     if name == "layernorm_backward_full":
-        assert L == 1 and spec["col_state"] == 2 and "Cfg = evt::RowCfg<3, 2, 64, 0, 2>" in op.module.source
+        assert L == 1 and spec["col_state"] == 2 and "Cfg = evt::RowCfg<3, 2, 64, 0, 2, 8>" in op.module.source
     if "column" in name and "broadcast" not in name and "full" not in name:
         # a sum over every row: one batch of L * M rows, partials per workgroup in the workspace
         assert L == 1 and spec["col_state"] == 1 and "sum" in " ".join(op.partition_names)
