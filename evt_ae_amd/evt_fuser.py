@@ -166,7 +166,7 @@ class FusedOpBase:
         Returns the block and the tensors it points into (keep them alive)."""
         M, N, K, L = self.problem
         A, lda, bsa, B, ldb, bsb = self.operands(args[-2], args[-1])
-        a = jit.EvtArgs()
+        a = self.argument_block()
         a.M, a.N, a.K, a.L = M, N, K, L
         a.A, a.lda, a.batch_stride_A = A.data_ptr(), lda, bsa
         a.B, a.ldb, a.batch_stride_B = B.data_ptr(), ldb, bsb
@@ -174,27 +174,41 @@ class FusedOpBase:
         self.fill_epilogue_arguments(a, keep, visitor_args, args)
         return a, keep
 
-    def fill_epilogue_arguments(self, a: jit.EvtArgs, keep: list, visitor_args: Dict[str, torch.Tensor], args) -> None:
-        """Tensor and scalar slots of the epilogue (shared by every anchor)."""
-        a.num_tensors = len(self.ir.slots)
-        a.num_scalars = len(self.ir.scalars)
-        for k, slot in enumerate(self.ir.slots):
-            ta = a.tensors[k]
-            if slot.kind == "rand":      # generated in the kernel: strides only
+    def argument_block(self) -> jit.EvtArgs:
+        """The op's argument block.  The launch call reads it before it returns, so
+        one block per op is reused from call to call; what never changes (slot
+        counts, strides, immediates) is written once."""
+        a = getattr(self, "_evt_args", None)
+        if a is None:
+            a = self._evt_args = jit.EvtArgs()
+            a.num_tensors = len(self.ir.slots)
+            a.num_scalars = len(self.ir.scalars)
+            for k, slot in enumerate(self.ir.slots):
+                ta = a.tensors[k]
                 ta.ptr = None
+                ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
+                ta.l_div = slot.strides.l_div
+                ta.l_mod = slot.strides.l_mod
+            for i, sc in enumerate(self.ir.scalars):
+                a.scalars[i] = sc
+            # per call: (slot, where its tensor comes from)
+            self._slot_plan = [(k, *self.slot_sources[k]) for k, slot in enumerate(self.ir.slots) if slot.kind != "rand"]
+        return a
+
+    def fill_epilogue_arguments(self, a: jit.EvtArgs, keep: list, visitor_args: Dict[str, torch.Tensor], args) -> None:
+        """Tensor pointers of the epilogue's slots (shared by every anchor); a
+        rand slot has no storage, its strides alone seed the generator."""
+        tensors = a.tensors
+        first_anchor = len(args) - self.num_anchor_inputs
+        for k, kind, ref in self._slot_plan:
+            if kind == "input":
+                t = args[ref]
+            elif kind == "anchor":
+                t = args[first_anchor + ref]
             else:
-                kind, ref = self.slot_sources[k]
-                if kind == "anchor":
-                    t = args[len(args) - self.num_anchor_inputs + ref]
-                else:
-                    t = args[ref] if kind == "input" else visitor_args[ref]
-                keep.append(t)
-                ta.ptr = t.data_ptr()
-            ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
-            ta.l_div = slot.strides.l_div
-            ta.l_mod = slot.strides.l_mod
-        for i, s in enumerate(self.ir.scalars):
-            a.scalars[i] = s
+                t = visitor_args[ref]
+            keep.append(t)
+            tensors[k].ptr = t.data_ptr()
         if self.ir.rng_scalar is not None:
             # 32-bit patterns, not float values: written through an integer view of the scalar array
             bits = (ctypes.c_uint32 * jit.EVT_MAX_SCALARS).from_buffer(a, jit.EvtArgs.scalars.offset)
@@ -207,7 +221,12 @@ class FusedOpBase:
     def workspace_for(self, a: jit.EvtArgs, stream, device) -> Tuple[int, int]:
         """Device workspace for cross-workgroup reductions, one per stream,
         zero-filled once (launches leave it clean)."""
-        ws_bytes = self.module.workspace_bytes(a)
+        # the size depends on the problem (fixed per op) and on the split-K switch, which may change between calls
+        mode = os.environ.get("EVT_SPLIT_K")
+        cached = getattr(self, "_ws_bytes", None)
+        if cached is None or cached[0] != mode:
+            cached = self._ws_bytes = (mode, self.module.workspace_bytes(a))
+        ws_bytes = cached[1]
         if not ws_bytes:
             return 0, 0
         key = stream.cuda_stream
@@ -249,7 +268,8 @@ class FusedOpBase:
         else:
             stream = default_stream
 
-        with torch.cuda.stream(stream):
+        # entering a stream context costs microseconds of host time per call: only when the op has a stream of its own
+        with (torch.cuda.stream(stream) if self.stream is not None else nullcontext()):
             device = args[-1].device
             visitor_args = self.allocate_outputs(device)
             for idx, input_name in enumerate(self.input_names):
@@ -527,7 +547,7 @@ class FusedRowOp(FusedOpBase):
     def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args) -> Tuple[jit.EvtArgs, list]:
         M, N, _, L = self.problem
         ops = [t.contiguous() for t in args[len(args) - self.num_anchor_inputs:]]
-        a = jit.EvtArgs()
+        a = self.argument_block()
         a.M, a.N, a.K, a.L = M, N, 1, L
         a.A, a.lda, a.batch_stride_A = ops[0].data_ptr(), N, M * N
         if len(ops) > 1:
