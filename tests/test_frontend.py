@@ -324,3 +324,16 @@ def test_row_anchor_limits():
     assert RowSpec.for_row_length("layernorm", 8192, "bf16") == RowSpec("layernorm", 16, 64, "bf16")
     with pytest.raises(NotImplementedError):
         RowSpec.for_row_length("softmax", 8200, "f16")
+
+
+def test_rows_too_long_for_the_row_kernel_stay_eager():
+    aten = torch.ops.aten
+
+    class WideSoftmax(torch.nn.Module):
+        def forward(self, x):
+            return aten.mul(aten._softmax(x, -1, False), 2.)
+
+    x = torch.empty(4, 16384, dtype=torch.float16, device="meta")
+    gm = W.fuse(WideSoftmax(), [x])
+    assert not fused_nodes(gm)
+    assert [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"] == ["_softmax", "mul"]

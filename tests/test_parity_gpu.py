@@ -478,3 +478,23 @@ def test_split_k(cfg, monkeypatch):
     assert tiles * 2 <= 256 and op.problem[2] >= 8 * tile.bk
     for o_auto, o_off in zip(results["auto"], results["1"]):
         assert evt_oracle.max_rel_err(o_auto, o_off.float()) <= 1e-2
+
+
+@pytest.mark.parametrize("name", ["softmax_aux_load", "layernorm1", "layernorm_backward_full"])
+def test_debug_mode_self_check_row_anchors(name):
+    """MODE=DEBUG on the row-wise anchors: the first call runs the anchor eagerly
+    (aten._softmax / native_layer_norm / native_layer_norm_backward), feeds its
+    result to the extracted epilogue module and compares with the kernel
+    (reference: FusedSoftmax.reference ... FusedLayerNormBackward.reference,
+    evt_fuser.py:748-753, 884-890, 952-958)."""
+    cls, _ = W.ROW_ANCHOR_PATTERNS[name]
+    inputs = [t.cuda() for t in W.pattern_inputs(name)]
+    gm = W.fuse(cls(), inputs)
+    (node,) = fused_nodes(gm)
+    op = node.target
+    op.mode = "DEBUG"
+    gm(*inputs)
+    assert op.launched
+    report = op.last_reference_report
+    assert len(report) == len(op.outputs)
+    assert all(r["match"] or r["atol_pass_rate"] > 0.999 or r["rtol_pass_rate"] > 0.98 for r in report), report
