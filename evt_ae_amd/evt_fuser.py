@@ -727,6 +727,12 @@ class EVTFuser:
             else:
                 output_node.replace_all_uses_with(view_node)
             graph_module.graph.inserting_after(view_node)
+        # The partition's own nodes are dead now.  Remove them here rather than leave it to dead-code elimination:
+        # fx keeps random ops (rand_like) alive as impure, and a stranded rand_like would keep its operand -- the
+        # whole unfused chain up to the GEMM -- running next to the fused kernel.
+        for node in reversed(partition):
+            if not node.users:
+                graph_module.graph.erase_node(node)
         self.fused_kernel = fused_kernel
         return fused_kernel
 

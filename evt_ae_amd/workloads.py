@@ -849,6 +849,50 @@ def row_edge_case(anchor: str, n: int, dtype, seed: int = 0):
     return _BareLayerNormBackward(n), [grad, x, mean, rstd]
 
 
+class DropoutBlock(torch.nn.Module):
+    """Feed-forward block with two dropouts and a post layer norm, in training
+    mode: `native_dropout` is decomposed to rand_like / ge / mul and the masks
+    are drawn inside the GEMM epilogues (reference: pass_decomposition.py:350-379,
+    unittest/evt_fuser/dropout.py)."""
+    P = 0.1
+
+    def __init__(self, d: int = 256, ffn: int = 512) -> None:
+        super().__init__()
+        self.l1 = torch.nn.Linear(d, ffn)
+        self.l2 = torch.nn.Linear(ffn, d)
+        self.ln = torch.nn.LayerNorm(d)
+
+    def forward(self, x, target):
+        F = torch.nn.functional
+        h = F.dropout(F.gelu(self.l1(x), approximate="tanh"), self.P, True)
+        y = self.ln(x + F.dropout(self.l2(h), self.P, True))
+        return ((y.float() - target) ** 2).sum()
+
+    def forward_with_masks(self, x, target, m1, m2):
+        """The same computation with the two keep masks given."""
+        F = torch.nn.functional
+        h = F.gelu(self.l1(x), approximate="tanh") * m1 / (1 - self.P)
+        y = self.ln(x + self.l2(h) * m2 / (1 - self.P))
+        return ((y.float() - target) ** 2).sum()
+
+
+def dropout_block(seed: int = 0, device: str = "cpu", dtype=torch.float16):
+    g = torch.Generator(device="cpu").manual_seed(0xD40 + seed)
+    model = DropoutBlock()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() == 2:
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+            elif name == "ln.weight":
+                p.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+            else:
+                p.copy_(0.02 * torch.randn(p.shape, generator=g))
+    model = model.to(dtype).to(device)
+    x = torch.randn(512, 256, generator=g).to(dtype).to(device)
+    target = torch.randn(512, 256, generator=g).to(device)
+    return model, (x, target)
+
+
 class EncoderLayer(torch.nn.Module):
     """fp16 post-LN transformer encoder layer with a squared-error loss: QKV
     projection, batched QK^T and PV products, softmax, output projection,

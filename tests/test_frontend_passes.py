@@ -252,3 +252,21 @@ def test_encoder_layer_joint_graph():
     assert not left & {"mm", "bmm", "addmm", "_softmax", "_softmax_backward_data", "native_layer_norm",
                        "native_layer_norm_backward", "gelu", "gelu_backward"}
     assert [n.name for n in box["fw"].graph.nodes if n.op == "placeholder"][-1].startswith("primals_")
+
+
+def test_dropout_in_a_training_step_is_fused_and_leaves_nothing_behind():
+    """native_dropout becomes rand_like / ge / mul inside the GEMM epilogues; the
+    masks are kernel outputs saved for backward.  fx keeps random ops alive as
+    impure, so the fuser removes a fused partition's nodes itself: no stray
+    rand_like (and with it no second, unfused copy of the GEMM chain) may remain."""
+    model, inputs = W.dropout_block(device="meta")
+    box = aot_capture(model, inputs)
+    fw, bw = box["fw"], box["bw"]
+    for gm in (fw, bw):
+        left = [str(n.target) for n in gm.graph.nodes if n.op == "call_function" and not n.meta.get("evt")]
+        assert not [t for t in left if "rand" in t or "aten.mm" in t or "gelu" in t or "dropout" in t], left
+    parts = [n.target.partition_names for n in fused_nodes(fw)]
+    assert sum("rand_like" in " ".join(p) for p in parts) == 2
+    saved_masks = [n for n in fw.graph.nodes if n.op == "output"][0].args[0]
+    bools = [a for a in saved_masks if hasattr(a, "meta") and getattr(a.meta.get("tensor_meta"), "dtype", None) == torch.bool]
+    assert len(bools) == 2

@@ -498,3 +498,34 @@ def test_debug_mode_self_check_row_anchors(name):
     report = op.last_reference_report
     assert len(report) == len(op.outputs)
     assert all(r["match"] or r["atol_pass_rate"] > 0.999 or r["rtol_pass_rate"] > 0.98 for r in report), report
+
+
+def test_aot_training_step_with_dropout():
+    """Dropout in training mode through the joint pipeline: the masks are drawn in
+    the GEMM epilogues (Philox, element-indexed) and saved for backward.  The
+    split forward / backward graphs are run by hand so the masks can be read
+    back; loss and gradients must equal the same block evaluated in fp32 with
+    those masks, and the keep rate must be 1 - p."""
+    import copy
+    from evt_ae_amd.aot_helper import aot_capture
+    model, (x, target) = W.dropout_block(device="cuda")
+    box = aot_capture(copy.deepcopy(model), (x, target))
+    fw, bw = box["fw"], box["bw"]
+    primals = [p.detach() for p in model.parameters()] + [x, target]
+    out = fw(*primals)
+    loss, saved = out[0], list(out[1:])
+    masks = [t for t in saved if t.dtype == torch.bool]
+    assert [tuple(m.shape) for m in masks] == [(512, 512), (512, 256)]
+    for m in masks:
+        assert abs(m.float().mean().item() - (1 - W.DropoutBlock.P)) < 5e-3
+    assert not torch.equal(masks[0][:, :256], masks[1])
+    grads = [g for g in bw(*saved, torch.ones_like(loss)) if g is not None]
+    torch.cuda.synchronize()
+    master = copy.deepcopy(model).float()
+    ref_loss = master.forward_with_masks(x.float(), target, masks[0].float(), masks[1].float())
+    ref_grads = torch.autograd.grad(ref_loss, list(master.parameters()))
+    assert abs(float(loss) - float(ref_loss)) <= 5e-3 * abs(float(ref_loss))
+    assert len(grads) == len(ref_grads)
+    for (name, _), g, r in zip(model.named_parameters(), grads, ref_grads):
+        err = float((g.float() - r).norm() / r.norm())
+        assert err <= 2e-2, f"{name}: norm-wise error {err:.3e}"
