@@ -27,7 +27,25 @@ def partition_func(joint_module: fx.GraphModule, joint_inputs, joint_compiler: C
     """Runs `joint_compiler` on the joint graph in place, then splits it where
     the original forward ended."""
     joint_compiler(joint_module)
-    return default_partition(joint_module, joint_inputs, **kwargs)
+    fw, bw = default_partition(joint_module, joint_inputs, **kwargs)
+    for gm in (fw, bw):
+        _drop_unused_random(gm)
+    return fw, bw
+
+
+def _drop_unused_random(gm: fx.GraphModule) -> None:
+    """torch.fx never removes random ops as dead code, so the split leaves a
+    copy of every `rand_like` the forward graph still runs eagerly in the
+    backward graph as well, its result unused (the backward reads the saved
+    mask).  An unused draw only costs time: remove it, and what it kept alive."""
+    changed = False
+    for node in reversed(list(gm.graph.nodes)):
+        if node.op == "call_function" and not node.users and "rand" in getattr(node.target, "__name__", str(node.target)):
+            gm.graph.erase_node(node)
+            changed = True
+    if changed:
+        gm.graph.eliminate_dead_code()
+        gm.recompile()
 
 
 def compiler_fn(fx_module: fx.GraphModule, _):

@@ -738,7 +738,7 @@ class RowCodegen(Codegen):
         # which spills the layer norm backward kernel)
         self.waves = 8 if ir.col_state else 4
         for n in ir.nodes.values():
-            if n.op == "colidx" or (n.op == "load" and ir.slots[n.slot].kind == "rand"):
+            if n.op == "colidx":
                 raise NotImplementedError(f"{n.op} behind a row-wise anchor")
         self.anchor_values = 1 + max([n.comp for n in ir.nodes.values() if n.op == "anchorval"], default=-1)
         # [N] vectors shared by every row (weight, bias, ...): read once per wave, not once per row
@@ -815,6 +815,10 @@ class RowCodegen(Codegen):
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = acc[c][j];")
             elif n.op == "anchorval":
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = av[{n.comp}][c][j];")
+            elif n.op == "load" and ir.slots[n.slot].kind == "rand":
+                k, r = n.slot, ir.rng_scalar
+                e(f"evt::rand8((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r}]) | ((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r + 1}]) << 32), "
+                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u, o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, {c});")
             elif n.op == "load" and name in self.hoisted:
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
             elif n.op == "load":
@@ -870,7 +874,7 @@ class RowCodegen(Codegen):
             "tensors": [{"name": s.name, "role": s.role, "dtype": s.dtype, "kind": s.kind,
                          "domain": s.domain} for s in self.ir.slots],
             "num_scalars": len(self.ir.scalars),
-            "rng_scalars": None,
+            "rng_scalars": self.ir.rng_scalar,
             # scalars[anchor_scalars] = eps of a layer norm anchor
             "anchor_scalars": self.ir.anchor_scalar,
             # layer norm backward: tensor slots of the forward pass's mean and rstd
@@ -938,7 +942,10 @@ class RowCodegen(Codegen):
         for k, s in enumerate(ir.slots):
             ct = DTYPE_CTYPES[s.dtype]
             e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
-            e("  if (!x.ptr || x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
+            if s.kind == "rand":   # generated values: no storage behind this slot
+                e("  if (x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
+            else:
+                e("  if (!x.ptr || x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
             e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
             e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div; "
               f"p.t{k}_lm = (int)x.l_mod;")

@@ -287,6 +287,24 @@ EVT_DEV void rand_row(uint64_t seed, uint32_t offset, uint32_t salt, int64_t e0,
   }
 }
 
+// 8 values of a row kernel's lane: elements e0, e0 + sn, ... (same stream as rand_row)
+EVT_DEV void rand8(uint64_t seed, uint32_t offset, uint32_t salt, int64_t e0, int64_t sn, float (&out)[8]) {
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  int64_t group = -1;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int64_t e = e0 + (int64_t)j * sn;
+    if (j == 0 || (e >> 2) != group) {
+      group = e >> 2;
+      w[0] = (uint32_t)group; w[1] = (uint32_t)((uint64_t)group >> 32); w[2] = offset; w[3] = salt;
+      philox4x32_10(w, (uint32_t)seed, (uint32_t)(seed >> 32));
+    }
+    const int sel = (int)(e & 3);
+    const uint32_t word = sel == 0 ? w[0] : sel == 1 ? w[1] : sel == 2 ? w[2] : w[3];
+    out[j] = (float)(word >> 8) * 5.9604644775390625e-08f;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // cross-lane exchange inside one 32-lane half of a wave (the 32 lanes that hold
 // the 32 columns of one accumulator row).  After the 5 steps every lane of the

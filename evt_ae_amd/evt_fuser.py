@@ -838,8 +838,8 @@ class EVTFuser:
         else:
             grad, xin, _, mean, rstd, gamma, _beta, mask = anchor.args[:8]
             mask = [bool(b) for b in mask]
-            if not mask[0]:
-                raise NotImplementedError(f"{anchor.name}: the input gradient is always computed")
+            # (with mask[0] unset -- the input needs no gradient -- the kernel still forms it in registers, the
+            # weight / bias sums share its row statistics; it is simply not stored)
             if (mask[1] or mask[2]) and L != 1:
                 # weight / bias gradients are sums over every row: one batch of rows
                 raise NotImplementedError(f"{anchor.name}: weight / bias gradients need the rows as one batch")

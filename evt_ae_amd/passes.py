@@ -321,6 +321,7 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                                      -> mul(mul(neg(one_hot(target)), tangent),
                                             unsqueeze(ne(target, ignore_index), 1)) [/ batch]   (:294-348;
                                         the reference compares with -1 instead of ignore_index)
+      masked_fill(x, mask, v)        -> where(mask, v, x)                        (scalar v; not in the reference)
       native_layer_norm(x, s, w, b, eps)
                                      -> add(mul(native_layer_norm(x, s, None, None, eps)[0], w), b)   (:504-544)
     and permute(permute(x)) folded into one permute or none.  The reference's
@@ -364,6 +365,10 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
             elif name == "threshold_backward":
                 g, y, t = node.args
                 new = mk(aten.mul, (g, mk(aten.gt, (y, t))))
+            elif name == "masked_fill" and len(node.args) == 3 and isinstance(node.args[2], (int, float)):
+                # a fill value under a mask is a select: where(mask, value, x) is in the epilogue vocabulary
+                x, mask, value = node.args
+                new = mk(aten.where, (mask, float(value), x))
             elif name == "_log_softmax" and len(node.args) == 3:
                 x, dim, half_to_float = node.args
                 new = mk(aten.log, (mk(aten._softmax, (x, dim, half_to_float)),))

@@ -70,6 +70,8 @@ def register_all() -> List[jit.LazyModule]:
     aot_capture(*W.mlp_classifier())
     aot_capture(*W.encoder_layer(device="meta"))
     aot_capture(*W.dropout_block(device="meta"))
+    aot_capture(*W.decoder_block(device="meta"))
+    aot_capture(*W.decoder_block(device="meta", dtype=torch.bfloat16))
     aot_capture(*W.encoder_layer(device="meta", **W.ENCODER_BENCH))      # bench.py's training-step leg
     # the same step through torch.compile: Dynamo's graph differs slightly, so
     # its kernels are registered as well (tracing stops at the first launch

@@ -14,6 +14,8 @@ import operator
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Sequence, Tuple
 
+import math
+
 import torch
 from torch.fx import GraphModule, symbolic_trace
 from torch.fx.passes.shape_prop import ShapeProp
@@ -472,8 +474,27 @@ class Dropout1Undecomposed(torch.nn.Module):
         return add_4, getitem_3
 
 
+class SoftmaxDropout(torch.nn.Module):
+    """Attention-probability dropout: softmax over masked scores, then the
+    decomposed native_dropout (pass_decomposition.py:359-369) on the
+    probabilities; both the mask and the dropped probabilities leave the kernel."""
+    P = 0.1
+
+    def forward(self, scores, causal):
+        masked = aten.where(causal, -65504.0, scores)
+        probs = aten._softmax(masked, -1, False)
+        mask = aten.ge(torch.rand_like(probs), self.P)
+        out = aten.mul(aten.mul(probs, mask), 1. / (1 - self.P))
+        return out, mask, probs
+
+
+def _causal(s):
+    return torch.ones(s, s, dtype=torch.bool).triu(1)
+
+
 # patterns that draw random numbers in the epilogue: checked with the generator's stream replayed on the CPU
 RANDOM_PATTERNS = {
+    "softmax_dropout": (SoftmaxDropout, lambda g: [_h(g, (3, 4, 136, 136)), _causal(136)]),
     "mm12": (MMPartition12, lambda g: [_h(g, (512, 24576), 0.01), _h(g, (1024, 24576)), _h(g, (512,))]),
     "dropout1": (Dropout1, lambda g: [_h(g, (1024, 1024)), _h(g, (1024, 1024), 0.03), _h(g, (1024,)),
                                       _h(g, (512, 2, 1024))]),
@@ -890,6 +911,62 @@ def dropout_block(seed: int = 0, device: str = "cpu", dtype=torch.float16):
     model = model.to(dtype).to(device)
     x = torch.randn(512, 256, generator=g).to(dtype).to(device)
     target = torch.randn(512, 256, generator=g).to(device)
+    return model, (x, target)
+
+
+class DecoderBlock(torch.nn.Module):
+    """Pre-layer-norm decoder block in training mode: causal `masked_fill` on the
+    scores (decomposed to `where`, fused behind the Q K^T BMM), softmax with the
+    attention-probability dropout drawn behind it in the same row kernel, GELU
+    feed-forward, residuals.  Not one of the reference's models: it exercises
+    rand_like behind a row-wise anchor and a layer norm backward whose input
+    gradient is the only one some consumers need."""
+    P = 0.1
+
+    def __init__(self, d: int = 256, heads: int = 4) -> None:
+        super().__init__()
+        self.h = heads
+        self.ln1 = torch.nn.LayerNorm(d)
+        self.ln2 = torch.nn.LayerNorm(d)
+        self.qkv = torch.nn.Linear(d, 3 * d)
+        self.o = torch.nn.Linear(d, d)
+        self.f1 = torch.nn.Linear(d, 4 * d)
+        self.f2 = torch.nn.Linear(4 * d, d)
+
+    def _block(self, x, target, drop):
+        F = torch.nn.functional
+        B, S, D = x.shape
+        H, dh = self.h, D // self.h
+        q, k, v = self.qkv(self.ln1(x)).view(B, S, 3, H, dh).permute(2, 0, 3, 1, 4)
+        att = (q @ k.transpose(-1, -2)) / math.sqrt(dh)
+        keep = torch.ones(S, S, dtype=torch.bool, device=x.device).tril()
+        att = drop(torch.softmax(att.masked_fill(~keep, float("-inf")), -1))
+        x = x + self.o((att @ v).permute(0, 2, 1, 3).reshape(B, S, D))
+        x = x + self.f2(F.gelu(self.f1(self.ln2(x)), approximate="tanh"))
+        return ((x.float() - target) ** 2).sum()
+
+    def forward(self, x, target):
+        return self._block(x, target, lambda p: torch.nn.functional.dropout(p, self.P, True))
+
+    def forward_with_masks(self, x, target, m):
+        """The same computation with the attention keep mask given."""
+        return self._block(x, target, lambda p: p * m / (1 - self.P))
+
+
+def decoder_block(seed: int = 0, device: str = "cpu", dtype=torch.float16, batch: int = 4, seq: int = 128):
+    g = torch.Generator(device="cpu").manual_seed(0xDEC + seed)
+    model = DecoderBlock()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() == 2:
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+            elif name.endswith("ln1.weight") or name.endswith("ln2.weight"):
+                p.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+            else:
+                p.copy_(0.02 * torch.randn(p.shape, generator=g))
+    model = model.to(dtype).to(device)
+    x = torch.randn(batch, seq, 256, generator=g).to(dtype).to(device)
+    target = torch.randn(batch, seq, 256, generator=g).to(device)
     return model, (x, target)
 
 

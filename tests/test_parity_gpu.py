@@ -157,10 +157,11 @@ def test_reference_dropout_test_verbatim():
     assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
 
 
-@pytest.mark.parametrize("name", ["mm12", "dropout1"])
+@pytest.mark.parametrize("name", ["mm12", "dropout1", "softmax_dropout"])
 def test_random_fuser_patterns(name):
     """rand_like fused into the epilogue (unittest/evt_fuser/mm.py:216-236,
-    dropout.py:33-75).  The reference can only check the keep rate; here the
+    dropout.py:33-75; softmax_dropout: the same decomposed dropout behind a
+    softmax anchor, 4-D probabilities, rows of 136).  The reference can only check the keep rate; here the
     generator's stream is replayed on the CPU (oracle/philox.py), so the masks
     must match bit for bit and the values to the fp16 tolerance, and two
     launches must draw different numbers."""
@@ -186,8 +187,9 @@ def test_random_fuser_patterns(name):
             else:
                 assert evt_oracle.max_rel_err(o, r) <= FP16_TOL
         masks.append(outs[1].cpu())
-    if name == "dropout1":
+    if name != "mm12":
         assert not torch.equal(masks[0], masks[1])
+    if name == "dropout1":
         keep = masks[0].float().mean().item()          # the reference's criterion (dropout.py:73-75)
         assert 0.3 - 1e-3 < keep < 0.3 + 1e-3
 
@@ -529,3 +531,40 @@ def test_aot_training_step_with_dropout():
     for (name, _), g, r in zip(model.named_parameters(), grads, ref_grads):
         err = float((g.float() - r).norm() / r.norm())
         assert err <= 2e-2, f"{name}: norm-wise error {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_aot_decoder_block_with_attention_dropout(dtype):
+    """A pre-layer-norm decoder block in training mode: the causal masked_fill
+    runs as a `where` behind the Q K^T BMM, the attention-probability dropout is
+    drawn behind the softmax anchor in the row kernel (same element-indexed
+    Philox stream as the GEMM epilogues), and both layer norm backward ops are
+    fused, the first layer's without an input gradient (x needs none).  Loss and gradients must equal the block evaluated in fp32 with the
+    saved mask."""
+    import copy
+    from evt_ae_amd.aot_helper import aot_capture
+    model, (x, target) = W.decoder_block(device="cuda", dtype=dtype)
+    box = aot_capture(copy.deepcopy(model), (x, target))
+    fw, bw = box["fw"], box["bw"]
+    kinds = [type(n.target).__name__ for g in (fw, bw) for n in fused_nodes(g)]
+    assert kinds.count("FusedSoftmax") == 1 and kinds.count("FusedSoftmaxBackward") == 1
+    assert kinds.count("FusedLayerNorm") == 2 and kinds.count("FusedLayerNormBackward") == 2
+    left = {str(n.target) for g in (fw, bw) for n in g.graph.nodes if n.op == "call_function"}
+    assert not [t for t in left if "rand" in t or "masked_fill" in t or "dropout" in t or "aten.bmm" in t], left
+    primals = [p.detach() for p in model.parameters()] + [x, target]
+    out = fw(*primals)
+    loss, saved = out[0], list(out[1:])
+    (mask,) = [t for t in saved if t.dtype == torch.bool and t.dim() == 4]
+    assert tuple(mask.shape) == (4, 4, 128, 128)
+    assert abs(mask.float().mean().item() - (1 - W.DecoderBlock.P)) < 5e-3
+    grads = [g for g in bw(*saved, torch.ones_like(loss)) if g is not None]
+    torch.cuda.synchronize()
+    master = copy.deepcopy(model).float()
+    ref_loss = master.forward_with_masks(x.float(), target, mask.float())
+    ref_grads = torch.autograd.grad(ref_loss, list(master.parameters()))
+    tol = 2e-2 if dtype == torch.float16 else 6e-2      # bf16 carries 8 mantissa bits through every saved activation
+    assert abs(float(loss) - float(ref_loss)) <= (5e-3 if dtype == torch.float16 else 2e-2) * abs(float(ref_loss))
+    assert len(grads) == len(ref_grads)
+    for (name, _), g, r in zip(model.named_parameters(), grads, ref_grads):
+        err = float((g.float() - r).norm() / r.norm())
+        assert err <= tol, f"{name}: norm-wise error {err:.3e}"
