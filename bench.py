@@ -65,7 +65,7 @@ class Case:
             dev_in = [t.cuda() for t in self.cpu_inputs]
             args = [dev_in[i] for i in self.arg_index]
             outs = self.op.allocate_outputs("cuda")
-            a, keep = self.op.build_arguments(outs, *args)
+            a, keep = self.op.build_arguments(outs, *args, block=self.op.new_argument_block())
             ws_ptr, ws_bytes = self.op.workspace_for(a, stream, "cuda")
             self.sets.append((a, keep, outs, dev_in, ws_ptr, ws_bytes))
         self.unfused = W.unfused_eager(cfg)

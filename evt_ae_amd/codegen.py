@@ -689,31 +689,48 @@ class RowSpec:
     The analogue of the reference's (rows_per_cta, warp_count, cache_input)
     tuple (python/gtl/compiler/autotuner/softmax_tuner.py)."""
     op: str             # "softmax" | "softmax_backward" | "layernorm" | "layernorm_backward"
-    ch: int             # chunks of lpr * 8 columns cached per lane
-    lpr: int            # lanes per row (power of two, <= 64)
+    ch: int             # chunks of lpr * wpr * 8 columns cached per lane
+    lpr: int            # lanes per row inside a wave (power of two, <= 64)
     elt: str            # "f16" | "bf16" | "f32"
+    wpr: int = 1        # waves per row (power of two, <= 16; above 1 a workgroup holds one row)
 
     OPS = ("softmax", "softmax_backward", "layernorm", "layernorm_backward")
 
     def tag(self) -> str:
-        return f"{self.op}_{self.elt}_ch{self.ch}_lpr{self.lpr}"
+        return f"{self.op}_{self.elt}_ch{self.ch}_lpr{self.lpr}" + (f"_w{self.wpr}" if self.wpr > 1 else "")
 
     @property
     def max_n(self) -> int:
-        return self.ch * self.lpr * 8
+        return self.ch * self.lpr * self.wpr * 8
+
+    @staticmethod
+    def registers(op: str, elt: str, ch: int, lookahead: bool) -> float:
+        """Registers per lane that hold row data: the fp32 working copies (two
+        for the backward anchors), the operands as loaded, twice when the next
+        row is fetched ahead, and layer norm backward's weight."""
+        two = 2 if op in ("softmax_backward", "layernorm_backward") else 1
+        weight = ch * 8 if op == "layernorm_backward" else 0      # this lane's columns of the weight, kept across rows
+        return ch * 8 * two * (1 + (1.0 if elt == "f32" else 0.5) * (2 if lookahead else 1)) + weight
 
     @staticmethod
     def for_row_length(op: str, n: int, elt: str) -> "RowSpec":
         """Smallest lane group that holds the row in at most 16 chunks, widened
         to a full wave once a row needs 4 or more chunks per lane (one row per
-        wave keeps every 16-byte access of a wave inside one row)."""
+        wave keeps every 16-byte access of a wave inside one row).  Rows longer
+        than 8192 go over 2 .. 16 waves, as few as keep the row data within
+        three quarters of the registers a lane can have at that workgroup size
+        (16 waves: 128 registers and no fetch ahead)."""
         lpr = 8
         while lpr < 64 and (n + lpr * 8 - 1) // (lpr * 8) > 2:
             lpr *= 2
         ch = (n + lpr * 8 - 1) // (lpr * 8)
-        if ch > 16:
-            raise NotImplementedError(f"rows of {n} elements do not fit the register-cached row kernel (max 8192)")
-        return RowSpec(op, ch, lpr, elt)
+        if ch <= 16:
+            return RowSpec(op, ch, lpr, elt)
+        for wpr, budget in ((2, 192), (4, 192), (8, 192), (16, 96)):
+            ch = (n + wpr * 512 - 1) // (wpr * 512)
+            if ch <= 16 and RowSpec.registers(op, elt, ch, wpr < 16) <= budget:
+                return RowSpec(op, ch, 64, elt, wpr)
+        raise NotImplementedError(f"rows of {n} {elt} elements do not fit the register-cached {op} kernel")
 
 
 class RowCodegen(Codegen):
@@ -730,13 +747,13 @@ class RowCodegen(Codegen):
             # the row would be a second pass over the anchor's own axis
             if r.axis != "col" or r.kind not in ("sum", "max"):
                 raise NotImplementedError(f"per-row reduction {r.name} behind a row-wise anchor")
-        if ir.col_state and (ir.L != 1 or ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536):
+        if ir.col_state and (spec.wpr > 1 or ir.L != 1 or ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536):
             raise NotImplementedError("per-column reduction behind a row-wise anchor: one batch and rows of at most "
                                       f"{65536 // (4 * max(ir.col_state, 1))} elements")
         # a kernel that reduces over the rows runs 8 waves per workgroup: as many rows in flight per CU from half
         # the workgroups, so half the partials for the second phase (16 waves would cap a wave at 128 registers,
         # which spills the layer norm backward kernel)
-        self.waves = 8 if ir.col_state else 4
+        self.waves = spec.wpr if spec.wpr > 1 else (8 if ir.col_state else 4)
         for n in ir.nodes.values():
             if n.op == "colidx":
                 raise NotImplementedError(f"{n.op} behind a row-wise anchor")
@@ -866,7 +883,7 @@ class RowCodegen(Codegen):
             "abi": 2,
             "name": self.name,
             "anchor": sp.op,
-            "row": {"chunks": sp.ch, "lanes_per_row": sp.lpr, "max_n": sp.max_n},
+            "row": {"chunks": sp.ch, "lanes_per_row": sp.lpr * sp.wpr, "waves_per_row": sp.wpr, "max_n": sp.max_n},
             "element": sp.elt,
             "batched": self.ir.batched,
             "row_state": 0,
@@ -905,7 +922,7 @@ class RowCodegen(Codegen):
         self.emit_row(e)
         e.dedent()
         e("};")
-        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}, {self.anchor_values}, {self.waves}>;")
+        e(f"using Cfg = evt::RowCfg<{op_id}, {sp.ch}, {sp.lpr}, {elt_id}, {self.anchor_values}, {self.waves}, {sp.wpr}>;")
         e(f"constexpr int kNumTensors = {len(ir.slots)};")
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
         e(f"constexpr int kEltBytes = {4 if sp.elt == 'f32' else 2};")
@@ -922,8 +939,9 @@ class RowCodegen(Codegen):
         e("g.A = (const char*)a->A; g.lda = a->lda; g.bsA = a->batch_stride_A;")
         e("g.B = (const char*)a->B; g.ldb = a->ldb; g.bsB = a->batch_stride_B;")
         e("if (a->lda < a->N) return EVT_ERR_BAD_ARGS;")
-        e("g.vecA = (((uintptr_t)a->A | (uintptr_t)(a->lda * kEltBytes) | (uintptr_t)(a->batch_stride_A * kEltBytes)) & 15) == 0;")
-        e("g.vecB = (((uintptr_t)a->B | (uintptr_t)(a->ldb * kEltBytes) | (uintptr_t)(a->batch_stride_B * kEltBytes)) & 15) == 0;")
+        e("// 16-byte accesses need dword alignment only")
+        e("g.vecA = (((uintptr_t)a->A | (uintptr_t)(a->lda * kEltBytes) | (uintptr_t)(a->batch_stride_A * kEltBytes)) & 3) == 0;")
+        e("g.vecB = (((uintptr_t)a->B | (uintptr_t)(a->ldb * kEltBytes) | (uintptr_t)(a->batch_stride_B * kEltBytes)) & 3) == 0;")
         e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0; g.colws = nullptr;")
         if ir.col_state:
             e("if (a->L != 1) return EVT_ERR_BAD_ARGS;      // the per-column reductions run over every row")
@@ -938,7 +956,7 @@ class RowCodegen(Codegen):
             if len(ir.anchor_slots) > 2:     # the weight, applied to the incoming gradient
                 kg = ir.anchor_slots[2]
                 e(f"if (!a->tensors[{kg}].ptr || a->tensors[{kg}].stride_n != 1) return EVT_ERR_BAD_ARGS;")
-                e(f"g.gamma = (const char*)a->tensors[{kg}].ptr; g.vecG = ((uintptr_t)g.gamma & 15) == 0;")
+                e(f"g.gamma = (const char*)a->tensors[{kg}].ptr; g.vecG = ((uintptr_t)g.gamma & 3) == 0;")
         for k, s in enumerate(ir.slots):
             ct = DTYPE_CTYPES[s.dtype]
             e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
@@ -950,7 +968,7 @@ class RowCodegen(Codegen):
             e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div; "
               f"p.t{k}_lm = (int)x.l_mod;")
             e(f"  p.t{k}_vec = (x.stride_n == 1 && (((uintptr_t)x.ptr | (uintptr_t)(x.stride_m * (int64_t)sizeof({ct})) | "
-              f"(uintptr_t)(x.stride_l * (int64_t)sizeof({ct}))) & 15) == 0) ? 1 : 0; }}")
+              f"(uintptr_t)(x.stride_l * (int64_t)sizeof({ct}))) & 3) == 0) ? 1 : 0; }}")
         for name in self.hoisted:
             k = ir.nodes[name].slot
             e(f"if (a->tensors[{k}].stride_l != 0 || a->tensors[{k}].stride_m != 0) return EVT_ERR_BAD_ARGS;   // read once per wave")
@@ -959,7 +977,7 @@ class RowCodegen(Codegen):
         vec_slots = [k for k, sl in enumerate(ir.slots) if k not in ir.anchor_slots and
                      ((sl.role == "load" and sl.kind in ("aux", "row")) or (sl.role == "store" and sl.domain == "tile"))]
         cond = " && ".join(f"p.t{k}_vec" for k in vec_slots) or "1"
-        e(f"p.fast = (g.fast && {cond}) ? 1 : 0;   // every per-element tensor of the epilogue is unit-stride and 16-byte aligned too")
+        e(f"p.fast = (g.fast && {cond}) ? 1 : 0;   // every per-element tensor of the epilogue is unit-stride and dword aligned too")
         e("return EVT_OK;")
         e.dedent()
         e("}")

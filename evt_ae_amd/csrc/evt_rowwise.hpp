@@ -16,7 +16,10 @@
 // through LDS and no workgroup barrier is needed, so a workgroup is just 4
 // independent waves.  The normalised
 // values stay in registers and are handed to the generated epilogue as the
-// "accumulator".
+// "accumulator".  Rows longer than 8192 elements (vocabulary-sized softmax)
+// are spread over the WPR = 2 .. 16 waves of one workgroup, still register
+// cached and read once; the only addition is that each row reduction ends
+// with an exchange of one value per wave through LDS and a barrier.
 #pragma once
 
 #include "evt_epilogue.hpp"
@@ -38,21 +41,28 @@ struct RowArgs {
   float eps;                 // layer norm
   int vecA, vecB;            // rows of A / B may be read with 16-byte loads
   float* colws;              // per-column reductions of the epilogue: [workgroups][COL_STATE][N] partials
-  int fast;                  // N % 8 == 0 and every anchor operand is 16-byte aligned: whole 8-column groups only
+  int fast;                  // N % 8 == 0 and every anchor operand is dword aligned: whole 8-column groups only
 };
 
 // ELT: 0 = f16, 1 = bf16, 2 = f32 element type of the anchor operands
 // AV: per-element values besides the result that the anchor hands to the epilogue (layer norm backward with
 // weight / bias gradients: the incoming gradient and the normalised input)
-template <int OP_, int CH_, int LPR_, int ELT_, int AV_ = 0, int WAVES_ = 4>
+// WPR: waves per row; above 1 the whole workgroup (WAVES == WPR full waves) holds one row
+template <int OP_, int CH_, int LPR_, int ELT_, int AV_ = 0, int WAVES_ = 4, int WPR_ = 1>
 struct RowCfg {
-  static constexpr int OP = OP_, CH = CH_, LPR = LPR_, ELT = ELT_, AV = AV_, WAVES = WAVES_;
+  static constexpr int OP = OP_, CH = CH_, LPR = LPR_, ELT = ELT_, AV = AV_, WAVES = WAVES_, WPR = WPR_;
   static constexpr int THREADS = WAVES * 64;
-  static constexpr int RPW = 64 / LPR;        // rows per wave
-  static constexpr int ROWS = WAVES * RPW;    // rows per workgroup
-  static constexpr int SPAN = LPR * 8;        // columns per chunk
+  static constexpr int RPW = 64 / LPR;              // rows per wave
+  static constexpr int ROWS = WAVES * RPW / WPR;    // rows per workgroup
+  static constexpr int GROUP = LPR * WPR;           // lanes per row
+  static constexpr int SPAN = GROUP * 8;            // columns per chunk
+  // a wave fetches its next row before it reduces the present one; 16 waves leave 128 registers per lane, not
+  // enough for two rows' worth
+  static constexpr bool LOOKAHEAD = WPR < 16;
   static_assert(LPR >= 1 && LPR <= 64 && (LPR & (LPR - 1)) == 0, "lanes per row: a power of two up to 64");
   static_assert(CH >= 1 && CH <= 16, "a row is cached in at most 128 registers per lane");
+  static_assert(WPR == 1 || (LPR == 64 && WAVES == WPR && WPR <= 16 && (WPR & (WPR - 1)) == 0),
+                "a row over several waves takes whole waves and the whole workgroup");
 };
 
 template <int ELT> struct RowElt;
@@ -106,24 +116,52 @@ EVT_DEV float group_reduce(float x) {
   }
   return x;
 }
-template <int LPR>
-EVT_DEV float group_sum(float x) { return group_reduce<LPR, OpSum>(x); }
-template <int LPR>
-EVT_DEV float group_max(float x) { return group_reduce<LPR, OpMax>(x); }
+// All-reduce over a row: the lane group of a wave, then (rows spread over several waves) one value per wave
+// through LDS.  Successive reductions alternate between two sets of slots, so one barrier each is enough: a wave
+// can only overwrite a set after the barrier of the reduction in between, which every wave reaches after it
+// has read that set.  Every wave of the workgroup must take part in every reduction.
+template <class Cfg>
+struct RowReduce {
+  float* slots;      // [2][16] floats of LDS (unused when a row lives in one wave)
+  int phase;
+  template <class Op>
+  EVT_DEV float all(float x) {
+    x = group_reduce<Cfg::LPR, Op>(x);
+    if constexpr (Cfg::WPR > 1) {
+      float* s = slots + phase * 16;
+      if ((threadIdx.x & 63) == 0) s[threadIdx.x >> 6] = x;
+      __syncthreads();
+      float y = s[0];
+#pragma unroll
+      for (int w = 1; w < Cfg::WPR; ++w) y = Op::f(y, s[w]);
+      x = y;
+      phase ^= 1;
+    }
+    return x;
+  }
+  EVT_DEV float sum(float x) { return all<OpSum>(x); }
+  EVT_DEV float max(float x) { return all<OpMax>(x); }
+};
+
+// 16 / 8 bytes moved by one instruction.  Multi-dword global accesses need dword alignment only, so the types
+// promise no more than that: rows whose length is no multiple of 8 elements (a 30522-entry vocabulary) still
+// move 16 bytes per lane wherever 8 whole columns are left.
+typedef uint32_t q16 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t q8 __attribute__((ext_vector_type(2), aligned(4)));
 
 // 8 consecutive elements starting at p[0] (unit stride), `valid` of them inside the row
 template <class T>
 EVT_DEV void load8(const T* p, bool vec, int valid, float fill, float (&out)[8]) {
   if (vec && valid == 8) {
     if constexpr (sizeof(T) == 2) {
-      union { uint4 q; T e[8]; } u;
-      u.q = *reinterpret_cast<const uint4*>(p);
+      union { q16 q; T e[8]; } u;
+      u.q = *reinterpret_cast<const q16*>(p);
 #pragma unroll
       for (int j = 0; j < 8; ++j) out[j] = (float)u.e[j];
     } else if constexpr (sizeof(T) == 4 && !std::is_same<T, bool>::value) {
-      union { uint4 q[2]; T e[8]; } u;
-      u.q[0] = reinterpret_cast<const uint4*>(p)[0];
-      u.q[1] = reinterpret_cast<const uint4*>(p)[1];
+      union { q16 q[2]; T e[8]; } u;
+      u.q[0] = reinterpret_cast<const q16*>(p)[0];
+      u.q[1] = reinterpret_cast<const q16*>(p)[1];
 #pragma unroll
       for (int j = 0; j < 8; ++j) out[j] = (float)u.e[j];
     } else {
@@ -151,17 +189,17 @@ template <class T>
 EVT_DEV void store8s(T* p, int64_t sn, bool vec, int valid, const float (&val)[8]) {
   if (sn == 1 && vec && valid == 8) {
     if constexpr (sizeof(T) == 2) {
-      union { uint4 q; T e[8]; } u;
+      union { q16 q; T e[8]; } u;
 #pragma unroll
       for (int j = 0; j < 8; ++j) u.e[j] = (T)val[j];
-      *reinterpret_cast<uint4*>(p) = u.q;
+      *reinterpret_cast<q16*>(p) = u.q;
       return;
     } else if constexpr (sizeof(T) == 4 && !std::is_same<T, bool>::value) {
-      union { uint4 q[2]; T e[8]; } u;
+      union { q16 q[2]; T e[8]; } u;
 #pragma unroll
       for (int j = 0; j < 8; ++j) u.e[j] = (T)val[j];
-      reinterpret_cast<uint4*>(p)[0] = u.q[0];
-      reinterpret_cast<uint4*>(p)[1] = u.q[1];
+      reinterpret_cast<q16*>(p)[0] = u.q[0];
+      reinterpret_cast<q16*>(p)[1] = u.q[1];
       return;
     }
   }
@@ -174,12 +212,12 @@ EVT_DEV void store8s(T* p, int64_t sn, bool vec, int valid, const float (&val)[8
 template <class T>
 EVT_DEV void load8v(const T* p, float (&out)[8]) {
   constexpr int Q = (sizeof(T) * 8 + 15) / 16;
-  union { uint4 q[Q]; T e[8]; } u;
+  union { q16 q[Q]; T e[8]; } u;
   if constexpr (sizeof(T) * 8 >= 16) {
 #pragma unroll
-    for (int i = 0; i < Q; ++i) u.q[i] = reinterpret_cast<const uint4*>(p)[i];
+    for (int i = 0; i < Q; ++i) u.q[i] = reinterpret_cast<const q16*>(p)[i];
   } else {   // 1-byte elements: one 8-byte load
-    *reinterpret_cast<uint2*>(&u) = *reinterpret_cast<const uint2*>(p);
+    *reinterpret_cast<q8*>(&u) = *reinterpret_cast<const q8*>(p);
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -190,7 +228,7 @@ EVT_DEV void load8v(const T* p, float (&out)[8]) {
 template <class T>
 EVT_DEV void store8v(T* p, const float (&val)[8]) {
   constexpr int Q = (sizeof(T) * 8 + 15) / 16;
-  union { uint4 q[Q]; T e[8]; } u;
+  union { q16 q[Q]; T e[8]; } u;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     if constexpr (std::is_same<T, bool>::value) u.e[j] = val[j] != 0.f;
@@ -198,9 +236,9 @@ EVT_DEV void store8v(T* p, const float (&val)[8]) {
   }
   if constexpr (sizeof(T) * 8 >= 16) {
 #pragma unroll
-    for (int i = 0; i < Q; ++i) reinterpret_cast<uint4*>(p)[i] = u.q[i];
+    for (int i = 0; i < Q; ++i) reinterpret_cast<q16*>(p)[i] = u.q[i];
   } else {
-    *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(&u);
+    *reinterpret_cast<q8*>(p) = *reinterpret_cast<const q8*>(&u);
   }
 }
 
@@ -223,9 +261,9 @@ template <class T>
 EVT_DEV void load8_raw(const T* p, bool vec, int valid, T fill, T (&out)[8]) {
   if (vec && valid == 8) {
     constexpr int Q = sizeof(T) * 8 / 16;
-    union { uint4 q[Q]; T e[8]; } u;
+    union { q16 q[Q]; T e[8]; } u;
 #pragma unroll
-    for (int i = 0; i < Q; ++i) u.q[i] = reinterpret_cast<const uint4*>(p)[i];
+    for (int i = 0; i < Q; ++i) u.q[i] = reinterpret_cast<const q16*>(p)[i];
 #pragma unroll
     for (int j = 0; j < 8; ++j) out[j] = u.e[j];
   } else {
@@ -246,8 +284,8 @@ EVT_DEV void row_fetch_one(const char* base, int64_t ld, int64_t bs, int vec, co
 #pragma unroll
     for (int c = 0; c < Cfg::CH; ++c) {
       const bool in = t.col0(c) < t.N;
-      union { uint4 q[Q]; T e[8]; } u;
-      const uint4* src = reinterpret_cast<const uint4*>(row + (in ? t.col0(c) : 0));
+      union { q16 q[Q]; T e[8]; } u;
+      const q16* src = reinterpret_cast<const q16*>(row + (in ? t.col0(c) : 0));
 #pragma unroll
       for (int i = 0; i < Q; ++i) u.q[i] = src[i];
 #pragma unroll
@@ -284,8 +322,9 @@ EVT_DEV void row_widen(const typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8], f
 
 template <class Cfg>
 EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>& raw, const float (&gz)[Cfg::CH][8],
-                      float (&acc)[Cfg::CH][8], float (&rv)[2], float (&av)[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8]) {
-  constexpr int CH = Cfg::CH, LPR = Cfg::LPR;
+                      float (&acc)[Cfg::CH][8], float (&rv)[2], float (&av)[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8],
+                      RowReduce<Cfg>& red) {
+  constexpr int CH = Cfg::CH;
   const float rn = 1.f / (float)g.N;
   if constexpr (Cfg::OP == ROW_SOFTMAX) {
     // aten._softmax over the last axis: exp(x - max) / sum, all in fp32
@@ -295,7 +334,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
     for (int c = 0; c < CH; ++c)
 #pragma unroll
       for (int j = 0; j < 8; ++j) mx = fmaxf(mx, acc[c][j]);
-    mx = group_max<LPR>(mx);
+    mx = red.max(mx);
     const float off = (mx == -INFINITY) ? 0.f : mx * kLog2e;    // a row of -inf gives NaN below, as torch does
     float s = 0.f;
 #pragma unroll
@@ -305,7 +344,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
         acc[c][j] = __builtin_amdgcn_exp2f(acc[c][j] * kLog2e - off);
         s += acc[c][j];
       }
-    s = group_sum<LPR>(s);
+    s = red.sum(s);
     const float inv = 1.f / s;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -322,7 +361,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
     for (int c = 0; c < CH; ++c)
 #pragma unroll
       for (int j = 0; j < 8; ++j) s += acc[c][j] * y[c][j];
-    s = group_sum<LPR>(s);
+    s = red.sum(s);
 #pragma unroll
     for (int c = 0; c < CH; ++c)
 #pragma unroll
@@ -337,7 +376,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
     for (int c = 0; c < CH; ++c)
 #pragma unroll
       for (int j = 0; j < 8; ++j) s += acc[c][j];
-    const float mean = group_sum<LPR>(s) * rn;
+    const float mean = red.sum(s) * rn;
     float q = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -349,7 +388,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
         q += j < v ? d * d : 0.f;
       }
     }
-    const float rstd = rsqrtf(group_sum<LPR>(q) * rn + g.eps);
+    const float rstd = rsqrtf(red.sum(q) * rn + g.eps);
 #pragma unroll
     for (int c = 0; c < CH; ++c)
 #pragma unroll
@@ -386,8 +425,8 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
         s2 += acc[c][j] * xh[c][j];
       }
     }
-    s1 = group_sum<LPR>(s1) * rn;
-    s2 = group_sum<LPR>(s2) * rn;
+    s1 = red.sum(s1) * rn;
+    s2 = red.sum(s2) * rn;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
 #pragma unroll
@@ -416,9 +455,12 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
   const int64_t stride = (int64_t)gridDim.x * Cfg::ROWS;
   RowCtx<Cfg> t;
   t.M = g.M; t.N = g.N; t.L = g.L;
-  t.sub = lane % Cfg::LPR;
+  t.sub = Cfg::WPR > 1 ? (int)threadIdx.x : lane % Cfg::LPR;
+  __shared__ float xch[2 * 16];
+  RowReduce<Cfg> red{xch, 0};
+  static_assert(CS == 0 || Cfg::WPR == 1, "per-column reductions need a row per wave");
   auto locate = [&](int64_t base) {
-    const int64_t r = base + lane / Cfg::LPR;
+    const int64_t r = base + (Cfg::WPR > 1 ? 0 : lane / Cfg::LPR);
     t.ok = r < rows;
     t.r = t.ok ? r : rows - 1;      // lanes past the end recompute the last row and store nothing
     t.l = (int)(t.r / g.M);
@@ -437,7 +479,9 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
         for (int k = 0; k < CS; ++k) cst[k][c][j] = id[k];
       }
   }
-  int64_t base = ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW;    // wave-uniform
+  // wave-uniform; the same for every wave of the workgroup when they share a row (so all of them reach the barriers
+  // of the reductions the same number of times)
+  int64_t base = Cfg::WPR > 1 ? (int64_t)blockIdx.x : ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW;
   if (base < rows) {
     RowRaw<Cfg> cur;
     locate(base);
@@ -465,17 +509,24 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
       const int64_t next = base + stride;
       const bool more = next < rows;                                         // wave-uniform
       RowRaw<Cfg> ahead;
-      if (more) {
-        locate(next);
-        row_fetch<Cfg, FAST>(g, t, ahead);
+      if constexpr (Cfg::LOOKAHEAD) {
+        if (more) {
+          locate(next);
+          row_fetch<Cfg, FAST>(g, t, ahead);
+        }
       }
       float acc[Cfg::CH][8];
       float rv[2];
       float av[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8];
-      row_main<Cfg>(g, here, cur, gz, acc, rv, av);
+      row_main<Cfg>(g, here, cur, gz, acc, rv, av, red);
       if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, av, hz, cst);
       if (!more) break;
-      cur = ahead;
+      if constexpr (Cfg::LOOKAHEAD) {
+        cur = ahead;
+      } else {
+        locate(next);
+        row_fetch<Cfg, FAST>(g, t, cur);
+      }
       base = next;
     }
   }

@@ -159,14 +159,17 @@ class FusedOpBase:
         """-> (A, lda, batch_stride_A, B, ldb, batch_stride_B) ready for the kernel."""
         raise NotImplementedError("Should be Overwritten by child class")
 
-    def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args) -> Tuple[jit.EvtArgs, list]:
+    def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args, block=None) -> Tuple[jit.EvtArgs, list]:
         """Marshal operands and epilogue tensors into the C-ABI argument block
         (the counterpart of GemmArguments / BmmArguments2x +
         operation.epilogue_type(visitor_args), evt_fuser.py:539-544, :674-678).
-        Returns the block and the tensors it points into (keep them alive)."""
+        Returns the block and the tensors it points into (keep them alive).
+        Without `block` the op's one reused block is filled, valid until the
+        next call; a caller that keeps several argument sets side by side
+        passes a block of its own (`new_argument_block()`) for each."""
         M, N, K, L = self.problem
         A, lda, bsa, B, ldb, bsb = self.operands(args[-2], args[-1])
-        a = self.argument_block()
+        a = block if block is not None else self.argument_block()
         a.M, a.N, a.K, a.L = M, N, K, L
         a.A, a.lda, a.batch_stride_A = A.data_ptr(), lda, bsa
         a.B, a.ldb, a.batch_stride_B = B.data_ptr(), ldb, bsb
@@ -180,19 +183,24 @@ class FusedOpBase:
         counts, strides, immediates) is written once."""
         a = getattr(self, "_evt_args", None)
         if a is None:
-            a = self._evt_args = jit.EvtArgs()
-            a.num_tensors = len(self.ir.slots)
-            a.num_scalars = len(self.ir.scalars)
-            for k, slot in enumerate(self.ir.slots):
-                ta = a.tensors[k]
-                ta.ptr = None
-                ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
-                ta.l_div = slot.strides.l_div
-                ta.l_mod = slot.strides.l_mod
-            for i, sc in enumerate(self.ir.scalars):
-                a.scalars[i] = sc
-            # per call: (slot, where its tensor comes from)
-            self._slot_plan = [(k, *self.slot_sources[k]) for k, slot in enumerate(self.ir.slots) if slot.kind != "rand"]
+            a = self._evt_args = self.new_argument_block()
+        return a
+
+    def new_argument_block(self) -> jit.EvtArgs:
+        """A block with everything but the per-call pointers filled in."""
+        a = jit.EvtArgs()
+        a.num_tensors = len(self.ir.slots)
+        a.num_scalars = len(self.ir.scalars)
+        for k, slot in enumerate(self.ir.slots):
+            ta = a.tensors[k]
+            ta.ptr = None
+            ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
+            ta.l_div = slot.strides.l_div
+            ta.l_mod = slot.strides.l_mod
+        for i, sc in enumerate(self.ir.scalars):
+            a.scalars[i] = sc
+        # per call: (slot, where its tensor comes from)
+        self._slot_plan = [(k, *self.slot_sources[k]) for k, slot in enumerate(self.ir.slots) if slot.kind != "rand"]
         return a
 
     def fill_epilogue_arguments(self, a: jit.EvtArgs, keep: list, visitor_args: Dict[str, torch.Tensor], args) -> None:
@@ -544,10 +552,10 @@ class FusedRowOp(FusedOpBase):
         self.spec = self.row_spec
         self.module = jit.load_module(self.ir, self.row_spec)
 
-    def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args) -> Tuple[jit.EvtArgs, list]:
+    def build_arguments(self, visitor_args: Dict[str, torch.Tensor], *args, block=None) -> Tuple[jit.EvtArgs, list]:
         M, N, _, L = self.problem
         ops = [t.contiguous() for t in args[len(args) - self.num_anchor_inputs:]]
-        a = self.argument_block()
+        a = block if block is not None else self.argument_block()
         a.M, a.N, a.K, a.L = M, N, 1, L
         a.A, a.lda, a.batch_stride_A = ops[0].data_ptr(), N, M * N
         if len(ops) > 1:

@@ -61,6 +61,9 @@ def register_all() -> List[jit.LazyModule]:
             for dt in W.ROW_EDGE_DTYPES:
                 mod, ins = W.row_edge_case(anchor, n, dt)
                 W.fuse(mod, _meta(ins))
+    for anchor, n, dt in W.ROW_LONG_CASES:
+        mod, ins = W.row_edge_case(anchor, n, dt)
+        W.fuse(mod, _meta(ins))
     for name, (cls, shapes, _) in W.ROW_BENCH.items():
         W.fuse(cls(), [torch.empty(sh, dtype=dt, device="meta") for sh, dt in shapes])
     from .aot_helper import aot_capture, evt_backend

@@ -797,6 +797,10 @@ def _row_bench_shapes():
     sm, ln = (256, 512, 512), (131072, 1024)
     h, f = torch.float16, torch.float32
     return {
+        # vocabulary-sized rows (one workgroup of 8 waves per row): BERT's 30522 as it is (no 16-byte accesses:
+        # rows start at odd multiples of 4 bytes) and padded to a multiple of 8
+        "softmax_vocab_30522": (RowBenchSoftmax, [((4096, 30522), h)], 2 * 2 * 4096 * 30522),
+        "softmax_vocab_30528": (RowBenchSoftmax, [((4096, 30528), h)], 2 * 2 * 4096 * 30528),
         # name: (module, [(shape, dtype), ...] inputs, algorithmic bytes per launch)
         "softmax": (RowBenchSoftmax, [(sm, h)], 2 * 2 * 256 * 512 * 512),
         "softmax_backward": (RowBenchSoftmaxBackward, [(sm, h), (sm, h)], 3 * 2 * 256 * 512 * 512),
@@ -849,6 +853,16 @@ class _BareLayerNormBackward(torch.nn.Module):
 
 ROW_EDGE_LENGTHS = (8, 24, 1000, 8192)
 ROW_EDGE_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
+# rows spread over the waves of a workgroup (longer than 8192): vocabulary-sized rows, the longest each anchor
+# takes, lengths that are no multiple of 8
+ROW_LONG_CASES = (
+    ("softmax", 8200, torch.float16), ("softmax", 30522, torch.float16), ("softmax", 50257, torch.bfloat16),
+    ("softmax", 65536, torch.float16), ("softmax", 30522, torch.float32),
+    ("softmax_backward", 8200, torch.float16), ("softmax_backward", 30522, torch.float16),
+    ("softmax_backward", 32768, torch.bfloat16), ("softmax_backward", 16384, torch.float32),
+    ("layernorm", 12288, torch.float16), ("layernorm", 65536, torch.bfloat16),
+    ("layernorm_backward", 12288, torch.float16), ("layernorm_backward", 24000, torch.bfloat16),
+)
 
 
 def row_edge_case(anchor: str, n: int, dtype, seed: int = 0):

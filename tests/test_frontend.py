@@ -281,7 +281,7 @@ def test_row_anchor_patterns_trace(name):
     if kind == "layernorm_backward":
         assert [op.ir.slots[k].name for k in spec["anchor_tensors"]] == ["mean", "invstd", "gamma"]
     if name == "layernorm_backward_full":
-        assert L == 1 and spec["col_state"] == 2 and "Cfg = evt::RowCfg<3, 2, 64, 0, 2, 8>" in op.module.source
+        assert L == 1 and spec["col_state"] == 2 and "Cfg = evt::RowCfg<3, 2, 64, 0, 2, 8, 1>" in op.module.source
     if "column" in name and "broadcast" not in name and "full" not in name:
         # a sum over every row: one batch of L * M rows, partials per workgroup in the workspace
         assert L == 1 and spec["col_state"] == 1 and "sum" in " ".join(op.partition_names)
@@ -322,8 +322,14 @@ def test_row_anchor_limits():
     assert RowSpec.for_row_length("softmax", 512, "f16") == RowSpec("softmax", 2, 32, "f16")
     assert RowSpec.for_row_length("layernorm", 1024, "f16") == RowSpec("layernorm", 2, 64, "f16")
     assert RowSpec.for_row_length("layernorm", 8192, "bf16") == RowSpec("layernorm", 16, 64, "bf16")
-    with pytest.raises(NotImplementedError):
-        RowSpec.for_row_length("softmax", 8200, "f16")
+    # longer rows go over several waves of a workgroup, as few as the registers allow
+    assert RowSpec.for_row_length("softmax", 8200, "f16") == RowSpec("softmax", 9, 64, "f16", 2)
+    assert RowSpec.for_row_length("softmax", 30522, "f16") == RowSpec("softmax", 8, 64, "f16", 8)
+    assert RowSpec.for_row_length("softmax", 65536, "bf16") == RowSpec("softmax", 8, 64, "bf16", 16)
+    assert RowSpec.for_row_length("softmax_backward", 30522, "f16") == RowSpec("softmax_backward", 4, 64, "f16", 16)
+    for op, n, elt in (("softmax", 65537, "f16"), ("layernorm", 50000, "f32"), ("softmax_backward", 32776, "f16")):
+        with pytest.raises(NotImplementedError):
+            RowSpec.for_row_length(op, n, elt)
 
 
 def test_rows_too_long_for_the_row_kernel_stay_eager():
@@ -333,7 +339,7 @@ def test_rows_too_long_for_the_row_kernel_stay_eager():
         def forward(self, x):
             return aten.mul(aten._softmax(x, -1, False), 2.)
 
-    x = torch.empty(4, 16384, dtype=torch.float16, device="meta")
+    x = torch.empty(4, 65600, dtype=torch.float16, device="meta")
     gm = W.fuse(WideSoftmax(), [x])
     assert not fused_nodes(gm)
     assert [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"] == ["_softmax", "mul"]

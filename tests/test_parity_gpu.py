@@ -5,6 +5,8 @@ Tolerances (the contract of the path): max relative error <= 2e-2 for fp16
 outputs and <= 1e-3 for fp32 reduction outputs, measured as
 max |out - ref| / max(|ref|, 1e-2 * rms(ref)).
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -405,6 +407,34 @@ def test_row_anchor_lengths_and_dtypes(anchor, n, dtype):
         assert err <= (REDUCTION_TOL if stat else tol), f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
 
 
+@pytest.mark.parametrize("anchor,n,dtype", W.ROW_LONG_CASES,
+                         ids=[f"{a}-{n}-{str(d).split('.')[-1]}" for a, n, d in W.ROW_LONG_CASES])
+def test_row_anchor_long_rows(anchor, n, dtype):
+    """Rows longer than one wave can cache (8192): the row is spread over the
+    2 .. 16 waves of a workgroup and each row reduction ends with an exchange
+    through LDS.  Vocabulary-sized rows (30522, 50257), the longest rows each
+    anchor takes, odd lengths, three element types, against the fp32 oracle."""
+    mod, inputs = W.row_edge_case(anchor, n, dtype)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    spec = node.target.row_spec
+    assert spec.wpr > 1 and spec.max_n >= n
+    outs = gm(*[t.cuda() for t in inputs])
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    tol = {torch.float16: FP16_TOL, torch.bfloat16: FP16_TOL, torch.float32: REDUCTION_TOL}[dtype]
+    for k, (o, r) in enumerate(zip(outs, refs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        err = evt_oracle.max_rel_err(o, r)
+        # probabilities of a 65536-wide softmax lie below fp16's normal range (6.1e-5), where the output format's
+        # spacing is 2^-24 whatever the value: there the bound is the relative one plus half that spacing
+        d, rr = (o.float().cpu() - r).abs(), r.abs()
+        denormal_ok = dtype == torch.float16 and k == 0 and bool((d <= tol * rr + 2.0 ** -25).all())
+        assert err <= (REDUCTION_TOL if k > 0 else tol) or denormal_ok, \
+            f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
+
+
 def test_aot_encoder_layer_training_step():
     """A transformer encoder layer, forward and backward, through AOT autograd
     with the joint pipeline (the reference's BERT flow, unittest/fx_passes/bert.py:
@@ -568,3 +598,23 @@ def test_aot_decoder_block_with_attention_dropout(dtype):
     for (name, _), g, r in zip(model.named_parameters(), grads, ref_grads):
         err = float((g.float() - r).norm() / r.norm())
         assert err <= tol, f"{name}: norm-wise error {err:.3e}"
+
+
+def test_bench_argument_sets_are_independent():
+    """bench.py keeps several argument blocks per config side by side (rotating
+    buffer sets): each must point at its own buffers, although an op called the
+    ordinary way reuses one block."""
+    import bench
+    case = bench.Case(2, torch, W, fused_nodes)
+    assert case.nsets >= 4
+    blocks = [s[0] for s in case.sets]
+    assert len({ctypes.addressof(b) for b in blocks}) == len(blocks)
+    assert len({b.tensors[k].ptr for b in blocks for k in range(b.num_tensors)}) == len(blocks) * blocks[0].num_tensors
+    for i in range(case.nsets):
+        case.launch(i)
+    torch.cuda.synchronize()
+    first = case.outputs(0)
+    assert all(float(o.float().abs().sum()) > 0 for o in first)
+    for i in range(1, case.nsets):
+        for a, b in zip(first, case.outputs(i)):
+            assert torch.equal(a, b)
