@@ -714,14 +714,16 @@ class RowSpec:
 
     @staticmethod
     def for_row_length(op: str, n: int, elt: str) -> "RowSpec":
-        """Smallest lane group that holds the row in at most 16 chunks, widened
-        to a full wave once a row needs 4 or more chunks per lane (one row per
-        wave keeps every 16-byte access of a wave inside one row).  Rows longer
+        """Smallest lane group that holds the row in two chunks per lane (four
+        for softmax), a full wave with up to 16 chunks for longer rows.  Rows longer
         than 8192 go over 2 .. 16 waves, as few as keep the row data within
         three quarters of the registers a lane can have at that workgroup size
         (16 waves: 128 registers and no fetch ahead)."""
+        # softmax holds one operand and little else: four chunks per lane, so more rows per wave, measured 12 %
+        # faster on 512-wide rows; the anchors with two operands or two reductions lose with more than two
+        per_lane = 4 if op == "softmax" else 2
         lpr = 8
-        while lpr < 64 and (n + lpr * 8 - 1) // (lpr * 8) > 2:
+        while lpr < 64 and (n + lpr * 8 - 1) // (lpr * 8) > per_lane:
             lpr *= 2
         ch = (n + lpr * 8 - 1) // (lpr * 8)
         if ch <= 16:
@@ -990,6 +992,10 @@ class RowCodegen(Codegen):
         e("// walking pays when row vectors are kept in registers across the rows of a wave, and bounds the number of")
         e("// partials of a per-column reduction")
         default_cap = 4 if ir.col_state else (16 if self.hoisted else 0)
+        if 1 < sp.wpr < 16:
+            # a row per workgroup: 8 waves per CU walk over the rows, each fetching its next row ahead (measured
+            # on 4096 x 30528: 100 us against 108 us with a workgroup per row)
+            default_cap = 8 // sp.wpr
         e("static unsigned grid_for(const evt::RowArgs& g) {")
         e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); int v = s ? atoi(s) : {default_cap}; "
           f"return {'v > 0 ? v : 4' if ir.col_state else 'v'}; }}();")

@@ -319,7 +319,8 @@ def test_row_anchor_limits():
     assert [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"].count("sum") == 1
     # row length -> lanes per row and chunks
     assert RowSpec.for_row_length("softmax", 64, "f16") == RowSpec("softmax", 1, 8, "f16")
-    assert RowSpec.for_row_length("softmax", 512, "f16") == RowSpec("softmax", 2, 32, "f16")
+    assert RowSpec.for_row_length("softmax", 512, "f16") == RowSpec("softmax", 4, 16, "f16")
+    assert RowSpec.for_row_length("softmax_backward", 512, "f16") == RowSpec("softmax_backward", 2, 32, "f16")
     assert RowSpec.for_row_length("layernorm", 1024, "f16") == RowSpec("layernorm", 2, 64, "f16")
     assert RowSpec.for_row_length("layernorm", 8192, "bf16") == RowSpec("layernorm", 16, 64, "bf16")
     # longer rows go over several waves of a workgroup, as few as the registers allow
