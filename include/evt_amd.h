@@ -81,7 +81,9 @@ typedef struct EvtTensorArg {
  * input (backward modules: the incoming gradient) and B the second operand of
  * the backward modules (softmax output / forward input), `lda`/`ldb` their row
  * strides and the batch strides their strides between batches, in elements;
- * K is ignored.  N may not exceed the module's "row"."max_n".  A layer norm's
+ * K is ignored.  N may not exceed the module's "row"."max_n"
+ * ("row"."waves_per_row" > 1: one workgroup per row).  Rows are read with
+ * 16-byte accesses when A / B and their strides are 4-byte aligned.  A layer norm's
  * eps is scalars["anchor_scalars"]; layer norm backward reads the forward
  * pass's mean and rstd (fp32, one per row, contiguous) and optionally the
  * weight from the tensor slots listed under "anchor_tensors".  These modules
