@@ -763,6 +763,10 @@ class RowCodegen(Codegen):
         # [N] vectors shared by every row (weight, bias, ...): read once per wave, not once per row
         self.hoisted = [n.name for n in ir.nodes.values() if n.op == "load" and ir.slots[n.slot].kind == "row"
                         and ir.slots[n.slot].strides.stride_l == 0 and n.slot not in ir.anchor_slots]
+        if spec.wpr > 1 or spec.ch * len(self.hoisted) > 8:
+            # long rows: the registers (8 per chunk and vector) go to the row itself; next to 4 KB and more of row
+            # data per lane group the vectors' trip from L2 once per row is small
+            self.hoisted = []
 
     def slot_row_off(self, k: int) -> str:
         return f"o_{k}"

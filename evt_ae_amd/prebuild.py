@@ -61,6 +61,10 @@ def register_all() -> List[jit.LazyModule]:
             for dt in W.ROW_EDGE_DTYPES:
                 mod, ins = W.row_edge_case(anchor, n, dt)
                 W.fuse(mod, _meta(ins))
+    from .passes import pass_decomposition, pass_fusion
+    for n in W.AFFINE_LN_LENGTHS:
+        mod, ins = W.affine_layer_norm(n)
+        W.fuse(mod, _meta(ins), passes=[pass_decomposition, pass_fusion])
     for anchor, n, dt in W.ROW_LONG_CASES:
         mod, ins = W.row_edge_case(anchor, n, dt)
         W.fuse(mod, _meta(ins))

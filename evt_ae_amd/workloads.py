@@ -851,6 +851,26 @@ class _BareLayerNormBackward(torch.nn.Module):
         return operator.getitem(ln, 0)
 
 
+class AffineLayerNorm(torch.nn.Module):
+    """Layer norm with weight and bias over rows of any length (GPT-3's hidden size 12288 goes over two waves)."""
+    def __init__(self, n):
+        super().__init__()
+        self.n = n
+
+    def forward(self, x, w, b):
+        ln = aten.native_layer_norm(x, [self.n], w, b, 1e-5)
+        return operator.getitem(ln, 0), operator.getitem(ln, 1), operator.getitem(ln, 2)
+
+
+def affine_layer_norm(n: int, dtype=torch.float16, rows: int = 40, seed: int = 0):
+    g = torch.Generator(device="cpu").manual_seed(0xAF1 + n + seed)
+    x = (torch.randn(rows, n, generator=g) * 1.5 + 0.25).to(dtype)
+    w = (1.0 + 0.2 * torch.randn(n, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(n, generator=g)).to(dtype)
+    return AffineLayerNorm(n), [x, w, b]
+
+
+AFFINE_LN_LENGTHS = (8192, 12288, 20480)
 ROW_EDGE_LENGTHS = (8, 24, 1000, 8192)
 ROW_EDGE_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
 # rows spread over the waves of a workgroup (longer than 8192): vocabulary-sized rows, the longest each anchor

@@ -435,6 +435,26 @@ def test_row_anchor_long_rows(anchor, n, dtype):
             f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
 
 
+@pytest.mark.parametrize("n", W.AFFINE_LN_LENGTHS)
+def test_layer_norm_with_weight_and_bias_on_long_rows(n):
+    """native_layer_norm with weight and bias (moved into the epilogue by
+    pass_decomposition) on rows of 8192 (16 chunks in one wave), 12288 and 20480
+    elements (rows over several waves; the [N] vectors are then read per row
+    instead of being kept in registers)."""
+    from evt_ae_amd.passes import pass_decomposition, pass_fusion
+    mod, inputs = W.affine_layer_norm(n)
+    gm = W.fuse(mod, inputs, passes=[pass_decomposition, pass_fusion])
+    (node,) = fused_nodes(gm)
+    assert type(node.target).__name__ == "FusedLayerNorm" and node.target.row_spec.max_n >= n
+    outs = list(gm(*[t.cuda() for t in inputs]))
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    for k, (o, r) in enumerate(zip(outs, refs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        err = evt_oracle.max_rel_err(o, r)
+        assert err <= (REDUCTION_TOL if k > 0 else FP16_TOL), f"n={n} output {k}: max rel err {err:.3e}"
+
+
 def test_aot_encoder_layer_training_step():
     """A transformer encoder layer, forward and backward, through AOT autograd
     with the joint pipeline (the reference's BERT flow, unittest/fx_passes/bert.py:
