@@ -851,6 +851,85 @@ class _BareLayerNormBackward(torch.nn.Module):
         return operator.getitem(ln, 0)
 
 
+class RandomEpilogue(torch.nn.Module):
+    """A seeded random epilogue tree behind a GEMM: 5 .. 9 element-wise steps
+    over the accumulator, a same-shape tensor, a row vector, a column vector
+    and immediates, drawn from the fuser's vocabulary; one or two results are
+    stored, and a per-row or per-column sum of one of them may come on top.
+    Beyond the reference's hand-written patterns: the generator has no idea
+    which combinations are easy."""
+    UNARY = ("relu", "tanh", "sigmoid", "neg", "abs", "gelu", "exp_small", "sqrt_abs", "rsqrt_abs1")
+    BINARY = ("add", "sub", "mul", "maximum", "minimum", "div_abs1", "where_gt")
+
+    def __init__(self, seed: int):
+        super().__init__()
+        import random
+        rng = random.Random(0xE71 + seed)
+        self.steps = []
+        n_vals = 4                       # accum, aux, row, col
+        # the first operand of every step comes from the accumulator's side (value 0 or an earlier step), so the
+        # whole tree belongs to the epilogue: a side expression run eagerly would hand over an fp16-rounded
+        # tensor, and a later subtraction can blow that rounding up beyond any fixed tolerance
+        from_acc = lambda: rng.choice([0] + list(range(4, n_vals)))   # noqa: E731
+        for _ in range(rng.randint(5, 9)):
+            if rng.random() < 0.45:
+                self.steps.append((rng.choice(self.UNARY), from_acc(), None))
+            else:
+                a = from_acc()
+                op = rng.choice(self.BINARY)
+                tensor_only = op in ("maximum", "minimum")         # aten.maximum / minimum take no immediates
+                b = rng.randrange(n_vals) if tensor_only or rng.random() < 0.75 else ("imm", rng.choice((0.5, -1.25, 2.0, 0.1)))
+                self.steps.append((op, a, b))
+            n_vals += 1
+        # results: the last value and possibly an earlier full-size one; the last always depends on the accumulator
+        self.extra = rng.randrange(4, n_vals - 1) if rng.random() < 0.6 else None      # an earlier step's value
+        self.reduce = rng.choice((None, None, 0, 1))
+
+    def forward(self, A, B, aux, row, col):
+        acc = aten.mm(A, B)
+        vals = [acc, aux, row, col]
+        for op, a, b in self.steps:
+            x = vals[a]
+            imm = isinstance(b, tuple)
+            y = None if b is None else (b[1] if imm else vals[b])
+            if op == "exp_small":
+                r = aten.exp(aten.mul(x, 0.125))
+            elif op == "sqrt_abs":
+                r = aten.sqrt(aten.abs(x))
+            elif op == "rsqrt_abs1":
+                r = aten.rsqrt(aten.add(aten.abs(x), 1.0))
+            elif op == "gelu":
+                r = aten.gelu(x, approximate="tanh")
+            elif op == "div_abs1":
+                d = abs(y) + 1.0 if imm else aten.add(aten.abs(y), 1.0)
+                r = aten.div(x, d)
+            elif op == "where_gt":
+                other = aten.mul(x, y) if imm else y
+                r = aten.where(aten.gt(x, other), x, aten.mul(other, 0.5))
+            elif b is None:
+                r = getattr(aten, op)(x)
+            else:
+                r = getattr(aten, op)(x, y)
+            vals.append(r)
+        last = aten.add(vals[-1], aten.mul(acc, 0.25))          # full size, accumulator inside
+        outs = [last]
+        if self.extra is not None:
+            outs.append(aten.add(vals[self.extra], aux))           # full size whatever the value's own shape
+        if self.reduce is not None:
+            outs.append(aten.sum(aten.abs(last), [self.reduce], True))
+        return tuple(outs)
+
+
+RANDOM_EPILOGUE_SEEDS = tuple(range(12))
+
+
+def random_epilogue(seed: int, M: int = 320, N: int = 192, K: int = 96):
+    """(module, CPU inputs) of the seeded random epilogue; M, N, K are no multiples of the large tiles."""
+    g = torch.Generator(device="cpu").manual_seed(0xE71 + seed)
+    h = lambda *sh: (torch.randn(*sh, generator=g) * 0.5).half()   # noqa: E731
+    return RandomEpilogue(seed), [h(M, K), h(K, N), h(M, N), h(N), h(M, 1)]
+
+
 class AffineLayerNorm(torch.nn.Module):
     """Layer norm with weight and bias over rows of any length (GPT-3's hidden size 12288 goes over two waves)."""
     def __init__(self, n):

@@ -435,6 +435,31 @@ def test_row_anchor_long_rows(anchor, n, dtype):
             f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
 
 
+@pytest.mark.parametrize("seed", W.RANDOM_EPILOGUE_SEEDS)
+def test_random_epilogue_trees(seed):
+    """Seeded random epilogue trees behind a 320 x 192 x 96 GEMM (no multiple of the
+    large tiles): 5 .. 9 element-wise steps from the fuser's vocabulary over the
+    accumulator, a same-shape tensor, a row vector, a column vector and
+    immediates, one or two stored results, sometimes a per-row or per-column sum.
+    Whatever part of the tree the partitioner gives the GEMM, every output must
+    match the fp32 oracle."""
+    mod, inputs = W.random_epilogue(seed)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    assert type(node.target).__name__ == "FusedGEMM"
+    outs = gm(*[t.cuda() for t in inputs])
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    assert len(outs) == len(refs)
+    for k, (o, r) in enumerate(zip(outs, refs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        reduced = r.numel() < inputs[2].numel()
+        err = evt_oracle.max_rel_err(o, r)
+        assert err <= (REDUCTION_TOL if reduced and o.dtype == torch.float32 else FP16_TOL), \
+            f"seed {seed} output {k}: max rel err {err:.3e}"
+
+
 @pytest.mark.parametrize("n", W.AFFINE_LN_LENGTHS)
 def test_layer_norm_with_weight_and_bias_on_long_rows(n):
     """native_layer_norm with weight and bias (moved into the epilogue by
