@@ -65,9 +65,10 @@ def register_all() -> List[jit.LazyModule]:
     for n in W.AFFINE_LN_LENGTHS:
         mod, ins = W.affine_layer_norm(n)
         W.fuse(mod, _meta(ins), passes=[pass_decomposition, pass_fusion])
-    for seed in W.RANDOM_EPILOGUE_SEEDS:
-        mod, ins = W.random_epilogue(seed)
-        W.fuse(mod, _meta(ins))
+    for anchor in W.RANDOM_EPILOGUE_ANCHORS:
+        for seed in W.RANDOM_EPILOGUE_SEEDS[:12 if anchor == "mm" else 6]:
+            mod, ins = W.random_epilogue(seed, anchor)
+            W.fuse(mod, _meta(ins))
     for anchor, n, dt in W.ROW_LONG_CASES:
         mod, ins = W.row_edge_case(anchor, n, dt)
         W.fuse(mod, _meta(ins))

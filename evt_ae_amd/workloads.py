@@ -861,10 +861,11 @@ class RandomEpilogue(torch.nn.Module):
     UNARY = ("relu", "tanh", "sigmoid", "neg", "abs", "gelu", "exp_small", "sqrt_abs", "rsqrt_abs1")
     BINARY = ("add", "sub", "mul", "maximum", "minimum", "div_abs1", "where_gt")
 
-    def __init__(self, seed: int):
+    def __init__(self, seed: int, anchor: str = "mm", n: int = 0):
         super().__init__()
         import random
-        rng = random.Random(0xE71 + seed)
+        rng = random.Random(0xE71 + seed + 1000 * ("mm", "bmm", "softmax", "layernorm").index(anchor))
+        self.anchor, self.n = anchor, n
         self.steps = []
         n_vals = 4                       # accum, aux, row, col
         # the first operand of every step comes from the accumulator's side (value 0 or an earlier step), so the
@@ -884,9 +885,18 @@ class RandomEpilogue(torch.nn.Module):
         # results: the last value and possibly an earlier full-size one; the last always depends on the accumulator
         self.extra = rng.randrange(4, n_vals - 1) if rng.random() < 0.6 else None      # an earlier step's value
         self.reduce = rng.choice((None, None, 0, 1))
+        if anchor in ("softmax", "layernorm") and self.reduce == 1:
+            self.reduce = 0              # behind a row-wise anchor only sums over the rows are fused
 
     def forward(self, A, B, aux, row, col):
-        acc = aten.mm(A, B)
+        if self.anchor == "mm":
+            acc = aten.mm(A, B)
+        elif self.anchor == "bmm":
+            acc = aten.bmm(A, B)
+        elif self.anchor == "softmax":
+            acc = aten._softmax(A, -1, False)
+        else:
+            acc = operator.getitem(aten.native_layer_norm(A, [self.n], None, None, 1e-5), 0)
         vals = [acc, aux, row, col]
         for op, a, b in self.steps:
             x = vals[a]
@@ -916,18 +926,28 @@ class RandomEpilogue(torch.nn.Module):
         if self.extra is not None:
             outs.append(aten.add(vals[self.extra], aux))           # full size whatever the value's own shape
         if self.reduce is not None:
-            outs.append(aten.sum(aten.abs(last), [self.reduce], True))
+            outs.append(aten.sum(aten.abs(last), [self.reduce + (1 if self.anchor == "bmm" else 0)], True))
         return tuple(outs)
 
 
 RANDOM_EPILOGUE_SEEDS = tuple(range(12))
 
 
-def random_epilogue(seed: int, M: int = 320, N: int = 192, K: int = 96):
-    """(module, CPU inputs) of the seeded random epilogue; M, N, K are no multiples of the large tiles."""
+RANDOM_EPILOGUE_ANCHORS = ("mm", "bmm", "softmax", "layernorm")
+
+
+def random_epilogue(seed: int, anchor: str = "mm", M: int = 320, N: int = 192, K: int = 96, L: int = 3):
+    """(module, CPU inputs) of the seeded random epilogue behind `anchor`; M, N, K are no multiples of the
+    large tiles.  The row-wise anchors take A alone ([M, N]); B is an unused input there."""
     g = torch.Generator(device="cpu").manual_seed(0xE71 + seed)
     h = lambda *sh: (torch.randn(*sh, generator=g) * 0.5).half()   # noqa: E731
-    return RandomEpilogue(seed), [h(M, K), h(K, N), h(M, N), h(N), h(M, 1)]
+    if anchor == "mm":
+        ins = [h(M, K), h(K, N), h(M, N), h(N), h(M, 1)]
+    elif anchor == "bmm":
+        ins = [h(L, M, K), h(L, K, N), h(L, M, N), h(N), h(M, 1)]
+    else:
+        ins = [h(M, N) * 4, h(1), h(M, N), h(N), h(M, 1)]
+    return RandomEpilogue(seed, anchor, N), ins
 
 
 class AffineLayerNorm(torch.nn.Module):

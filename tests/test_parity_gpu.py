@@ -14,6 +14,7 @@ import torch
 from evt_ae_amd import workloads as W
 from evt_ae_amd.autotuner.tuner_base import force_tile
 from oracle import evt_oracle
+from evt_ae_amd.passes import target_name
 from tests.util import fused_nodes, rand_slot
 
 aten = torch.ops.aten
@@ -435,18 +436,26 @@ def test_row_anchor_long_rows(anchor, n, dtype):
             f"{anchor} n={n} {dtype} output {k}: max rel err {err:.3e}"
 
 
-@pytest.mark.parametrize("seed", W.RANDOM_EPILOGUE_SEEDS)
-def test_random_epilogue_trees(seed):
-    """Seeded random epilogue trees behind a 320 x 192 x 96 GEMM (no multiple of the
-    large tiles): 5 .. 9 element-wise steps from the fuser's vocabulary over the
-    accumulator, a same-shape tensor, a row vector, a column vector and
-    immediates, one or two stored results, sometimes a per-row or per-column sum.
-    Whatever part of the tree the partitioner gives the GEMM, every output must
-    match the fp32 oracle."""
-    mod, inputs = W.random_epilogue(seed)
+_RANDOM_TREES = [(a, s) for a in W.RANDOM_EPILOGUE_ANCHORS for s in W.RANDOM_EPILOGUE_SEEDS[:12 if a == "mm" else 6]]
+
+
+@pytest.mark.parametrize("anchor,seed", _RANDOM_TREES, ids=[f"{a}-{s}" for a, s in _RANDOM_TREES])
+def test_random_epilogue_trees(anchor, seed):
+    """Seeded random epilogue trees behind a 320 x 192 x 96 GEMM, a batch of three
+    such products, a softmax and a layer norm over 320 x 192 (no multiples of the
+    large tiles or of a lane group): 5 .. 9 element-wise steps from the fuser's
+    vocabulary over the anchor's result, a same-shape tensor, a row vector, a
+    column vector and immediates, one or two stored results, sometimes a sum over
+    the rows or along them.  The whole tree must end up in one fused kernel and
+    every output must match the fp32 oracle."""
+    mod, inputs = W.random_epilogue(seed, anchor)
     gm = W.fuse(mod, inputs)
     (node,) = fused_nodes(gm)
-    assert type(node.target).__name__ == "FusedGEMM"
+    assert type(node.target).__name__ == {"mm": "FusedGEMM", "bmm": "FusedBMM", "softmax": "FusedSoftmax",
+                                           "layernorm": "FusedLayerNorm"}[anchor]
+    left = [n for n in gm.graph.nodes if n.op == "call_function" and target_name(n.target) not in ("getitem", "view")
+            and n is not node]
+    assert not left, left
     outs = gm(*[t.cuda() for t in inputs])
     outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
     torch.cuda.synchronize()
@@ -457,7 +466,7 @@ def test_random_epilogue_trees(seed):
         reduced = r.numel() < inputs[2].numel()
         err = evt_oracle.max_rel_err(o, r)
         assert err <= (REDUCTION_TOL if reduced and o.dtype == torch.float32 else FP16_TOL), \
-            f"seed {seed} output {k}: max rel err {err:.3e}"
+            f"{anchor} seed {seed} output {k}: max rel err {err:.3e}"
 
 
 @pytest.mark.parametrize("n", W.AFFINE_LN_LENGTHS)
