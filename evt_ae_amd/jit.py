@@ -14,6 +14,7 @@ import ctypes
 import hashlib
 import json
 import re
+import logging
 import os
 import sqlite3
 import subprocess
@@ -154,6 +155,7 @@ def compile_source(source: str, out: Path, extra_flags=()) -> None:
     src.write_text(source)
     tmp = out.with_suffix(f".tmp{os.getpid()}.so")
     cmd = [HIPCC, *HIPCC_FLAGS, *extra_flags, f"-I{CSRC_DIR}", f"-I{INCLUDE_DIR}", str(src), "-o", str(tmp)]
+    logging.getLogger("evt_ae_amd.jit").info("compiling %s", src.name)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{proc.stderr[-4000:]}")

@@ -49,6 +49,10 @@ def register_all() -> List[jit.LazyModule]:
             if shapes is None:   # the benchmark's --clock-probe builds of the headline kernels
                 op = W.fused_nodes(gm)[0].target
                 jit.load_module(op.ir, op.spec, clock_probe=True)
+    # shapes of single tests: the determinism test's classifier, bf16 operands
+    W.fuse(W.CONFIGS[5].module(), _shapes_of(5, dict(M=256, N=8192, K=256)))
+    W.fuse(W.CONFIGS[1].module(), [torch.empty(t.shape, dtype=torch.bfloat16 if t.dtype == torch.float16 else t.dtype,
+                                               device="meta") for t in _shapes_of(1, W.SMALL_SHAPES[1])])
     for name, (cls, _) in W.RANDOM_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
     W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
