@@ -192,7 +192,7 @@ class AutoTunerBase:
         nbytes = (A.numel() + B.numel()) * 2
         for k, s in enumerate(self.ir.slots):
             st = s.strides
-            span = ((L - 1) // st.l_div) * st.stride_l + (M - 1) * st.stride_m + (N - 1) * st.stride_n + 1
+            span = ((L - 1) // st.l_div) * st.stride_l + (st.l_div - 1) * st.stride_l2 + (M - 1) * st.stride_m + (N - 1) * st.stride_n + 1
             dtype = DTYPE_BY_NAME[s.dtype]
             if dtype.is_floating_point:
                 t = torch.randn(span, device=dev, dtype=torch.float32).to(dtype)
@@ -202,6 +202,7 @@ class AutoTunerBase:
             nbytes += t.numel() * t.element_size()
             ta = a.tensors[k]
             ta.ptr, ta.stride_l, ta.stride_m, ta.stride_n, ta.l_div = t.data_ptr(), st.stride_l, st.stride_m, st.stride_n, st.l_div
+            ta.l_mod, ta.stride_l2 = st.l_mod, st.stride_l2
         for i, v in enumerate(self.ir.scalars):
             a.scalars[i] = v
         return a, keep, nbytes

@@ -146,7 +146,7 @@ class Codegen:
         raise NotImplementedError(n.op)
 
     def slot_off(self, k: int, batch: str = "t.batch") -> str:
-        return f"(int64_t)evt::batch_index({batch}, p.t{k}_lm, p.t{k}_ld) * p.t{k}_sl"
+        return f"evt::batch_offset({batch}, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2)"
 
     # -- sections ---------------------------------------------------------------
     def emit_params(self, e: _Emitter):
@@ -155,7 +155,7 @@ class Codegen:
         for k, s in enumerate(self.ir.slots):
             const = "const " if s.role == "load" else ""
             e(f"{const}{DTYPE_CTYPES[s.dtype]}* t{k};  // {s.role} {s.kind} '{s.name}'")
-            e(f"int64_t t{k}_sl, t{k}_sm, t{k}_sn; int t{k}_ld; int t{k}_lm; int t{k}_vec;")
+            e(f"int64_t t{k}_sl, t{k}_sl2, t{k}_sm, t{k}_sn; int t{k}_ld; int t{k}_lm; int t{k}_vec;")
         e(f"float s[{max(1, len(self.ir.scalars))}];")
         e("int fast;   // every per-element tensor is unit-stride / vector-aligned: interior tiles skip all checks")
         e.dedent()
@@ -490,7 +490,7 @@ class Codegen:
     def module_spec(self) -> dict:
         t = self.spec.tile
         return {
-            "abi": 2,
+            "abi": 3,
             "name": self.name,
             "tile": asdict(t),
             "a_k_contiguous": self.spec.a_kc,
@@ -557,6 +557,9 @@ class Codegen:
         e("g.M = a->M; g.N = a->N; g.K = a->K; g.L = a->L;")
         e("g.A = (const char*)a->A; g.lda = a->lda; g.bsA = a->batch_stride_A;")
         e("g.B = (const char*)a->B; g.ldb = a->ldb; g.bsB = a->batch_stride_B;")
+        e("if (a->batch_div_A < 0 || a->batch_div_B < 0 || a->batch_div_A > 0x7fffffff || a->batch_div_B > 0x7fffffff) return EVT_ERR_BAD_ARGS;")
+        e("g.bdivA = a->batch_div_A > 1 ? (int)a->batch_div_A : 1; g.bs2A = a->batch_div_A > 1 ? a->batch_stride2_A : 0;")
+        e("g.bdivB = a->batch_div_B > 1 ? (int)a->batch_div_B : 1; g.bs2B = a->batch_div_B > 1 ? a->batch_stride2_B : 0;")
         e("g.tiles_m = (a->M + Cfg::BM - 1) / Cfg::BM;")
         e("g.tiles_n = (a->N + Cfg::BN - 1) / Cfg::BN;")
         e("g.workspace = nullptr;")
@@ -606,7 +609,7 @@ class Codegen:
         if t.dma:
             e("// fast path: 16-byte global->LDS transfers, buffer range check for the tails")
             e("if (((uintptr_t)a->A | (uintptr_t)a->B) & 15) return EVT_ERR_ALIGNMENT;")
-            e("if ((a->lda | a->ldb | a->batch_stride_A | a->batch_stride_B) & 7) return EVT_ERR_ALIGNMENT;")
+            e("if ((a->lda | a->ldb | a->batch_stride_A | a->batch_stride_B | g.bs2A | g.bs2B) & 7) return EVT_ERR_ALIGNMENT;")
             if sp.a_kc:
                 e("if (a->K & 7) return EVT_ERR_ALIGNMENT;")
                 e("if ((int64_t)Cfg::BM * a->lda * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
@@ -627,10 +630,10 @@ class Codegen:
             else:
                 e("  if (!x.ptr || x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
             e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
-            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div; "
-              f"p.t{k}_lm = (int)x.l_mod;")
+            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sl2 = x.stride_l2; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; "
+              f"p.t{k}_ld = (int)x.l_div; p.t{k}_lm = (int)x.l_mod;")
             e(f"  p.t{k}_vec = (x.stride_n == 1 ? 1 : 0) | ((x.stride_n == 1 && ((uintptr_t)x.ptr % (sizeof({ct}) * Cfg::NI)) == 0 && "
-              f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0) ? 2 : 0); }}")
+              f"x.stride_m % Cfg::NI == 0 && x.stride_l % Cfg::NI == 0 && x.stride_l2 % Cfg::NI == 0) ? 2 : 0); }}")
         e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
         tile_slots = [k for k, sl in enumerate(ir.slots)
                       if (sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux")]
@@ -809,7 +812,7 @@ class RowCodegen(Codegen):
           f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8], float (&cst)[{max(ir.col_state, 1)}][Cfg::CH][8]) {{")
         e.indent()
         for k, s in enumerate(ir.slots):
-            e(f"const int64_t o_{k} = (int64_t)evt::batch_index(t.l, p.t{k}_lm, p.t{k}_ld) * p.t{k}_sl + (int64_t)t.m * p.t{k}_sm;")
+            e(f"const int64_t o_{k} = evt::batch_offset(t.l, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2) + (int64_t)t.m * p.t{k}_sm;")
         for name in outer:
             n = ir.nodes[name]
             c = _cname(name)
@@ -886,7 +889,7 @@ class RowCodegen(Codegen):
     def module_spec(self) -> dict:
         sp = self.row_spec
         return {
-            "abi": 2,
+            "abi": 3,
             "name": self.name,
             "anchor": sp.op,
             "row": {"chunks": sp.ch, "lanes_per_row": sp.lpr * sp.wpr, "waves_per_row": sp.wpr, "max_n": sp.max_n},
@@ -971,10 +974,10 @@ class RowCodegen(Codegen):
             else:
                 e("  if (!x.ptr || x.l_div <= 0 || x.l_mod < 0) return EVT_ERR_BAD_ARGS;")
             e(f"  p.t{k} = ({'const ' if s.role == 'load' else ''}{ct}*)x.ptr;")
-            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; p.t{k}_ld = (int)x.l_div; "
-              f"p.t{k}_lm = (int)x.l_mod;")
+            e(f"  p.t{k}_sl = x.stride_l; p.t{k}_sl2 = x.stride_l2; p.t{k}_sm = x.stride_m; p.t{k}_sn = x.stride_n; "
+              f"p.t{k}_ld = (int)x.l_div; p.t{k}_lm = (int)x.l_mod;")
             e(f"  p.t{k}_vec = (x.stride_n == 1 && (((uintptr_t)x.ptr | (uintptr_t)(x.stride_m * (int64_t)sizeof({ct})) | "
-              f"(uintptr_t)(x.stride_l * (int64_t)sizeof({ct}))) & 3) == 0) ? 1 : 0; }}")
+              f"(uintptr_t)(x.stride_l * (int64_t)sizeof({ct})) | (uintptr_t)(x.stride_l2 * (int64_t)sizeof({ct}))) & 3) == 0) ? 1 : 0; }}")
         for name in self.hoisted:
             k = ir.nodes[name].slot
             e(f"if (a->tensors[{k}].stride_l != 0 || a->tensors[{k}].stride_m != 0) return EVT_ERR_BAD_ARGS;   // read once per wave")

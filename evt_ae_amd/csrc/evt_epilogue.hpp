@@ -395,6 +395,11 @@ __host__ __device__ inline WsLayout ws_layout_split(const GemmArgs& g) {
 __host__ __device__ inline int batch_index(int batch, int l_mod, int l_div) {
   return (l_mod > 0 ? batch % l_mod : batch) / l_div;
 }
+// element offset of a batch: two levels, batch = outer * l_div + inner (stride_l2 = 0: the l_div inner ones share)
+__host__ __device__ inline int64_t batch_offset(int batch, int l_mod, int l_div, int64_t stride_l, int64_t stride_l2) {
+  const int lb = l_mod > 0 ? batch % l_mod : batch;
+  return (int64_t)(lb / l_div) * stride_l + (int64_t)(lb % l_div) * stride_l2;
+}
 // folded per-row reductions: the result a batch contributes to, and the j-th batch that contributes to a result
 __host__ __device__ inline int fold_key(const GemmArgs& g, int batch) {
   return g.row_fold_count == 1 ? batch : (g.row_fold_mod ? batch % g.row_fold_step : batch / g.row_fold_count);

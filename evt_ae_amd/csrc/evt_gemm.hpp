@@ -51,6 +51,10 @@ struct GemmArgs {
   int64_t lda, bsA;   // elements
   const char* B;
   int64_t ldb, bsB;   // elements
+  // two-level batch index of an operand: batch l starts (l / bdiv) * bs + (l % bdiv) * bs2 elements in
+  // (bdiv = 1: one level); a [B, S, H, D] tensor then serves as B * H batches of [S, D] without a copy
+  int bdivA, bdivB;
+  int64_t bs2A, bs2B;
   int tiles_m, tiles_n;
   char* workspace;
   // phase 2 of a cross-tile reduction runs inside this kernel (last workgroup
@@ -731,8 +735,10 @@ struct Mainloop {
       // this workgroup's share of K: [k_lo, k_lo + Kw)
       const int k_lo = split * g.k_chunk;
       const int Kw_ = g.K - k_lo < g.k_chunk ? g.K - k_lo : g.k_chunk;
-      const char* pa = g.A + ((int64_t)batch * g.bsA + (Cfg::A_KC ? (int64_t)m0 * g.lda + k_lo : (int64_t)m0 + (int64_t)k_lo * g.lda)) * 2;
-      const char* pb = g.B + ((int64_t)batch * g.bsB + (Cfg::B_KC ? (int64_t)n0 * g.ldb + k_lo : (int64_t)n0 + (int64_t)k_lo * g.ldb)) * 2;
+      const int64_t boA = (int64_t)(batch / g.bdivA) * g.bsA + (int64_t)(batch % g.bdivA) * g.bs2A;
+      const int64_t boB = (int64_t)(batch / g.bdivB) * g.bsB + (int64_t)(batch % g.bdivB) * g.bs2B;
+      const char* pa = g.A + (boA + (Cfg::A_KC ? (int64_t)m0 * g.lda + k_lo : (int64_t)m0 + (int64_t)k_lo * g.lda)) * 2;
+      const char* pb = g.B + (boB + (Cfg::B_KC ? (int64_t)n0 * g.ldb + k_lo : (int64_t)n0 + (int64_t)k_lo * g.ldb)) * 2;
       a.init(pa, g.lda, g.M - m0, Kw_, tid);
       b.init(pb, g.ldb, g.N - n0, Kw_, tid);
     }

@@ -189,6 +189,7 @@ class FusedOpBase:
     def new_argument_block(self) -> jit.EvtArgs:
         """A block with everything but the per-call pointers filled in."""
         a = jit.EvtArgs()
+        a.batch_div_A = a.batch_div_B = 1
         a.num_tensors = len(self.ir.slots)
         a.num_scalars = len(self.ir.scalars)
         for k, slot in enumerate(self.ir.slots):
@@ -197,6 +198,7 @@ class FusedOpBase:
             ta.stride_l, ta.stride_m, ta.stride_n = slot.strides.stride_l, slot.strides.stride_m, slot.strides.stride_n
             ta.l_div = slot.strides.l_div
             ta.l_mod = slot.strides.l_mod
+            ta.stride_l2 = slot.strides.stride_l2
         for i, sc in enumerate(self.ir.scalars):
             a.scalars[i] = sc
         # per call: (slot, where its tensor comes from)
@@ -364,6 +366,47 @@ class FusedOpBase:
         return 1
 
 
+# layout-only ops between a tensor in memory and a batched-product operand (the head split of an attention layer:
+# view [B, S, H, D] -> permute [0, 2, 1, 3] -> expand -> clone -> view [B * H, S, D])
+_OPERAND_CHAIN_OPS = ("view", "_unsafe_view", "reshape", "permute", "expand", "clone", "unsqueeze", "squeeze")
+
+
+def operand_chain(node, allowed=None) -> Tuple[List[Node], Any]:
+    """The layout-only nodes, each with one user, that end in the operand
+    `node`, in graph order, and the tensor they start from."""
+    chain: List[Node] = []
+    while (isinstance(node, Node) and node.op == "call_function" and target_name(node.target) in _OPERAND_CHAIN_OPS
+           and len(node.users) == 1 and (allowed is None or allowed(node))):
+        chain.append(node)
+        node = node.args[0]
+    chain.reverse()
+    return chain, node
+
+
+def operand_strides(chain: Sequence[Node], shape3: Sequence[int]) -> Optional[Strides]:
+    """Addressing of the operand [L, R, C] that `chain` produces inside the
+    (contiguous) tensor the chain starts from: offset(l, r, c) = (l // l_div)
+    * stride_l + (l % l_div) * stride_l2 + r * stride_m + c * stride_n, or None
+    when the chain does not reduce to that form (a copy is needed then)."""
+    L, R, C = (int(x) for x in shape3)
+    coord = Coord((L, R, C), lambda l, m, n: (l * R + m) * C + n)
+    for node in reversed(chain):
+        in_shape, _ = node_shape_dtype(node.args[0])
+        if target_name(node.target) == "permute":
+            coord = coord.inverse_permute([int(d) for d in node.args[1]], in_shape)
+        else:
+            numel = 1
+            for d in in_shape:
+                numel *= int(d)
+            if numel != coord.numel():        # an expand that broadcasts
+                return None
+            coord = coord.reshape(in_shape)
+    st = fit_strides(coord, L, R, C)
+    if st is None or st.l_mod:
+        return None
+    return st
+
+
 def _dma_ok(a_kc: bool, b_kc: bool, M: int, N: int, K: int, lda: int, ldb: int, bsa: int, bsb: int) -> bool:
     """The fast global->LDS path moves 16-byte chunks: every operand row must
     start on a 16-byte boundary and the contiguous extent must be a multiple
@@ -440,7 +483,10 @@ class FusedGEMM(FusedOpBase):
 
 class FusedBMM(FusedOpBase):
     """Batched variant; A/B may be 3-D permutations of their source tensors
-    (reference: evt_fuser.py:561-697, python/gtl/ops/bmm.py:23-64)."""
+    (reference: evt_fuser.py:561-697, python/gtl/ops/bmm.py:23-64), or come out
+    of any chain of views, permutes and copies that amounts to strided
+    addressing with a batch index in two levels (the head split / merge of an
+    attention layer), which the kernel then reads in place."""
     __name__ = "cutlass_bmm_with_visitor"
     target = aten.bmm
     mainloop_fusion_targets = [aten.permute]
@@ -448,12 +494,6 @@ class FusedBMM(FusedOpBase):
     def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
         super().__init__(node, epilogue_visitor)
         lhs_node, rhs_node = node.args[0], node.args[1]
-        self.A = self.get_src(lhs_node)
-        self.B = self.get_src(rhs_node)
-        self.args = [self.A, self.B]
-        self.permute_A = self.get_permutation(lhs_node)
-        self.permute_B = self.get_permutation(rhs_node)
-
         lhs_shape, dtype = node_shape_dtype(lhs_node)
         rhs_shape, _ = node_shape_dtype(rhs_node)
         L, M, K = lhs_shape
@@ -462,28 +502,34 @@ class FusedBMM(FusedOpBase):
         if dtype not in (torch.float16, torch.bfloat16):
             raise NotImplementedError(f"BMM operands of dtype {dtype}")
 
-        # strides of the logical [L, M, K] / [L, K, N] operands inside their
-        # (contiguous) source tensors
-        sa = self._logical_strides(self.A, self.permute_A)
-        sb = self._logical_strides(self.B, self.permute_B)
+        # the layout-only producers of each operand that belong to the partition, and the operand's strides
+        # inside the (contiguous) tensor they start from
+        inside = lambda n: n.name in self.partition_names      # noqa: E731
+        self.chain_A, self.A = operand_chain(lhs_node, inside)
+        self.chain_B, self.B = operand_chain(rhs_node, inside)
+        sa = operand_strides(self.chain_A, lhs_shape)
+        sb = operand_strides(self.chain_B, rhs_shape)
+        self.args = [self.A, self.B]
         self.copy_A = self.copy_B = False
-        if sa[2] == 1:
-            self.a_kc, self.lda, self.bsa = True, sa[1], sa[0]
-        elif sa[1] == 1:
-            self.a_kc, self.lda, self.bsa = False, sa[2], sa[0]
-        else:   # batch-last source: make the permuted operand contiguous first (evt_fuser.py:663-672)
-            self.copy_A, self.a_kc, self.lda, self.bsa = True, True, K, M * K
-        if sb[1] == 1:
-            self.b_kc, self.ldb, self.bsb = True, sb[2], sb[0]
-        elif sb[2] == 1:
-            self.b_kc, self.ldb, self.bsb = False, sb[1], sb[0]
+        self.bdiva, self.bs2a, self.bdivb, self.bs2b = 1, 0, 1, 0
+        if sa is not None and sa.stride_n == 1 and (M == 1 or sa.stride_m >= K):
+            self.a_kc, self.lda = True, (sa.stride_m if M > 1 else K)
+        elif sa is not None and sa.stride_m == 1 and (K == 1 or sa.stride_n >= M):
+            self.a_kc, self.lda = False, (sa.stride_n if K > 1 else M)
+        else:   # batch-last source and the like: make the operand contiguous first (evt_fuser.py:663-672)
+            self.copy_A, self.a_kc, self.lda, sa = True, True, K, Strides(M * K, K, 1)
+        if sb is not None and sb.stride_m == 1 and (N == 1 or sb.stride_n >= K):
+            self.b_kc, self.ldb = True, (sb.stride_n if N > 1 else K)
+        elif sb is not None and sb.stride_n == 1 and (K == 1 or sb.stride_m >= N):
+            self.b_kc, self.ldb = False, (sb.stride_m if K > 1 else N)
         else:
-            self.copy_B, self.b_kc, self.ldb, self.bsb = True, False, N, K * N
-        if M == 1 and self.a_kc is False:
-            pass
+            self.copy_B, self.b_kc, self.ldb, sb = True, False, N, Strides(K * N, N, 1)
+        self.bsa, self.bdiva, self.bs2a = sa.stride_l, sa.l_div, sa.stride_l2
+        self.bsb, self.bdivb, self.bs2b = sb.stride_l, sb.l_div, sb.stride_l2
         self.lhs_layout = "RowMajor" if self.a_kc else "ColumnMajor"
         self.rhs_layout = "ColumnMajor" if self.b_kc else "RowMajor"
-        dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb, self.bsa, self.bsb)
+        dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb,
+                      self.bsa | self.bs2a, self.bsb | self.bs2b)
 
         with (_pop_mode_temporarily() if _len_torch_dispatch_stack() > 0 else nullcontext()):
             tuner = BMMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
@@ -492,26 +538,43 @@ class FusedBMM(FusedOpBase):
             self.spec = KernelSpec(self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
             self.module = jit.load_module(self.ir, self.spec)
 
-    def get_permutation(self, node: Node) -> List[int]:
-        if packet(node.target) == aten.permute and node.name in self.partition_names:
-            return [int(i) for i in node.args[1]]
+    # kept for callers that ask which 3-D permutation an operand went through
+    @property
+    def permute_A(self) -> List[int]:
+        return self._single_permute(self.chain_A)
+
+    @property
+    def permute_B(self) -> List[int]:
+        return self._single_permute(self.chain_B)
+
+    @staticmethod
+    def _single_permute(chain) -> List[int]:
+        if len(chain) == 1 and target_name(chain[0].target) == "permute":
+            return [int(i) for i in chain[0].args[1]]
         return [0, 1, 2]
 
     @staticmethod
-    def _logical_strides(src: Node, perm: List[int]) -> Tuple[int, int, int]:
-        shape, _ = node_shape_dtype(src)
-        st = _contig_strides(shape)
-        return tuple(st[p] for p in perm)
+    def _replay(chain, x):
+        """The operand as eager PyTorch computes it from its source tensor."""
+        for node in chain:
+            x = node.target(x, *node.args[1:], **node.kwargs)
+        return x
 
     def operands(self, A, B):
         if self.copy_A:
-            A = aten.permute(A, self.permute_A).contiguous()
+            A = self._replay(self.chain_A, A).contiguous()
         if self.copy_B:
-            B = aten.permute(B, self.permute_B).contiguous()
+            B = self._replay(self.chain_B, B).contiguous()
         return A, self.lda, self.bsa, B, self.ldb, self.bsb
 
+    def build_arguments(self, visitor_args, *args, block=None):
+        a, keep = super().build_arguments(visitor_args, *args, block=block)
+        a.batch_div_A, a.batch_stride2_A = self.bdiva, self.bs2a
+        a.batch_div_B, a.batch_stride2_B = self.bdivb, self.bs2b
+        return a, keep
+
     def anchor_eager(self, A, B):
-        return torch.bmm(aten.permute(A, self.permute_A), aten.permute(B, self.permute_B))
+        return torch.bmm(self._replay(self.chain_A, A), self._replay(self.chain_B, B))
 
 
 def _unsupported_anchor(name: str, where: str):
@@ -678,7 +741,16 @@ class EVTFuser:
             members = set(partition) | set(extra)
             partition = [n for n in graph_module.graph.nodes if n in members]
             self.partition_names = [n.name for n in partition]
-        epilogue_partition = [n for n in partition if n is not anchor and anchor not in n.users]
+        # producers of the anchor's operands inside the partition (layout-only chains) are read through the
+        # operands' strides: main-loop fusion, not epilogue
+        pre: set = set()
+        stack = [a for a in anchor.all_input_nodes if a in partition]
+        while stack:
+            n = stack.pop()
+            if n not in pre:
+                pre.add(n)
+                stack.extend(a for a in n.all_input_nodes if a in partition)
+        epilogue_partition = [n for n in partition if n is not anchor and n not in pre]
         epi_set = set(epilogue_partition)
 
         # Step 2: inputs and outputs of the epilogue, in graph order
@@ -960,7 +1032,7 @@ class EVTFuser:
                 post.insert(0, ("view", list(nshape)))
             node = src
         sshape, _ = node_shape_dtype(node)
-        key = (value, st.stride_l, st.stride_m, st.stride_n, st.l_div, st.l_mod, dtype, domain)
+        key = (value, st.stride_l, st.stride_m, st.stride_n, st.l_div, st.l_mod, st.stride_l2, dtype, domain)
         if key in store_key:
             self.output2store[name] = store_key[key]
             stored_shape = self.store_meta[store_key[key]][0]
@@ -998,7 +1070,7 @@ class EVTFuser:
             st = fit_strides(coord, self.L, self.M, self.N)
             if st is None:
                 raise NotImplementedError(f"input {node.name}: broadcast pattern is not strided in (l, m, n)")
-            key = (node.name, (st.stride_l, st.stride_m, st.stride_n, st.l_div, st.l_mod))
+            key = (node.name, (st.stride_l, st.stride_m, st.stride_n, st.l_div, st.l_mod, st.stride_l2))
             if key in self.load_cache:
                 return self.load_cache[key]
             if dtype not in DTYPE_NAMES:
@@ -1256,7 +1328,7 @@ class EVTFuser:
             # also summed over the batches that agree modulo l_mod (e.g. a [S, B, H*D] view of a BMM over
             # L = B*H batches, reduced over S and B: unittest/evt_fuser/bmm.py:48-67)
             axis, fold, fold_step, fold_count = "row", "mod", st.l_mod, self.L // st.l_mod
-        elif st.stride_n == 0 and not st.l_mod and st.l_div > 1 and numel == (self.L // st.l_div) * self.M:
+        elif st.stride_n == 0 and not st.l_mod and st.l_div > 1 and not st.stride_l2 and numel == (self.L // st.l_div) * self.M:
             axis, fold, fold_step, fold_count = "row", "div", 1, st.l_div     # l_div consecutive batches summed
         elif st.stride_m == 0 and numel == self.L * self.N and (self.L == 1 or st.stride_l != 0):
             axis = "col"

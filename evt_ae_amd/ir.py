@@ -148,17 +148,24 @@ def accum_coord(L: int, M: int, N: int, batched: bool) -> Coord:
 
 @dataclass
 class Strides:
-    """offset(l, m, n) = (lb // l_div) * stride_l + m * stride_m + n * stride_n,
+    """offset(l, m, n) = (lb // l_div) * stride_l + (lb % l_div) * stride_l2 + m * stride_m + n * stride_n,
     lb = l % l_mod if l_mod else l."""
     stride_l: int
     stride_m: int
     stride_n: int
     l_div: int = 1
     l_mod: int = 0       # > 0: the batch index enters modulo l_mod (batches l and l + l_mod share elements)
+    # batch index in two levels, l = outer * l_div + inner (a [B, S, H, D] tensor against L = B * H batches of
+    # [S, D]): stride of the inner level; 0: the l_div consecutive batches share elements
+    stride_l2: int = 0
 
     def batch_index(self, l):
         lb = l % self.l_mod if self.l_mod else l
         return lb // self.l_div
+
+    def batch_offset(self, l):
+        lb = l % self.l_mod if self.l_mod else l
+        return (lb // self.l_div) * self.stride_l + (lb % self.l_div) * self.stride_l2
 
     @property
     def kind(self) -> str:
@@ -176,8 +183,8 @@ class Strides:
 
 def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Sequence[int]] = None,
                 seed: int = 0) -> Optional[Strides]:
-    """Fit  offset(l, m, n) = (lb // l_div) * sl + m * sm + n * sn,  lb = l % l_mod
-    (or l), to `coord`.
+    """Fit  offset(l, m, n) = (lb // l_div) * sl + (lb % l_div) * sl2 + m * sm + n * sn,
+    lb = l % l_mod (or l), to `coord`.
 
     `elem_strides` are the memory strides of the tensor (default: contiguous).
     Returns None when the mapping is not of that form (checked on the corners,
@@ -208,33 +215,46 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
         return None
     sm = int(offset(z, z + 1, z)[0]) if M > 1 else 0
     sn = int(offset(z, z, z + 1)[0]) if N > 1 else 0
-    # batch: find the smallest l at which the offset changes
-    sl, l_div, l_mod = 0, 1, 0
-    if L > 1:
-        ls = np.arange(L, dtype=np.int64)
-        offs = offset(ls, np.zeros_like(ls), np.zeros_like(ls))
-        nz = np.nonzero(offs)[0]
-        if len(nz):
-            l_div = int(nz[0])
-            sl = int(offs[l_div])
-            # periodic in l: the smallest period that divides L (a full period is no period)
-            for period in range(l_div + 1, L):
-                if L % period == 0 and np.array_equal(offs, offs[ls % period]):
-                    l_mod = period
-                    break
-    st = Strides(sl, sm, sn, l_div, l_mod)
     rng = np.random.default_rng(seed)
     npts = 4096
-    l = rng.integers(0, L, npts)
-    m = rng.integers(0, M, npts)
-    n = rng.integers(0, N, npts)
+    pl = rng.integers(0, L, npts)
+    pm = rng.integers(0, M, npts)
+    pn = rng.integers(0, N, npts)
     # always include the far corner
-    l[0], m[0], n[0] = L - 1, M - 1, N - 1
-    want = offset(l, m, n)
-    got = st.batch_index(l) * sl + m * sm + n * sn
-    if not np.array_equal(want, got):
-        return None
-    return st
+    pl[0], pm[0], pn[0] = L - 1, M - 1, N - 1
+    want = offset(pl, pm, pn)
+
+    def fits(st: Strides) -> bool:
+        return np.array_equal(want, st.batch_offset(pl) + pm * sm + pn * sn)
+
+    if L == 1:
+        st = Strides(0, sm, sn)
+        return st if fits(st) else None
+    ls = np.arange(L, dtype=np.int64)
+    offs = offset(ls, np.zeros_like(ls), np.zeros_like(ls))
+    # one level: l_div consecutive batches share elements, then sl per group; possibly periodic in l
+    sl, l_div, l_mod = 0, 1, 0
+    nz = np.nonzero(offs)[0]
+    if len(nz):
+        l_div = int(nz[0])
+        sl = int(offs[l_div])
+        # periodic in l: the smallest period that divides L (a full period is no period)
+        for period in range(l_div + 1, L):
+            if L % period == 0 and np.array_equal(offs, offs[ls % period]):
+                l_mod = period
+                break
+    st = Strides(sl, sm, sn, l_div, l_mod)
+    if fits(st):
+        return st
+    # two levels: sl2 per batch until, at l = l_div, the offset jumps to sl
+    step = int(offs[1])
+    brk = np.nonzero(offs != ls * step)[0]
+    if len(brk) and step:
+        l_div = int(brk[0])
+        st = Strides(int(offs[l_div]), sm, sn, l_div, 0, step)
+        if L % l_div == 0 and fits(st):
+            return st
+    return None
 
 
 # --------------------------------------------------------------------------

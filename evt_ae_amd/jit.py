@@ -31,7 +31,7 @@ INCLUDE_DIR = PKG_DIR.parent / "include"
 KERNEL_DIR = Path(os.environ.get("EVT_KERNEL_DIR", PKG_DIR / "_kernels"))
 CACHE_FILE = KERNEL_DIR / "compiled_cache.db"
 
-EVT_ABI_VERSION = 2
+EVT_ABI_VERSION = 3
 EVT_MAX_TENSORS = 16
 EVT_MAX_SCALARS = 16
 
@@ -46,13 +46,16 @@ HIPCC_FLAGS = [
 
 class EvtTensorArg(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("stride_l", ctypes.c_int64), ("stride_m", ctypes.c_int64),
-                ("stride_n", ctypes.c_int64), ("l_div", ctypes.c_int64), ("l_mod", ctypes.c_int64)]
+                ("stride_n", ctypes.c_int64), ("l_div", ctypes.c_int64), ("l_mod", ctypes.c_int64),
+                ("stride_l2", ctypes.c_int64)]
 
 
 class EvtArgs(ctypes.Structure):
     _fields_ = [("M", ctypes.c_int32), ("N", ctypes.c_int32), ("K", ctypes.c_int32), ("L", ctypes.c_int32),
                 ("A", ctypes.c_void_p), ("lda", ctypes.c_int64), ("batch_stride_A", ctypes.c_int64),
                 ("B", ctypes.c_void_p), ("ldb", ctypes.c_int64), ("batch_stride_B", ctypes.c_int64),
+                ("batch_div_A", ctypes.c_int64), ("batch_stride2_A", ctypes.c_int64),
+                ("batch_div_B", ctypes.c_int64), ("batch_stride2_B", ctypes.c_int64),
                 ("num_tensors", ctypes.c_int32), ("num_scalars", ctypes.c_int32),
                 ("tensors", EvtTensorArg * EVT_MAX_TENSORS), ("scalars", ctypes.c_float * EVT_MAX_SCALARS)]
 

@@ -20,7 +20,7 @@ from typing import List, Sequence, Set
 import torch
 from torch.fx import Graph, GraphModule, Node
 
-from .evt_fuser import EVTFuser, legalize_graph, packet, target_name
+from .evt_fuser import EVTFuser, legalize_graph, operand_chain, operand_strides, packet, target_name
 from .partitioner import same_phase
 from .frontend_passes import (GTLFrontend, inherit_meta, pass_clean_up, pass_cse,  # noqa: F401  (one namespace,
                               pass_loss_elimination)                                # as gtl.compiler.passes)
@@ -59,10 +59,62 @@ def _mainloop_permutes(anchor: Node, taken: Set[Node]) -> List[Node]:
     the operand's strides (reference: pass_fusion.py:773-781, 1019-1030)."""
     out = []
     for arg in anchor.args[:2]:
+        if packet(anchor.target) == aten.bmm and isinstance(arg, Node):
+            # a whole chain of views / permutes / copies in front of a batched-product operand (the head split
+            # of an attention layer), when it amounts to strided addressing the kernel can read in place
+            chain, _ = operand_chain(arg, lambda n: n not in taken)
+            if chain and any(target_name(n.target) in ("clone", "permute") for n in chain):
+                shape = arg.meta["tensor_meta"].shape if "tensor_meta" in arg.meta else None
+                st = operand_strides(chain, shape) if shape is not None and len(shape) == 3 else None
+                if st is not None and (st.stride_n == 1 or st.stride_m == 1):
+                    out.extend(chain)
+                    continue
         if (isinstance(arg, Node) and arg.op == "call_function" and packet(arg.target) == aten.permute
                 and len(arg.users) == 1 and arg not in taken):
             out.append(arg)
     return out
+
+
+def _private_operand_chains(graph_module: GraphModule) -> None:
+    """The layout chain in front of a batched-product operand can only be read in
+    place when it feeds nothing else.  In a joint graph the split heads of an
+    attention layer feed the forward product and, through a transpose, the
+    backward products: every product whose operand chain amounts to strided
+    addressing gets a private copy of the chain's (layout-only) nodes next to
+    it, tagged with its own phase; what is left without users goes."""
+    graph = graph_module.graph
+    changed = False
+    for anchor in [n for n in graph.nodes if n.op == "call_function" and packet(n.target) == aten.bmm]:
+        for arg in list(anchor.args[:2]):
+            if not isinstance(arg, Node) or "tensor_meta" not in arg.meta:
+                continue
+            chain, src = [], arg
+            while (isinstance(src, Node) and src.op == "call_function"
+                   and target_name(src.target) in ("view", "_unsafe_view", "reshape", "permute", "expand", "clone")):
+                chain.append(src)
+                src = src.args[0]
+            chain.reverse()
+            if not chain or all(len(n.users) == 1 for n in chain):
+                continue
+            if not any(target_name(n.target) == "clone" for n in chain):
+                continue
+            shape = tuple(arg.meta["tensor_meta"].shape)
+            st = operand_strides(chain, shape) if len(shape) == 3 else None
+            if st is None or not (st.stride_n == 1 or st.stride_m == 1):
+                continue
+            tags = {k: anchor.meta[k] for k in ("partitioner_tag", "seq_nr", "autograd_backward") if k in anchor.meta}
+            x = src
+            with graph.inserting_before(anchor):
+                for n in chain:
+                    y = graph.call_function(n.target, (x, *n.args[1:]), dict(n.kwargs))
+                    y.meta = {k: v for k, v in n.meta.items() if k in ("tensor_meta", "val")}
+                    y.meta.update(tags)
+                    x = y
+            anchor.replace_input_with(arg, x)
+            changed = True
+    if changed:
+        graph.eliminate_dead_code()
+        graph_module.recompile()
 
 
 def _absorb_side_expressions(anchor: Node, inside: Set[Node], desc: Set[Node], taken: Set[Node]) -> None:
@@ -161,6 +213,7 @@ class Partitioning:
 
     def call(self, graph_module: GraphModule) -> None:
         graph = graph_module.graph
+        _private_operand_chains(graph_module)
         anchors = [n for n in graph.nodes
                    if n.op == "call_function" and packet(n.target) in EVTFuser.supported_targets]
         planned = self.plan_ilp(graph_module, anchors) if self.strategy == "ilp" \

@@ -84,6 +84,7 @@ def register_all() -> List[jit.LazyModule]:
     aot_capture(*W.mlp_classifier(device="meta"))
     aot_capture(*W.mlp_classifier())
     aot_capture(*W.encoder_layer(device="meta"))
+    aot_capture(*W.encoder_layer(device="meta", fused_qkv=False))
     aot_capture(*W.dropout_block(device="meta"))
     aot_capture(*W.decoder_block(device="meta"))
     aot_capture(*W.decoder_block(device="meta", dtype=torch.bfloat16))

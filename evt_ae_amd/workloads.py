@@ -1104,14 +1104,21 @@ def decoder_block(seed: int = 0, device: str = "cpu", dtype=torch.float16, batch
 
 
 class EncoderLayer(torch.nn.Module):
-    """fp16 post-LN transformer encoder layer with a squared-error loss: QKV
-    projection, batched QK^T and PV products, softmax, output projection,
-    two layer norms and the GELU feed-forward block (the shape of the
-    reference's BERT test, unittest/fx_passes/bert.py, at a small size)."""
-    def __init__(self, d: int = 256, heads: int = 4, ffn: int = 1024) -> None:
+    """fp16 post-LN transformer encoder layer with a squared-error loss: Q, K, V
+    projections (three Linear layers as in the reference's BERT, or one fused
+    [d, 3d] projection), batched QK^T and PV products, softmax, output
+    projection, two layer norms and the GELU feed-forward block (the shape of
+    the reference's BERT test, unittest/fx_passes/bert.py, at a small size)."""
+    def __init__(self, d: int = 256, heads: int = 4, ffn: int = 1024, fused_qkv: bool = True) -> None:
         super().__init__()
         self.heads = heads
-        self.qkv = torch.nn.Linear(d, 3 * d)
+        self.fused_qkv = fused_qkv
+        if fused_qkv:
+            self.qkv = torch.nn.Linear(d, 3 * d)
+        else:
+            self.q = torch.nn.Linear(d, d)
+            self.k = torch.nn.Linear(d, d)
+            self.v = torch.nn.Linear(d, d)
         self.out = torch.nn.Linear(d, d)
         self.ln1 = torch.nn.LayerNorm(d)
         self.ln2 = torch.nn.LayerNorm(d)
@@ -1122,8 +1129,12 @@ class EncoderLayer(torch.nn.Module):
         B, S, D = x.shape
         H = self.heads
         dh = D // H
-        qkv = self.qkv(x).view(B, S, 3, H, dh).permute(2, 0, 3, 1, 4)
-        q, k, v = qkv[0], qkv[1], qkv[2]
+        if self.fused_qkv:
+            qkv = self.qkv(x).view(B, S, 3, H, dh).permute(2, 0, 3, 1, 4)
+            q, k, v = qkv[0], qkv[1], qkv[2]
+        else:
+            split = lambda t: t.view(B, S, H, dh).permute(0, 2, 1, 3)      # noqa: E731
+            q, k, v = split(self.q(x)), split(self.k(x)), split(self.v(x))
         att = torch.softmax((q @ k.transpose(-1, -2)) / (dh ** 0.5), -1)
         ctx = (att @ v).permute(0, 2, 1, 3).reshape(B, S, D)
         x = self.ln1(x + self.out(ctx))
@@ -1131,14 +1142,15 @@ class EncoderLayer(torch.nn.Module):
         return ((x.float() - target) ** 2).sum()
 
 
-ENCODER_BENCH = dict(d=1024, heads=16, ffn=4096, batch=8, seq=512)     # a BERT-large layer
+# a BERT-large layer, with separate Q / K / V projections as in the reference's BERT
+ENCODER_BENCH = dict(d=1024, heads=16, ffn=4096, batch=8, seq=512, fused_qkv=False)
 
 
 def encoder_layer(seed: int = 0, device: str = "cpu", dtype=torch.float16, d: int = 256, heads: int = 4,
-                  ffn: int = 1024, batch: int = 8, seq: int = 128):
+                  ffn: int = 1024, batch: int = 8, seq: int = 128, fused_qkv: bool = True):
     """(model, (x, target)) with seeded parameters and inputs (default: batch 8, sequence 128, width 256)."""
     g = torch.Generator(device="cpu").manual_seed(0xE9C + seed)
-    model = EncoderLayer(d, heads, ffn)
+    model = EncoderLayer(d, heads, ffn, fused_qkv)
     with torch.no_grad():
         for name, p in model.named_parameters():
             if p.dim() == 2:

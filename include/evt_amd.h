@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define EVT_ABI_VERSION 2
+#define EVT_ABI_VERSION 3
 #define EVT_MAX_TENSORS 16
 #define EVT_MAX_SCALARS 16
 
@@ -42,11 +42,15 @@ extern "C" {
 
 /* One epilogue tensor (load or store).  Element (l, m, n) of the logical
  * [L, M, N] iteration space lives at
- *     ptr + (lb / l_div) * stride_l + m * stride_m + n * stride_n   (elements),
+ *     ptr + (lb / l_div) * stride_l + (lb % l_div) * stride_l2
+ *         + m * stride_m + n * stride_n                              (elements),
  *     lb = l_mod > 0 ? l % l_mod : l.
- * A broadcast dimension has stride 0.  l_div > 1: l_div consecutive batches
- * share elements (a [B, ...] tensor against L = B*H batches); l_mod > 0: batches
- * that agree modulo l_mod do (an [H, ...] tensor against the same L).  For the
+ * A broadcast dimension has stride 0.  l_div > 1 with stride_l2 = 0: l_div
+ * consecutive batches share elements (a [B, ...] tensor against L = B*H
+ * batches); with stride_l2 != 0 the batch index has two levels (a [B, S, H, D]
+ * tensor read or written as L = B*H batches of [S, D]: the head split of an
+ * attention layer without a copy); l_mod > 0: batches
+ * that agree modulo l_mod share elements (an [H, ...] tensor against the same L).  For the
  * output of a per-row reduction, batches that share elements are summed into
  * them (the reduction then runs over N and over those batches).  Replaces the (M, N, L)-strided
  * tensor arguments of VisitorAuxLoad / VisitorRowBroadcast / VisitorRowStore
@@ -65,6 +69,7 @@ typedef struct EvtTensorArg {
   int64_t stride_n;
   int64_t l_div;
   int64_t l_mod;
+  int64_t stride_l2;
 } EvtTensorArg;
 
 /* Launch arguments.  A is [L, M, K], B is [L, K, N]; which of the two
@@ -99,6 +104,15 @@ typedef struct EvtArgs {
   const void* B;
   int64_t ldb;
   int64_t batch_stride_B;
+  /* two-level batch index of an operand: batch l starts at
+   *   (l / batch_div_X) * batch_stride_X + (l % batch_div_X) * batch_stride2_X
+   * elements (batch_div_X = 0 or 1: one level, batch_stride2_X ignored).  Lets a [B, S, H, D] tensor serve as
+   * L = B*H batches of [S, D] with row stride H*D (reference: the permuted
+   * BMM operands of BmmArguments2x, python/gtl/ops/bmm.py:23-64). */
+  int64_t batch_div_A;
+  int64_t batch_stride2_A;
+  int64_t batch_div_B;
+  int64_t batch_stride2_B;
   int32_t num_tensors;
   int32_t num_scalars;
   EvtTensorArg tensors[EVT_MAX_TENSORS];

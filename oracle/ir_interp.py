@@ -67,7 +67,7 @@ def _gather_strided(t: torch.Tensor, st, L, M, N) -> torch.Tensor:
     l = torch.arange(L).view(L, 1, 1)
     m = torch.arange(M).view(1, M, 1)
     n = torch.arange(N).view(1, 1, N)
-    off = st.batch_index(l) * st.stride_l + m * st.stride_m + n * st.stride_n
+    off = st.batch_offset(l) + m * st.stride_m + n * st.stride_n
     return flat[off.reshape(-1)].reshape(L, M, N).to(torch.float32)
 
 
@@ -124,7 +124,7 @@ def interpret(ir, accum: torch.Tensor, slot_tensors: Dict[int, torch.Tensor]) ->
         slot = ir.slots[s.slot]
         st = slot.strides
         v = val[s.input].expand(L, M, N)
-        off = (st.batch_index(l) * st.stride_l + m * st.stride_m + n * st.stride_n).expand(L, M, N)
+        off = (st.batch_offset(l) + m * st.stride_m + n * st.stride_n).expand(L, M, N)
         size = int(off.max()) + 1
         buf = torch.zeros(size, dtype=torch.float32)
         buf[off.reshape(-1)] = v.reshape(-1)

@@ -43,10 +43,10 @@ def test_every_built_module_exports_the_abi():
         for sym in declared_symbols():
             assert hasattr(lib, sym), f"{p.name} lacks {sym}"
         lib.evt_abi_version.restype = ctypes.c_int
-        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 2
+        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 3
         lib.evt_module_spec.restype = ctypes.c_char_p
         spec = json.loads(lib.evt_module_spec().decode())
-        assert spec["abi"] == 2
+        assert spec["abi"] == 3
         if "anchor" in spec:      # row-wise reduce-apply module
             assert spec["anchor"] in ("softmax", "softmax_backward", "layernorm", "layernorm_backward")
             assert spec["element"] in ("f16", "bf16", "f32") and spec["row"]["max_n"] >= 1
@@ -54,11 +54,28 @@ def test_every_built_module_exports_the_abi():
             assert spec["element"] in ("f16", "bf16") and "tile" in spec
 
 
-def test_struct_layout_matches_header():
-    # EvtTensorArg: pointer + 5 x int64 ; EvtArgs: 4 x int32, 2 x (ptr, int64, int64), 2 x int32, arrays
-    assert ctypes.sizeof(jit.EvtTensorArg) == 48
-    assert ctypes.sizeof(jit.EvtArgs) == 16 + 48 + 8 + 16 * 48 + 16 * 4
-    assert jit.EvtArgs.tensors.offset == 72 and jit.EvtArgs.scalars.offset == 72 + 768
+def test_struct_layout_matches_header(tmp_path):
+    """The ctypes mirrors against the header itself: a C program compiled with gcc
+    prints sizeof / offsetof of every field of include/evt_amd.h."""
+    import subprocess
+    fields_t = [f[0] for f in jit.EvtTensorArg._fields_]
+    fields_a = [f[0] for f in jit.EvtArgs._fields_]
+    src = ['#include <stdio.h>', '#include <stddef.h>', '#include "evt_amd.h"', 'int main(void) {',
+           '  printf("%zu %zu\\n", sizeof(EvtTensorArg), sizeof(EvtArgs));']
+    src += [f'  printf("%zu\\n", offsetof(EvtTensorArg, {f}));' for f in fields_t]
+    src += [f'  printf("%zu\\n", offsetof(EvtArgs, {f}));' for f in fields_a]
+    src += ['  printf("%d %d %d\\n", EVT_ABI_VERSION, EVT_MAX_TENSORS, EVT_MAX_SCALARS);', '  return 0; }']
+    c = tmp_path / "layout.c"
+    c.write_text("\n".join(src))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", str(jit.INCLUDE_DIR), str(c), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    nums = [int(x) for x in out]
+    assert nums[0] == ctypes.sizeof(jit.EvtTensorArg) == 56       # pointer + 6 x int64
+    assert nums[1] == ctypes.sizeof(jit.EvtArgs)
+    want = [getattr(jit.EvtTensorArg, f).offset for f in fields_t] + [getattr(jit.EvtArgs, f).offset for f in fields_a]
+    assert nums[2:2 + len(want)] == want
+    assert nums[-3:] == [jit.EVT_ABI_VERSION, jit.EVT_MAX_TENSORS, jit.EVT_MAX_SCALARS]
 
 
 def test_module_spec_describes_slots(module):

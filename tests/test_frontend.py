@@ -272,7 +272,7 @@ def test_row_anchor_patterns_trace(name):
     assert K == 1 and N == inputs[0].shape[-1] and L * M * N == inputs[0].numel()
     assert op.row_spec.max_n >= N and op.row_spec.lpr in (8, 16, 32, 64) and 1 <= op.row_spec.ch <= 16
     spec = op.module.spec
-    assert spec["abi"] == 2 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
+    assert spec["abi"] == 3 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
     assert op.num_anchor_inputs == {"softmax": 1, "softmax_backward": 2, "layernorm": 1, "layernorm_backward": 5}[kind]
     if kind == "layernorm":
         # eps travels as a scalar; mean and rstd are per-row stores

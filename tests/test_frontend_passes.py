@@ -254,6 +254,36 @@ def test_encoder_layer_joint_graph():
     assert [n.name for n in box["fw"].graph.nodes if n.op == "placeholder"][-1].startswith("primals_")
 
 
+def test_head_split_and_merge_are_read_and_written_in_place():
+    """Separate Q / K / V projections (the reference's BERT): the chains
+    view -> permute -> expand -> clone -> view in front of the batched products,
+    shared between the forward product and the backward ones, are given to each
+    product privately and folded into its operand strides (batch index in two
+    levels), and the merge behind the products into the stores: no clone is
+    left in either graph and the products' arguments are the projections' own
+    outputs."""
+    from evt_ae_amd.evt_fuser import FusedBMM
+    model, inputs = W.encoder_layer(device="meta", fused_qkv=False)
+    box = aot_capture(model, inputs)
+    for g in (box["fw"], box["bw"]):
+        names = [target_name(n.target) for n in g.graph.nodes if n.op == "call_function"]
+        assert "clone" not in names and "bmm" not in names, names
+    ops = [n.target for g in (box["fw"], box["bw"]) for n in fused_nodes(g) if isinstance(n.target, FusedBMM)]
+    assert len(ops) == 6
+    B, S, H, dh = 8, 128, 4, 64
+    two_level = 0
+    for op in ops:
+        for div, s1, s2 in ((op.bdiva, op.bsa, op.bs2a), (op.bdivb, op.bsb, op.bs2b)):
+            if div > 1:
+                two_level += 1
+                assert (div, s1, s2) == (H, S * H * dh, dh)
+    assert two_level >= 8          # q, k, v and their gradients' partners: operands read straight from [B, S, H * dh]
+    # the merged result is stored straight into [B, S, H * dh]
+    pv = next(op for op in ops if op.problem == (S, dh, S, B * H) and any(s.strides.stride_l2 for s in op.ir.slots))
+    (st,) = [s.strides for s in pv.ir.slots if s.role == "store"]
+    assert (st.l_div, st.stride_l, st.stride_l2, st.stride_m, st.stride_n) == (H, S * H * dh, dh, H * dh, 1)
+
+
 def test_dropout_in_a_training_step_is_fused_and_leaves_nothing_behind():
     """native_dropout becomes rand_like / ge / mul inside the GEMM epilogues; the
     masks are kernel outputs saved for backward.  fx keeps random ops alive as

@@ -489,20 +489,27 @@ def test_layer_norm_with_weight_and_bias_on_long_rows(n):
         assert err <= (REDUCTION_TOL if k > 0 else FP16_TOL), f"n={n} output {k}: max rel err {err:.3e}"
 
 
-def test_aot_encoder_layer_training_step():
+@pytest.mark.parametrize("fused_qkv", [True, False], ids=["fused_qkv", "separate_qkv"])
+def test_aot_encoder_layer_training_step(fused_qkv):
     """A transformer encoder layer, forward and backward, through AOT autograd
     with the joint pipeline (the reference's BERT flow, unittest/fx_passes/bert.py:
     frontend, decomposition, CSE, fusion, default_partition): projections with
     bias / residual / GELU epilogues, batched QK^T and PV products with their
     permutes and the 1/sqrt(d) scale, softmax and softmax backward, both layer
-    norms with weight and bias, all as fused launches.  Loss and gradients
-    against the same model in fp32."""
+    norms with weight and bias, all as fused launches.  With separate Q / K / V
+    projections (the reference's BERT) the head split and merge
+    (view -> permute -> clone -> view around the batched products, forward and
+    backward) are read and written in place through two-level batch strides: no
+    copy kernel is left.  Loss and gradients against the same model in fp32."""
     import copy
     from evt_ae_amd.aot_helper import aot_capture, aot_optimize
-    model, (x, target) = W.encoder_layer(device="cuda")
+    model, (x, target) = W.encoder_layer(device="cuda", fused_qkv=fused_qkv)
     box = aot_capture(copy.deepcopy(model), (x, target))
     kinds = [type(n.target).__name__ for n in fused_nodes(box["fw"])] + [type(n.target).__name__ for n in fused_nodes(box["bw"])]
-    assert kinds.count("FusedGEMM") == 11 and kinds.count("FusedBMM") == 6
+    assert kinds.count("FusedGEMM") == (11 if fused_qkv else 15) and kinds.count("FusedBMM") == 6
+    if not fused_qkv:
+        left = [target_name(n.target) for g in (box["fw"], box["bw"]) for n in g.graph.nodes if n.op == "call_function"]
+        assert "clone" not in left and "bmm" not in left, left
     assert kinds.count("FusedSoftmax") == 1 and kinds.count("FusedSoftmaxBackward") == 1
     assert kinds.count("FusedLayerNorm") == 2 and kinds.count("FusedLayerNormBackward") == 2
     master = copy.deepcopy(model).float()
