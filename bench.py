@@ -287,7 +287,11 @@ def bench_encoder_step(torch, W, iters=20):
     f_loop, f_graph = run(fused, list(model.parameters()))
     ref = [p.grad.float() for p in eager.parameters()]
     got = [p.grad.float() for p in model.parameters()]
-    err = max(float((a - b).norm() / b.norm().clamp_min(1e-30)) for a, b in zip(got, ref))
+    # norm-wise per parameter.  The key projection's bias has no influence on a softmax over keys: its exact
+    # gradient is zero and both runs return rounding noise, so a gradient far below the others' scale is measured
+    # against that scale (1e-3 of the largest per-element RMS) instead of against its own norm
+    rms = max(float(b.norm()) / b.numel() ** 0.5 for b in ref)
+    err = max(float((a - b).norm()) / max(float(b.norm()), 1e-3 * rms * b.numel() ** 0.5, 1e-30) for a, b in zip(got, ref))
     best_e = min(t for t in (e_loop, e_graph) if t)
     best_f = min(t for t in (f_loop, f_graph) if t)
     out = {"model": "post-LN encoder layer", **W.ENCODER_BENCH, "dtype": "f16",
