@@ -368,7 +368,7 @@ class FusedOpBase:
 
 # layout-only ops between a tensor in memory and a batched-product operand (the head split of an attention layer:
 # view [B, S, H, D] -> permute [0, 2, 1, 3] -> expand -> clone -> view [B * H, S, D])
-_OPERAND_CHAIN_OPS = ("view", "_unsafe_view", "reshape", "permute", "expand", "clone", "unsqueeze", "squeeze")
+_OPERAND_CHAIN_OPS = ("view", "_unsafe_view", "reshape", "permute", "expand", "clone", "unsqueeze", "squeeze", "select")
 
 
 def operand_chain(node, allowed=None) -> Tuple[List[Node], Any]:
@@ -394,6 +394,8 @@ def operand_strides(chain: Sequence[Node], shape3: Sequence[int]) -> Optional[St
         in_shape, _ = node_shape_dtype(node.args[0])
         if target_name(node.target) == "permute":
             coord = coord.inverse_permute([int(d) for d in node.args[1]], in_shape)
+        elif target_name(node.target) == "select":
+            coord = coord.inverse_select(int(node.args[1]), int(node.args[2]), in_shape)
         else:
             numel = 1
             for d in in_shape:
@@ -401,7 +403,7 @@ def operand_strides(chain: Sequence[Node], shape3: Sequence[int]) -> Optional[St
             if numel != coord.numel():        # an expand that broadcasts
                 return None
             coord = coord.reshape(in_shape)
-    st = fit_strides(coord, L, R, C)
+    st = fit_strides(coord, L, R, C, allow_base=True)
     if st is None or st.l_mod:
         return None
     return st
@@ -524,12 +526,12 @@ class FusedBMM(FusedOpBase):
             self.b_kc, self.ldb = False, (sb.stride_m if K > 1 else N)
         else:
             self.copy_B, self.b_kc, self.ldb, sb = True, False, N, Strides(K * N, N, 1)
-        self.bsa, self.bdiva, self.bs2a = sa.stride_l, sa.l_div, sa.stride_l2
-        self.bsb, self.bdivb, self.bs2b = sb.stride_l, sb.l_div, sb.stride_l2
+        self.bsa, self.bdiva, self.bs2a, self.offa = sa.stride_l, sa.l_div, sa.stride_l2, sa.base
+        self.bsb, self.bdivb, self.bs2b, self.offb = sb.stride_l, sb.l_div, sb.stride_l2, sb.base
         self.lhs_layout = "RowMajor" if self.a_kc else "ColumnMajor"
         self.rhs_layout = "ColumnMajor" if self.b_kc else "RowMajor"
         dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb,
-                      self.bsa | self.bs2a, self.bsb | self.bs2b)
+                      self.bsa | self.bs2a | self.offa, self.bsb | self.bs2b | self.offb)
 
         with (_pop_mode_temporarily() if _len_torch_dispatch_stack() > 0 else nullcontext()):
             tuner = BMMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
@@ -571,6 +573,10 @@ class FusedBMM(FusedOpBase):
         a, keep = super().build_arguments(visitor_args, *args, block=block)
         a.batch_div_A, a.batch_stride2_A = self.bdiva, self.bs2a
         a.batch_div_B, a.batch_stride2_B = self.bdivb, self.bs2b
+        if self.offa:       # the operand starts inside its source tensor (a `select`): elements of 2 bytes
+            a.A = a.A + 2 * self.offa
+        if self.offb:
+            a.B = a.B + 2 * self.offb
         return a, keep
 
     def anchor_eager(self, A, B):

@@ -113,6 +113,22 @@ class Coord:
 
         return Coord(src_shape, fn)
 
+    def inverse_select(self, dim: int, index: int, src_shape: Sequence[int]) -> "Coord":
+        """`self` indexes select(src, dim, index); return the index into src."""
+        src_shape = tuple(int(s) for s in src_shape)
+        dim = dim % len(src_shape)
+        index = index % src_shape[dim]
+        my_shape = self.shape
+        my_fn = self.fn
+
+        def fn(l, m, n):
+            flat = my_fn(l, m, n)
+            idx = list(np.unravel_index(flat, my_shape)) if my_shape else []
+            idx.insert(dim, np.full_like(flat, index))
+            return np.ravel_multi_index(tuple(idx), src_shape)
+
+        return Coord(src_shape, fn)
+
     def reduce(self, dims: Sequence[int], keepdim: bool) -> "Coord":
         """Index of the reduction result element that (l, m, n) contributes to."""
         shape = self.shape
@@ -158,6 +174,8 @@ class Strides:
     # batch index in two levels, l = outer * l_div + inner (a [B, S, H, D] tensor against L = B * H batches of
     # [S, D]): stride of the inner level; 0: the l_div consecutive batches share elements
     stride_l2: int = 0
+    # operands only: elements in front of element (0, 0, 0) (a `select` of a larger tensor)
+    base: int = 0
 
     def batch_index(self, l):
         lb = l % self.l_mod if self.l_mod else l
@@ -182,7 +200,7 @@ class Strides:
 
 
 def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Sequence[int]] = None,
-                seed: int = 0) -> Optional[Strides]:
+                seed: int = 0, allow_base: bool = False) -> Optional[Strides]:
     """Fit  offset(l, m, n) = (lb // l_div) * sl + (lb % l_div) * sl2 + m * sm + n * sn,
     lb = l % l_mod (or l), to `coord`.
 
@@ -198,7 +216,7 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
             acc *= s
         elem_strides = tuple(reversed(elem_strides))
 
-    def offset(l, m, n):
+    def raw_offset(l, m, n):
         flat = coord.fn(np.asarray(l, dtype=np.int64), np.asarray(m, dtype=np.int64),
                         np.asarray(n, dtype=np.int64))
         if not shape:
@@ -210,9 +228,12 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
         return off
 
     z = np.zeros(1, dtype=np.int64)
-    base = int(offset(z, z, z)[0])
-    if base != 0:
+    base = int(raw_offset(z, z, z)[0])
+    if base != 0 and not allow_base:
         return None
+
+    def offset(l, m, n):
+        return raw_offset(l, m, n) - base
     sm = int(offset(z, z + 1, z)[0]) if M > 1 else 0
     sn = int(offset(z, z, z + 1)[0]) if N > 1 else 0
     rng = np.random.default_rng(seed)
@@ -228,7 +249,7 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
         return np.array_equal(want, st.batch_offset(pl) + pm * sm + pn * sn)
 
     if L == 1:
-        st = Strides(0, sm, sn)
+        st = Strides(0, sm, sn, base=base)
         return st if fits(st) else None
     ls = np.arange(L, dtype=np.int64)
     offs = offset(ls, np.zeros_like(ls), np.zeros_like(ls))
@@ -243,7 +264,7 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
             if L % period == 0 and np.array_equal(offs, offs[ls % period]):
                 l_mod = period
                 break
-    st = Strides(sl, sm, sn, l_div, l_mod)
+    st = Strides(sl, sm, sn, l_div, l_mod, base=base)
     if fits(st):
         return st
     # two levels: sl2 per batch until, at l = l_div, the offset jumps to sl
@@ -251,7 +272,7 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
     brk = np.nonzero(offs != ls * step)[0]
     if len(brk) and step:
         l_div = int(brk[0])
-        st = Strides(int(offs[l_div]), sm, sn, l_div, 0, step)
+        st = Strides(int(offs[l_div]), sm, sn, l_div, 0, step, base)
         if L % l_div == 0 and fits(st):
             return st
     return None

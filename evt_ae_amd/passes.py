@@ -90,7 +90,7 @@ def _private_operand_chains(graph_module: GraphModule) -> None:
                 continue
             chain, src = [], arg
             while (isinstance(src, Node) and src.op == "call_function"
-                   and target_name(src.target) in ("view", "_unsafe_view", "reshape", "permute", "expand", "clone")):
+                   and target_name(src.target) in ("view", "_unsafe_view", "reshape", "permute", "expand", "clone", "select")):
                 chain.append(src)
                 src = src.args[0]
             chain.reverse()
@@ -375,6 +375,7 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                                             unsqueeze(ne(target, ignore_index), 1)) [/ batch]   (:294-348;
                                         the reference compares with -1 instead of ignore_index)
       masked_fill(x, mask, v)        -> where(mask, v, x)                        (scalar v; not in the reference)
+      getitem(unbind(x, d), i)       -> select(x, d, i)                          (not in the reference)
       native_layer_norm(x, s, w, b, eps)
                                      -> add(mul(native_layer_norm(x, s, None, None, eps)[0], w), b)   (:504-544)
     and permute(permute(x)) folded into one permute or none.  The reference's
@@ -463,6 +464,20 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                 if not node.users:
                     graph.erase_node(node)
                     changed = True
+                continue
+            elif name == "unbind" and all(u.op == "call_function" and u.target is operator.getitem for u in node.users):
+                # getitem(unbind(x, d), i) is select(x, d, i): a layout op the batched products read through
+                x = node.args[0]
+                dim = int(node.args[1]) if len(node.args) > 1 else int(node.kwargs.get("dim", 0))
+                for user in list(node.users):
+                    sel = inherit_meta(graph.call_function(aten.select, (x, dim, int(user.args[1]))), user)
+                    for k in ("tensor_meta", "val"):
+                        if k in user.meta:
+                            sel.meta[k] = user.meta[k]
+                    user.replace_all_uses_with(sel)
+                    graph.erase_node(user)
+                graph.erase_node(node)
+                changed = True
                 continue
             elif name == "native_dropout" and len(node.args) == 3 and node.args[2] is True:
                 x, p = node.args[0], node.args[1]

@@ -284,6 +284,23 @@ def test_head_split_and_merge_are_read_and_written_in_place():
     assert (st.l_div, st.stride_l, st.stride_l2, st.stride_m, st.stride_n) == (H, S * H * dh, dh, H * dh, 1)
 
 
+def test_fused_qkv_forward_reads_its_heads_in_place():
+    """One [d, 3d] projection: q, k and v are `select`s (or an `unbind`) of a
+    permuted view of its output; each batched product reads its operand inside
+    that output through a base offset and two-level batch strides, so the
+    forward graph holds no select, expand or clone."""
+    from evt_ae_amd.evt_fuser import FusedBMM
+    for model, inputs in (W.encoder_layer(device="meta"), W.decoder_block(device="meta")):
+        box = aot_capture(model, inputs)
+        names = [target_name(n.target) for n in box["fw"].graph.nodes if n.op == "call_function"]
+        assert not {"clone", "select", "unbind", "expand", "bmm"} & set(names), names
+        ops = [n.target for n in fused_nodes(box["fw"]) if isinstance(n.target, FusedBMM)]
+        assert len(ops) == 2
+        d = 256
+        assert sorted((ops[0].offa, ops[0].offb)) == [0, d] and ops[1].offb == 2 * d       # q, k ; v
+        assert ops[0].bdiva == ops[0].bdivb == ops[1].bdivb == 4 and ops[0].lda == ops[0].ldb == 3 * d
+
+
 def test_dropout_in_a_training_step_is_fused_and_leaves_nothing_behind():
     """native_dropout becomes rand_like / ge / mul inside the GEMM epilogues; the
     masks are kernel outputs saved for backward.  fx keeps random ops alive as
