@@ -88,6 +88,8 @@ def _private_operand_chains(graph_module: GraphModule) -> None:
         for arg in list(anchor.args[:2]):
             if not isinstance(arg, Node) or "tensor_meta" not in arg.meta:
                 continue
+            if arg.meta["tensor_meta"].dtype not in (torch.float16, torch.bfloat16):
+                continue        # not a product the fuser takes: a private chain would only add copies
             chain, src = [], arg
             while (isinstance(src, Node) and src.op == "call_function"
                    and target_name(src.target) in ("view", "_unsafe_view", "reshape", "permute", "expand", "clone", "select")):
