@@ -4,7 +4,8 @@ ships next to its benchmarks, e.g. benchmark/bert/tuner_cache.db).
 
     python -m evt_ae_amd.autotuner.tune_workloads --build-only   # compile every candidate (no GPU needed)
     python -m evt_ae_amd.autotuner.tune_workloads [--cache FILE]  # time them on the GPU, store the best
-    ... --encoder [--short-list]   # also the GEMMs / batched products of the BERT-large encoder layer step
+    ... --encoder [--short-list] [--dims d,heads,ffn,batch,seq]   # the GEMMs / batched products of an encoder
+                                                                  # layer's training step (default: BERT-large)
 """
 from __future__ import annotations
 
@@ -31,15 +32,18 @@ def _tuners():
     return out
 
 
-def _encoder_tuners():
+def _encoder_tuners(dims=None):
     """One tuner per distinct fused GEMM / BMM of the encoder layer's training
-    step at the benchmark's size (traced on the meta device: the GPU's dtypes)."""
+    step at the benchmark's size, or at `dims` = (d, heads, ffn, batch, seq)
+    with separate Q / K / V projections (traced on the meta device: the GPU's
+    dtypes)."""
     from .. import workloads as W
     from ..aot_helper import aot_capture
     from ..autotuner.bmm_tuner import BMMTuner
     from ..autotuner.gemm_tuner import MMTuner
     from ..evt_fuser import FusedBMM, FusedGEMM
-    box = aot_capture(*W.encoder_layer(device="meta", **W.ENCODER_BENCH))
+    kw = W.ENCODER_BENCH if dims is None else dict(zip(("d", "heads", "ffn", "batch", "seq"), dims), fused_qkv=False)
+    box = aot_capture(*W.encoder_layer(device="meta", **kw))
     out, seen = [], set()
     for node in W.fused_nodes(box["joint"]):
         op = node.target
@@ -63,13 +67,15 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--build-only", action="store_true")
     ap.add_argument("--encoder", action="store_true", help="tune the encoder layer's problems instead of the five configs")
+    ap.add_argument("--dims", default=None, help="with --encoder: d,heads,ffn,batch,seq of the layer (default: the benchmark's)")
     ap.add_argument("--short-list", action="store_true", help="only the tiles of SHORT_LIST")
     ap.add_argument("--cache", default=None, help="tuner cache file to write (default: the package's)")
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     args = ap.parse_args()
     # candidates must be enumerated without consulting an existing cache
     os.environ["EVT_TUNER_CACHE"] = "/nonexistent/tuner_cache.db"
-    tuners = _encoder_tuners() if args.encoder else _tuners()
+    dims = tuple(int(x) for x in args.dims.split(",")) if args.dims else None
+    tuners = _encoder_tuners(dims) if args.encoder else _tuners()
     if args.short_list:
         for _, t in tuners:
             full = t.candidates()
