@@ -668,7 +668,7 @@ class Codegen:
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
         e("  const int64_t need = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
-        e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
+        e("  if (need > 0 && (!ws || ws_bytes < need || ((uintptr_t)ws & 15))) return EVT_ERR_WORKSPACE;   // 16-byte aligned")
         e("  g.workspace = (char*)ws;")
         e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L * g.splits);")
         e("  hipLaunchKernelGGL((evt::evt_gemm_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")

@@ -138,7 +138,7 @@ const char* evt_module_spec(void);
  * output tile (few tiles, long K) also one fp32 accumulator tile per split and
  * one counter per tile.  The counters must be zero before the first launch
  * (evt_workspace_init) and every launch leaves them zero; launches that share
- * a workspace must not overlap in time.  Takes the place of the host-side
+ * a workspace must not overlap in time.  The workspace is 16-byte aligned.  Takes the place of the host-side
  * pre-zeroing of reduction outputs (evt_fuser.py:217-225). */
 int64_t evt_workspace_bytes(const EvtArgs* args);
 
