@@ -262,15 +262,11 @@ class FusedOpBase:
         return "accum" if output is self.node else output.name
 
     def __call__(self, *args_):
-        if not torch.cuda.is_available():
+        if not _hip_device_present():
             raise RuntimeError("the fused EVT kernels run on a HIP device only; none is available")
-        args = []
-        for arg in args_:
-            if isinstance(arg, torch.Tensor):
-                args.append(arg.contiguous())
-            else:
-                args.append(arg)
-
+        # every microsecond here is paid per launch: no copies of what is contiguous already, no stream context
+        # unless the op has a stream of its own, the result plan (store, views / permutes) worked out once
+        args = [a if (not isinstance(a, torch.Tensor) or a.is_contiguous()) else a.contiguous() for a in args_]
         default_stream = torch.cuda.current_stream()
         if self.stream is not None:
             self.stream.wait_stream(default_stream)
@@ -278,13 +274,8 @@ class FusedOpBase:
         else:
             stream = default_stream
 
-        # entering a stream context costs microseconds of host time per call: only when the op has a stream of its own
         with (torch.cuda.stream(stream) if self.stream is not None else nullcontext()):
-            device = args[-1].device
-            visitor_args = self.allocate_outputs(device)
-            for idx, input_name in enumerate(self.input_names):
-                visitor_args.setdefault(input_name, args[idx])
-
+            visitor_args = self.allocate_outputs(args[-1].device)
             self.call(visitor_args, stream, *args)
 
             if self.stream is not None:
@@ -292,11 +283,15 @@ class FusedOpBase:
                     if isinstance(arg, torch.Tensor):
                         arg.record_stream(self.stream)
 
+            plan = getattr(self, "_result_plan", None)
+            if plan is None:
+                plan = self._result_plan = [
+                    (self.output2store[self.get_output_name(o)], tuple(self.post_reshape_permute.get(self.get_output_name(o), ())))
+                    for o in self.outputs]
             results = []
-            for output in self.outputs:
-                name = self.get_output_name(output)
-                out = visitor_args[self.output2store[name]]
-                for op, arg in self.post_reshape_permute.get(name, ()):
+            for store, ops in plan:
+                out = visitor_args[store]
+                for op, arg in ops:
                     out = out.view(arg) if op == "view" else out.permute(arg)
                 results.append(out)
 
@@ -407,6 +402,17 @@ def operand_strides(chain: Sequence[Node], shape3: Sequence[int]) -> Optional[St
     if st is None or st.l_mod:
         return None
     return st
+
+
+_HIP_PRESENT: Optional[bool] = None
+
+
+def _hip_device_present() -> bool:
+    """torch.cuda.is_available(), asked once (a fused op runs thousands of times per second)."""
+    global _HIP_PRESENT
+    if _HIP_PRESENT is None:
+        _HIP_PRESENT = bool(torch.cuda.is_available())
+    return _HIP_PRESENT
 
 
 def _dma_ok(a_kc: bool, b_kc: bool, M: int, N: int, K: int, lda: int, ldb: int, bsa: int, bsb: int) -> bool:
