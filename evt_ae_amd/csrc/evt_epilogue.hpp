@@ -370,7 +370,7 @@ template <int ROW_STATE, int COL_STATE>
 __host__ __device__ inline WsLayout ws_layout(const GemmArgs& g) {
   WsLayout w;
   const bool row = ROW_STATE > 0 && row_uses_workspace(g);
-  const bool col = COL_STATE > 0 && g.tiles_m > 1;
+  const bool col = COL_STATE > 0 && (g.tiles_m > 1 || g.col_fold_count > 1);
   const int64_t ncnt = (row ? (int64_t)g.L * g.tiles_m : 0) + (col ? (int64_t)g.L * g.tiles_n : 0);
   w.counter_bytes = (ncnt * 4 + 255) / 256 * 256;
   w.row_bytes = row ? ((int64_t)g.L * g.tiles_n * g.M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
@@ -406,6 +406,14 @@ __host__ __device__ inline int fold_key(const GemmArgs& g, int batch) {
 }
 __host__ __device__ inline int fold_member(const GemmArgs& g, int key, int j) {
   return g.row_fold_count == 1 ? key : (g.row_fold_mod ? key + j * g.row_fold_step : key * g.row_fold_count + j);
+}
+// folded per-column reductions (batches that agree modulo col_fold_step share a result)
+__host__ __device__ inline bool col_uses_workspace(const GemmArgs& g) { return g.tiles_m > 1 || g.col_fold_count > 1; }
+__host__ __device__ inline int col_fold_key(const GemmArgs& g, int batch) {
+  return g.col_fold_count == 1 ? batch : batch % g.col_fold_step;
+}
+__host__ __device__ inline int col_fold_member(const GemmArgs& g, int key, int j) {
+  return g.col_fold_count == 1 ? key : key + j * g.col_fold_step;
 }
 
 // Device-scope accesses for data exchanged between workgroups inside one
@@ -547,7 +555,7 @@ EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, co
       for (int c = 0; c < CS; ++c) st[c] = lds[lc * CS + c];
 #pragma unroll
       for (int w = 1; w < Cfg::WM; ++w) Epi::col_combine(st, lds + (w * Cfg::BN + lc) * CS);
-      if (t.tiles_m == 1) {
+      if (!col_uses_workspace(g)) {
         Epi::col_finalize(p, t.batch, col, st);
       } else {
         float* dst = part + (((int64_t)t.batch * t.tiles_m + t.tile_m) * t.N + col) * CS;
@@ -555,10 +563,10 @@ EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, co
         for (int c = 0; c < CS; ++c) st_device(dst + c, st[c]);
       }
     }
-    if (t.tiles_m == 1 || !g.col_inkernel) return false;
+    if (!col_uses_workspace(g) || !g.col_inkernel) return false;
     const int row_counters = (Epi::ROW_STATE > 0 && row_uses_workspace(g)) ? t.L * t.tiles_m : 0;
-    int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
-    return arrive_last(counter, t.tiles_m, flag);
+    int* counter = (int*)t.workspace + row_counters + col_fold_key(g, t.batch) * t.tiles_n + t.tile_n;
+    return arrive_last(counter, t.tiles_m * g.col_fold_count, flag);
   } else {
     return false;
   }
@@ -575,8 +583,9 @@ EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, c
     const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     const float* part = (const float*)(t.workspace + wl.counter_bytes + wl.row_bytes);
     const int row_counters = (Epi::ROW_STATE > 0 && row_uses_workspace(g)) ? t.L * t.tiles_m : 0;
-    int* counter = (int*)t.workspace + row_counters + t.batch * t.tiles_n + t.tile_n;
-    // SHARES threads per column each fold every SHARES-th partial in tile order
+    const int key = col_fold_key(g, t.batch);
+    int* counter = (int*)t.workspace + row_counters + key * t.tiles_n + t.tile_n;
+    // SHARES threads per column each fold every SHARES-th partial in (batch, tile) order
     // (independent loads in flight together), LDS then combines the shares in order
     const int lc = t.tid % Cfg::BN, share = t.tid / Cfg::BN;
     const int col = t.n0 + lc;
@@ -584,12 +593,13 @@ EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, c
     float st[CS];
     Epi::col_identity(st);
     if (live) {
-      const float* src = part + ((int64_t)t.batch * t.tiles_m * t.N + col) * CS;
 #pragma unroll 8
-      for (int j = share; j < t.tiles_m; j += SHARES) {
+      for (int q = share; q < t.tiles_m * g.col_fold_count; q += SHARES) {
+        const int f = q / t.tiles_m, j = q - f * t.tiles_m;
+        const float* src = part + (((int64_t)col_fold_member(g, key, f) * t.tiles_m + j) * t.N + col) * CS;
         float o[CS];
 #pragma unroll
-        for (int c = 0; c < CS; ++c) o[c] = ld_device(src + (int64_t)j * t.N * CS + c);
+        for (int c = 0; c < CS; ++c) o[c] = ld_device(src + c);
         Epi::col_combine(st, o);
       }
     }
@@ -601,7 +611,7 @@ EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, c
     __syncthreads();
     if (live && share == 0) {
       for (int s2 = 1; s2 < SHARES; ++s2) Epi::col_combine(st, lds + (s2 * Cfg::BN + lc) * CS);
-      Epi::col_finalize(p, t.batch, col, st);
+      Epi::col_finalize(p, key, col, st);
     }
     if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }

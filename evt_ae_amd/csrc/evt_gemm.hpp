@@ -65,6 +65,9 @@ struct GemmArgs {
   // (result keyed by l % row_fold_step), otherwise row_fold_count consecutive
   // ones (keyed by l / row_fold_count).  (0, 1, 1): every batch on its own.
   int row_fold_mod, row_fold_step, row_fold_count;
+  // A per-column reduction may fold the batches that agree modulo col_fold_step (col_fold_count of them) into
+  // one result, keyed by l % col_fold_step.  (1, 1): every batch on its own.
+  int col_fold_step, col_fold_count;
   // Split-K: `splits` workgroups share an output tile, each over `k_chunk` (a multiple of BK) of the K extent;
   // they leave their accumulators in the workspace and the last one to arrive adds them up in split order and
   // runs the epilogue.  splits == 1: one workgroup per tile, nothing goes through the workspace.

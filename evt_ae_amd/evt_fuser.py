@@ -543,6 +543,10 @@ class FusedBMM(FusedOpBase):
             tuner = BMMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
             tile = tuner.get_best_config()
             self.tile = tile
+            for r in self.ir.reduces.values():
+                # folded per-column partials are combined inside the kernel only: at most 64 per result
+                if r.axis == "col" and r.fold and -(-M // tile.bm) * r.fold_count > 64:
+                    raise NotImplementedError(f"{r.name}: {-(-M // tile.bm) * r.fold_count} partials per column")
             self.spec = KernelSpec(self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
             self.module = jit.load_module(self.ir, self.spec)
 
@@ -1344,16 +1348,20 @@ class EVTFuser:
             axis, fold, fold_step, fold_count = "row", "div", 1, st.l_div     # l_div consecutive batches summed
         elif st.stride_m == 0 and numel == self.L * self.N and (self.L == 1 or st.stride_l != 0):
             axis = "col"
+        elif (st.stride_m == 0 and st.stride_n != 0 and st.l_mod and st.l_div == 1 and not st.stride_l2
+              and numel == st.l_mod * self.N and kind in ("sum", "max")):
+            # per column, and over the batches that agree modulo l_mod: the bias gradient behind a batched product
+            # whose result is merged back into [B, S, H * D] (sum over B and S for every head and column)
+            axis, fold, fold_step, fold_count = "col", "mod", st.l_mod, self.L // st.l_mod
         else:
             raise NotImplementedError(
                 f"{node.name}: reduces over something other than the N axis (optionally with batches folded) "
                 f"or exactly the M axis")
         if fold and kind not in ("sum", "max"):
             raise NotImplementedError(f"{node.name}: {kind} reduction that also folds batches")
-        if axis == "row":
-            for other in self.ir.reduces.values():
-                if other.axis == "row" and (other.fold, other.fold_step, other.fold_count) != (fold, fold_step, fold_count):
-                    raise NotImplementedError(f"{node.name}: per-row reductions of one epilogue fold batches differently")
+        for other in self.ir.reduces.values():
+            if other.axis == axis and (other.fold, other.fold_step, other.fold_count) != (fold, fold_step, fold_count):
+                raise NotImplementedError(f"{node.name}: per-{axis} reductions of one epilogue fold batches differently")
         rname = f"{node.name}_red"
         red = self.ir.add_reduce(rname, kind, axis, value)
         red.fold, red.fold_step, red.fold_count = fold, fold_step, fold_count

@@ -69,6 +69,9 @@ def register_all() -> List[jit.LazyModule]:
     for n in W.AFFINE_LN_LENGTHS:
         mod, ins = W.affine_layer_norm(n)
         W.fuse(mod, _meta(ins), passes=[pass_decomposition, pass_fusion])
+    for transposed in (False, True):
+        mod, ins = W.head_merge_bias_grad(transposed=transposed)
+        W.fuse(mod, _meta(ins))
     for anchor in W.RANDOM_EPILOGUE_ANCHORS:
         for seed in W.RANDOM_EPILOGUE_SEEDS[:12 if anchor == "mm" else 6]:
             mod, ins = W.random_epilogue(seed, anchor)

@@ -851,6 +851,37 @@ class _BareLayerNormBackward(torch.nn.Module):
         return operator.getitem(ln, 0)
 
 
+class HeadMergeBiasGrad(torch.nn.Module):
+    """What the backward pass of an attention layer does with the gradient of a
+    projection's output: a batched product over L = B * H heads whose result is
+    merged back into [B * S, H * D] (permute + copy, folded into the store) and
+    summed over all rows for the bias gradient -- per column and over the
+    batches that agree modulo H.  `transposed`: the product comes out as
+    [D, S] per head (the key gradient), so the same sum runs along rows."""
+    def __init__(self, B: int, H: int, S: int, D: int, transposed: bool = False) -> None:
+        super().__init__()
+        self.dims, self.transposed = (B, H, S, D), transposed
+
+    def forward(self, a, b):
+        B, H, S, D = self.dims
+        out = aten.bmm(a, b)
+        if self.transposed:                                      # [L, D, S]
+            merged = aten.permute(aten.view(out, [B, H, D, S]), [0, 3, 1, 2])
+        else:                                                    # [L, S, D]
+            merged = aten.permute(aten.view(out, [B, H, S, D]), [0, 2, 1, 3])
+        w = aten.view(aten.clone(merged, memory_format=torch.contiguous_format), [B * S, H * D])
+        return w, aten.view(aten.sum(w, [0], True), [H * D])
+
+
+def head_merge_bias_grad(B: int = 4, H: int = 6, S: int = 320, D: int = 64, K: int = 96, transposed: bool = False,
+                         seed: int = 0):
+    g = torch.Generator(device="cpu").manual_seed(0xB1A5 + seed)
+    h = lambda *sh: (torch.randn(*sh, generator=g) * 0.3).half()   # noqa: E731
+    a = h(B * H, D, K) if transposed else h(B * H, S, K)
+    b = h(B * H, K, S) if transposed else h(B * H, K, D)
+    return HeadMergeBiasGrad(B, H, S, D, transposed), [a, b]
+
+
 class RandomEpilogue(torch.nn.Module):
     """A seeded random epilogue tree behind a GEMM: 5 .. 9 element-wise steps
     over the accumulator, a same-shape tensor, a row vector, a column vector

@@ -109,10 +109,11 @@ def interpret(ir, accum: torch.Tensor, slot_tensors: Dict[int, torch.Tensor]) ->
                 if r.kind not in ("sum", "max"):
                     raise NotImplementedError(f"folded {r.kind}")
                 cnt = r.fold_count
-                grouped = out.view(cnt, L // cnt, M, 1) if r.fold == "mod" else out.view(L // cnt, cnt, M, 1)
+                tail = (M, 1) if r.axis == "row" else (1, N)
+                grouped = out.view(cnt, L // cnt, *tail) if r.fold == "mod" else out.view(L // cnt, cnt, *tail)
                 axis = 0 if r.fold == "mod" else 1
                 tot = grouped.sum(axis, keepdim=True) if r.kind == "sum" else grouped.amax(axis, keepdim=True)
-                out = tot.expand_as(grouped).reshape(L, M, 1)
+                out = tot.expand_as(grouped).reshape(L, *tail)
             val[name] = out
         else:
             val[name] = _apply(node.op, [val[i] for i in node.inputs])

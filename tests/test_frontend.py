@@ -344,3 +344,22 @@ def test_rows_too_long_for_the_row_kernel_stay_eager():
     gm = W.fuse(WideSoftmax(), [x])
     assert not fused_nodes(gm)
     assert [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"] == ["_softmax", "mul"]
+
+
+@pytest.mark.parametrize("transposed", [False, True])
+def test_bias_gradient_behind_a_head_merge_lowers_correctly(transposed):
+    """A batched product over B * H heads, merged into [B * S, H * D] by a permuted
+    store, with the bias gradient (sum over every row) on top: per column and
+    over the batches that agree modulo H, or, for the transposed product, along
+    the rows with the same fold.  One kernel, values from the IR interpreter."""
+    mod, inputs = W.head_merge_bias_grad(B=2, H=3, S=40, D=16, K=24, transposed=transposed)
+    gm = W.fuse(mod, inputs)
+    (n,) = fused_nodes(gm)
+    assert not [x for x in gm.graph.nodes if x.op == "call_function" and target_name(x.target) in ("sum", "clone", "bmm")]
+    (red,) = n.target.ir.reduces.values()
+    assert (red.axis, red.fold, red.fold_step, red.fold_count) == ("row" if transposed else "col", "mod", 3, 2)
+    got = run_emulated(gm, inputs)
+    ref = evt_oracle.eval_fp32(mod, inputs)
+    for o, r in zip(got, ref):
+        assert tuple(o.shape) == tuple(r.shape)
+        assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3

@@ -679,3 +679,26 @@ def test_bench_argument_sets_are_independent():
     for i in range(1, case.nsets):
         for a, b in zip(first, case.outputs(i)):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("transposed", [False, True], ids=["per_column", "per_row"])
+def test_bias_gradient_behind_a_head_merge(transposed):
+    """The backward pattern of an attention projection: batched product over
+    B * H heads, result merged into [B * S, H * D] by the store, bias gradient
+    = sum over all rows, i.e. per column (or, for the transposed product, per
+    row) and over the batches that agree modulo H.  Several row tiles and
+    several batches per result; repeated launches are bit-identical."""
+    mod, inputs = W.head_merge_bias_grad(transposed=transposed)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    (red,) = node.target.ir.reduces.values()
+    assert red.fold == "mod" and red.axis == ("row" if transposed else "col") and red.fold_count == 4
+    dev = [t.cuda() for t in inputs]
+    outs = [o.clone() for o in gm(*dev)]
+    again = gm(*dev)
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    for o, a, r in zip(outs, again, refs):
+        assert torch.equal(o, a)
+        assert tuple(o.shape) == tuple(r.shape)
+        assert evt_oracle.max_rel_err(o, r) <= FP16_TOL

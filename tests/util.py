@@ -22,7 +22,7 @@ def emulate_fused(op: FusedOpBase, *args):
         Bl = B.t() if op.b_kc else B
         acc = Al @ Bl
     else:
-        acc = torch.bmm(aten.permute(A, op.permute_A), aten.permute(B, op.permute_B))
+        acc = op.anchor_eager(A, B)        # replays the operands' layout chains
     loads = {}
     for k, slot in enumerate(op.ir.slots):
         kind, ref = op.slot_sources[k]
