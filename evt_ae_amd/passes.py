@@ -123,10 +123,21 @@ def _absorb_side_expressions(anchor: Node, inside: Set[Node], desc: Set[Node], t
     """Broadcast-side expressions (e.g. a mask built from a small tensor) whose
     every user is inside the partition join it.  They are not downstream of the
     anchor, so this cannot close a cycle between partitions."""
+    # producers of the anchor's operands inside the partition (layout chains read through strides): what feeds
+    # them is the operand's source tensor, never a side expression of the epilogue
+    pre: Set[Node] = set()
+    stack = [a for a in anchor.all_input_nodes if a in inside]
+    while stack:
+        n = stack.pop()
+        if n not in pre:
+            pre.add(n)
+            stack.extend(a for a in n.all_input_nodes if a in inside)
     changed = True
     while changed:
         changed = False
         for node in list(inside):
+            if node in pre:
+                continue
             for i in node.all_input_nodes:
                 if (i in inside or i in desc or i in taken or i.op != "call_function"
                         or target_name(i.target) not in _SMALL_SIDE or node is anchor
