@@ -389,6 +389,8 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                                         the reference compares with -1 instead of ignore_index)
       masked_fill(x, mask, v)        -> where(mask, v, x)                        (scalar v; not in the reference)
       getitem(unbind(x, d), i)       -> select(x, d, i)                          (not in the reference)
+      add of select_backward(g_i, s, d, i) over every i
+                                     -> stack([g_0, g_1, ...], d)                (not in the reference)
       native_layer_norm(x, s, w, b, eps)
                                      -> add(mul(native_layer_norm(x, s, None, None, eps)[0], w), b)   (:504-544)
     and permute(permute(x)) folded into one permute or none.  The reference's
@@ -478,6 +480,29 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                     graph.erase_node(node)
                     changed = True
                 continue
+            elif name == "add" and len(node.args) == 2 and node.kwargs.get("alpha", 1) == 1:
+                # add(add(select_backward(g0, s, d, 0), select_backward(g1, s, d, 1)), ...) over every index of d
+                # is stack([g0, g1, ...], d): one copy instead of a zero-filled tensor per slice and the adds
+                leaves, ok = [], True
+
+                def collect(x):
+                    nonlocal ok
+                    if not (isinstance(x, Node) and x.op == "call_function" and len(x.users) == 1) and x is not node:
+                        ok = False
+                    elif target_name(x.target) == "select_backward":
+                        leaves.append(x)
+                    elif target_name(x.target) == "add" and len(x.args) == 2 and x.kwargs.get("alpha", 1) == 1:
+                        collect(x.args[0])
+                        collect(x.args[1])
+                    else:
+                        ok = False
+                collect(node)
+                if ok and leaves:
+                    shape, dim = list(leaves[0].args[1]), int(leaves[0].args[2])
+                    by_index = {int(x.args[3]): x.args[0] for x in leaves
+                                if list(x.args[1]) == shape and int(x.args[2]) == dim}
+                    if len(by_index) == len(leaves) == shape[dim] and sorted(by_index) == list(range(shape[dim])):
+                        new = mk(aten.stack, ([by_index[i] for i in range(shape[dim])], dim))
             elif name == "unbind" and all(u.op == "call_function" and u.target is operator.getitem for u in node.users):
                 # getitem(unbind(x, d), i) is select(x, d, i): a layout op the batched products read through
                 x = node.args[0]
@@ -513,6 +538,7 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
             changed = True
     changed = _fold_permutes(graph) or changed
     if changed:
+        graph.eliminate_dead_code()        # what a rewrite replaced piecewise (the adds under a stack, ...)
         graph.lint()
         module.recompile()
         _repropagate(module)

@@ -301,6 +301,35 @@ def test_fused_qkv_forward_reads_its_heads_in_place():
         assert ops[0].bdiva == ops[0].bdivb == ops[1].bdivb == 4 and ops[0].lda == ops[0].ldb == 3 * d
 
 
+def test_select_backward_sum_becomes_a_stack():
+    """The gradient of q, k, v = qkv[0], qkv[1], qkv[2]: three zero-filled tensors
+    with one slice set, added up.  pass_decomposition turns the sum into one
+    stack (same values), and an incomplete or mixed sum is left alone."""
+    import operator
+    from evt_ae_amd.passes import pass_decomposition
+    aten = torch.ops.aten
+
+    class Full(torch.nn.Module):
+        def forward(self, a, b, c):
+            s = [3, 2, 4]
+            return aten.add(aten.add(aten.select_backward(a, s, 0, 0), aten.select_backward(b, s, 0, 1)),
+                            aten.select_backward(c, s, 0, 2))
+
+    class Partial(torch.nn.Module):
+        def forward(self, a, b, c):
+            s = [3, 2, 4]
+            return aten.add(aten.add(aten.select_backward(a, s, 0, 0), aten.select_backward(b, s, 0, 1)),
+                            aten.select_backward(c, s, 0, 1))
+
+    ins = [torch.randn(2, 4) for _ in range(3)]
+    for mod, want_stack in ((Full(), True), (Partial(), False)):
+        gm = W.trace_module(mod, ins)
+        pass_decomposition(gm, gm.graph)
+        names = [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+        assert ("stack" in names) == want_stack and ("select_backward" in names) != want_stack, names
+        assert torch.equal(gm(*ins), mod(*ins))
+
+
 def test_dropout_in_a_training_step_is_fused_and_leaves_nothing_behind():
     """native_dropout becomes rand_like / ge / mul inside the GEMM epilogues; the
     masks are kernel outputs saved for backward.  fx keeps random ops alive as
