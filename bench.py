@@ -231,11 +231,12 @@ def bench_row_anchors(torch, W, steps, warmup):
     return out
 
 
-def bench_encoder_step(torch, W, iters=20):
+def bench_encoder_step(torch, W, iters=20, only=None):
     """One training step (forward + backward) of a BERT-large encoder layer in
     fp16, through AOT autograd with every GEMM / BMM / softmax / layer norm
     fused, against the same model run eagerly; both also replayed from a HIP
-    graph, which removes the host-side launch cost of either."""
+    graph, which removes the host-side launch cost of either.  `only` =
+    "fused" | "eager" runs just that side in a plain loop (for kernel traces)."""
     import copy
     from evt_ae_amd.aot_helper import aot_optimize
     model, (x, target) = W.encoder_layer(device="cuda", **W.ENCODER_BENCH)
@@ -283,6 +284,14 @@ def bench_encoder_step(torch, W, iters=20):
             torch.cuda.synchronize()
         return loop_ms, graph_ms
 
+    if only is not None:
+        fn, params = (fused, list(model.parameters())) if only == "fused" else (eager, list(eager.parameters()))
+        for _ in range(3 + iters):
+            for p in params:
+                p.grad = None
+            fn(x, target).backward()
+        torch.cuda.synchronize()
+        return {"model": "post-LN encoder layer", **W.ENCODER_BENCH, "dtype": "f16", "only": only, "steps": 3 + iters}
     e_loop, e_graph = run(eager, list(eager.parameters()))
     f_loop, f_graph = run(fused, list(model.parameters()))
     ref = [p.grad.float() for p in eager.parameters()]
@@ -345,6 +354,9 @@ def main():
                     help="timed regions of --steps launches per config; the median is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--only-encoder-step", choices=("fused", "eager"), default=None,
+                    help="run nothing but the encoder layer's training step, that side only, in a plain loop, and print "
+                         "a short JSON line (for rocprofv3 kernel traces of the step)")
     ap.add_argument("--no-encoder-step", dest="encoder_step", action="store_false",
                     help="skip the fused-vs-eager training step of an encoder layer (encoder_layer_step in the output)")
     ap.add_argument("--no-row-anchors", dest="row_anchors", action="store_false",
@@ -368,6 +380,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no HIP device available")
     torch.cuda.set_device(0)
+    if args.only_encoder_step:
+        print(json.dumps({"encoder_layer_step": bench_encoder_step(torch, W, only=args.only_encoder_step)}), flush=True)
+        return
     cfgs = [int(c) for c in args.configs.split(",")]
     details = {}
     for cfg in cfgs:
