@@ -366,6 +366,71 @@ def _fold_permutes(graph: Graph) -> bool:
     return changed
 
 
+def _stack_merge_to_cat(graph: Graph) -> bool:
+    """stack([x_0 .. x_{n-1}], 0) -> permute -> clone -> view, where the permute
+    leaves the stacked axis in front of the axes that the view merges into the
+    last one (the gradient of a fused [d, 3d] projection: [3, B, H, S, D] ->
+    [B, S, 3, H, D] -> [B * S, 3 * H * D]), is the concatenation along the last
+    axis of the x_i, each permuted and merged by itself:
+        cat([view(clone(permute(x_i, p')), [..., H * D]) for i], -1).
+    One copy (the cat) instead of two (stack, clone), and the per-tensor
+    permute / clone / view is a layout chain the producing kernel's store takes
+    over."""
+    changed = False
+    for node in list(graph.nodes):
+        if not (node.op == "call_function" and target_name(node.target) == "stack"):
+            continue
+        tensors = list(node.args[0])
+        dim = int(node.args[1]) if len(node.args) > 1 else int(node.kwargs.get("dim", 0))
+        if dim != 0 or len(node.users) != 1 or not all(isinstance(t, Node) and "tensor_meta" in t.meta for t in tensors):
+            continue
+        perm = next(iter(node.users))
+        if not (perm.op == "call_function" and target_name(perm.target) == "permute" and len(perm.users) == 1):
+            continue
+        clone = next(iter(perm.users))
+        if not (clone.op == "call_function" and target_name(clone.target) == "clone" and len(clone.users) == 1):
+            continue
+        view = next(iter(clone.users))
+        if not (view.op == "call_function" and target_name(view.target) in ("view", "_unsafe_view", "reshape")):
+            continue
+        dims = [int(d) for d in perm.args[1]]
+        rank = len(dims)
+        k = dims.index(0)                        # where the stacked axis lands
+        if k == 0 or k == rank - 1:
+            continue
+        src_shape = [int(x) for x in tensors[0].meta["tensor_meta"].shape]
+        if any([int(x) for x in t.meta["tensor_meta"].shape] != src_shape for t in tensors):
+            continue
+        lead = [src_shape[d - 1] for d in dims[:k]]
+        tail = 1
+        for d in dims[k + 1:]:
+            tail *= src_shape[d - 1]
+        out_shape = [int(x) for x in view.args[1]]
+        lead_numel = 1
+        for x in lead:
+            lead_numel *= x
+        # the view must merge exactly the stacked axis and what follows it into its last axis
+        rest = 1
+        for x in out_shape[:-1]:
+            rest *= x
+        if out_shape[-1] != len(tensors) * tail or rest != lead_numel:
+            continue
+        sub = [d - 1 for d in dims[:k] + dims[k + 1:]]
+        with graph.inserting_before(view):
+            parts = []
+            for t in tensors:
+                p = inherit_meta(graph.call_function(aten.permute, (t, sub)), view)
+                c = inherit_meta(graph.call_function(aten.clone, (p,), {"memory_format": torch.contiguous_format}), view)
+                parts.append(inherit_meta(graph.call_function(aten.view, (c, out_shape[:-1] + [tail])), view))
+            cat = inherit_meta(graph.call_function(aten.cat, (parts, -1)), view)
+            for k_ in ("tensor_meta", "val"):
+                if k_ in view.meta:
+                    cat.meta[k_] = view.meta[k_]
+        view.replace_all_uses_with(cat)
+        changed = True
+    return changed
+
+
 def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: Sequence[str] = ()):
     """The subset of the reference's Decomposition pass
     (python/gtl/compiler/passes/pass_decomposition.py:192-502, entry :817) that
@@ -391,6 +456,8 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
       getitem(unbind(x, d), i)       -> select(x, d, i)                          (not in the reference)
       add of select_backward(g_i, s, d, i) over every i
                                      -> stack([g_0, g_1, ...], d)                (not in the reference)
+      view(clone(permute(stack(xs, 0)))) that merges the stacked axis into the last one
+                                     -> cat([view(clone(permute(x))) for x in xs], -1)   (not in the reference)
       native_layer_norm(x, s, w, b, eps)
                                      -> add(mul(native_layer_norm(x, s, None, None, eps)[0], w), b)   (:504-544)
     and permute(permute(x)) folded into one permute or none.  The reference's
@@ -537,6 +604,8 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
             graph.erase_node(node)
             changed = True
     changed = _fold_permutes(graph) or changed
+    if "stack" not in disabled:
+        changed = _stack_merge_to_cat(graph) or changed
     if changed:
         graph.eliminate_dead_code()        # what a rewrite replaced piecewise (the adds under a stack, ...)
         graph.lint()

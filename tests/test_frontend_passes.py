@@ -330,6 +330,36 @@ def test_select_backward_sum_becomes_a_stack():
         assert torch.equal(gm(*ins), mod(*ins))
 
 
+def test_stack_merge_becomes_a_cat_of_merged_parts():
+    """stack -> permute -> clone -> view that merges the stacked axis into the last
+    one (the gradient of a fused [d, 3d] projection) is rewritten into a cat of
+    the parts, each permuted and merged by itself: same values, no stack; other
+    permutes of a stack are left alone."""
+    from evt_ae_amd.passes import pass_decomposition
+    aten = torch.ops.aten
+    B, H, S, D = 2, 3, 5, 4
+
+    class Merge(torch.nn.Module):
+        def forward(self, a, b, c):
+            st = aten.stack([a, b, c], 0)
+            return aten.view(aten.clone(aten.permute(st, [1, 3, 0, 2, 4]), memory_format=torch.contiguous_format),
+                             [B * S, 3 * H * D])
+
+    class Other(torch.nn.Module):
+        def forward(self, a, b, c):
+            st = aten.stack([a, b, c], 0)
+            return aten.view(aten.clone(aten.permute(st, [1, 0, 3, 2, 4]), memory_format=torch.contiguous_format),
+                             [B * 3, S * H * D])
+
+    ins = [torch.randn(B, H, S, D) for _ in range(3)]
+    for mod, rewritten in ((Merge(), True), (Other(), False)):
+        gm = W.trace_module(mod, ins)
+        pass_decomposition(gm, gm.graph)
+        names = [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+        assert ("cat" in names) == rewritten and ("stack" in names) != rewritten, names
+        assert torch.equal(gm(*ins), mod(*ins))
+
+
 def test_dropout_in_a_training_step_is_fused_and_leaves_nothing_behind():
     """native_dropout becomes rand_like / ge / mul inside the GEMM epilogues; the
     masks are kernel outputs saved for backward.  fx keeps random ops alive as
