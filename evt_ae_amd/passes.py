@@ -427,6 +427,31 @@ def _stack_merge_to_cat(graph: Graph) -> bool:
                 if k_ in view.meta:
                     cat.meta[k_] = view.meta[k_]
         view.replace_all_uses_with(cat)
+        # a sum over the rows of the concatenation (the fused projection's bias gradient) is the concatenation of
+        # the parts' sums, and each of those joins the epilogue of the kernel that produces its part
+        frontier = [cat]
+        while frontier:
+            x = frontier.pop()
+            for user in list(x.users):
+                name_u = target_name(user.target) if user.op == "call_function" else ""
+                if name_u in ("view", "_unsafe_view", "reshape") and "tensor_meta" in user.meta \
+                        and int(user.meta["tensor_meta"].shape[-1]) == out_shape[-1]:
+                    frontier.append(user)            # regroups the rows only
+                    continue
+                if name_u != "sum" or len(user.args) < 2 or "tensor_meta" not in user.meta:
+                    continue
+                rank_x = len(x.meta["tensor_meta"].shape) if "tensor_meta" in x.meta else len(out_shape)
+                if sorted(int(d) % rank_x for d in user.args[1]) != list(range(rank_x - 1)):
+                    continue                         # not a sum over every row
+                with graph.inserting_before(user):
+                    sums = [inherit_meta(graph.call_function(aten.sum, (p_, list(range(len(out_shape) - 1)), True)), user)
+                            for p_ in parts]
+                    total = inherit_meta(graph.call_function(aten.cat, (sums, -1)), user)
+                    total = inherit_meta(graph.call_function(aten.view, (total, [int(d) for d in user.meta["tensor_meta"].shape])), user)
+                    for k_ in ("tensor_meta", "val"):
+                        if k_ in user.meta:
+                            total.meta[k_] = user.meta[k_]
+                user.replace_all_uses_with(total)
         changed = True
     return changed
 

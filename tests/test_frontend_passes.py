@@ -351,6 +351,14 @@ def test_stack_merge_becomes_a_cat_of_merged_parts():
             return aten.view(aten.clone(aten.permute(st, [1, 0, 3, 2, 4]), memory_format=torch.contiguous_format),
                              [B * 3, S * H * D])
 
+    class MergeAndBias(torch.nn.Module):       # the bias gradient: sum over every row, through a regrouping view
+        def forward(self, a, b, c):
+            st = aten.stack([a, b, c], 0)
+            m = aten.view(aten.clone(aten.permute(st, [1, 3, 0, 2, 4]), memory_format=torch.contiguous_format),
+                          [B, S, 3 * H * D])
+            rows = aten.view(m, [B * S, 3 * H * D])
+            return rows, aten.sum(rows, [0], True)
+
     ins = [torch.randn(B, H, S, D) for _ in range(3)]
     for mod, rewritten in ((Merge(), True), (Other(), False)):
         gm = W.trace_module(mod, ins)
@@ -358,6 +366,12 @@ def test_stack_merge_becomes_a_cat_of_merged_parts():
         names = [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"]
         assert ("cat" in names) == rewritten and ("stack" in names) != rewritten, names
         assert torch.equal(gm(*ins), mod(*ins))
+    gm = W.trace_module(MergeAndBias(), ins)
+    pass_decomposition(gm, gm.graph)
+    sums = [n for n in gm.graph.nodes if n.op == "call_function" and target_name(n.target) == "sum"]
+    assert len(sums) == 3 and all(tuple(n.meta["tensor_meta"].shape) == (1, 1, H * D) for n in sums)
+    for got, want in zip(gm(*ins), MergeAndBias()(*ins)):
+        assert got.shape == want.shape and torch.allclose(got, want, atol=1e-5)
 
 
 def test_dropout_in_a_training_step_is_fused_and_leaves_nothing_behind():
