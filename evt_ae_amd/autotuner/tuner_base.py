@@ -22,7 +22,7 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 
-from ..codegen import KernelSpec, TileConfig
+from ..codegen import KernelSpec, TileConfig, reduction_lds_bytes
 from ..ir import EpilogueIR
 
 NUM_CUS = 256
@@ -95,7 +95,10 @@ class AutoTunerBase:
         known = {f.name for f in fields(TileConfig)}
         if any(k not in known and v for k, v in cfg.items()):
             return None      # uses an option this version does not have: ignore the row
-        return TileConfig(**{k: v for k, v in cfg.items() if k in known})
+        tile = TileConfig(**{k: v for k, v in cfg.items() if k in known})
+        # the key holds the epilogue's node counts, not its reduction states: a row tuned for another epilogue
+        # with the same counts may be too small for this one's exchange area
+        return tile if self.fits(tile) else None
 
     def store(self, tile: TileConfig, us: float) -> None:
         con = self._connect()
@@ -106,9 +109,6 @@ class AutoTunerBase:
 
     # -- search space --------------------------------------------------------------
     def candidates(self) -> List[TileConfig]:
-        red_lds = lambda t: ((t.wn * t.bm * self.ir.row_state * 4 + 16 if self.ir.row_state else 0) +   # noqa: E731
-                             (max(t.wm, max(1, t.wm * t.wn * 64 // t.bn)) * t.bn * self.ir.col_state * 4 + 16
-                              if self.ir.col_state else 0))
         out = []
         if self.dma:
             # (bm, bn, bk, wave grid, LDS stages, pipeline): plain ring (0), look-ahead ring (1),
@@ -141,9 +141,13 @@ class AutoTunerBase:
             shapes += [(bm, bn, bk, wm, wn, 1, 0) for (bm, bn, _, wm, wn, st, pipe) in shapes if pipe == 0 and st == 2]
         for bm, bn, bk, wm, wn, st, pipe in shapes:
             t = TileConfig(bm, bn, bk, wm, wn, st, self.dma, 4, pipe)
-            if t.lds_bytes() <= LDS_LIMIT and t.lds_bytes() >= red_lds(t) and t not in out:
+            if self.fits(t) and t not in out:
                 out.append(t)
         return out
+
+    def fits(self, t: TileConfig) -> bool:
+        """The tile's stages fit the LDS and hold this epilogue's reduction exchange area."""
+        return reduction_lds_bytes(t, self.ir.row_state, self.ir.col_state) <= t.lds_bytes() <= LDS_LIMIT
 
     def heuristic(self) -> TileConfig:
         """Pick the candidate with the lowest modelled time: number of

@@ -31,7 +31,8 @@ class TileConfig:
     group_m: int = 4
     # 0: plain ring; 1: look-ahead ring with pinned instruction order (stages >= 3);
     # 2: ping-pong, the two waves of a SIMD alternate MFMA and LDS-read phases (8 waves, stages >= 2);
-    # 3: ping-pong with one barrier per k-tile
+    # 3: ping-pong with one barrier per k-tile; 4 + flags: as 3 with 1 = the barrier inside group 0's MFMA phase,
+    # 2 = group 0 issues its transfers between its LDS reads, 4 = group 1 as well (stages >= 3)
     pipe: int = 0
 
     def tag(self) -> str:
@@ -48,6 +49,18 @@ class KernelSpec:
     b_kc: bool          # B contiguous along K (column-major, i.e. stored [N, K])
     bf16: bool
     tile: TileConfig
+
+
+def reduction_lds_bytes(t: "TileConfig", row_state: int, col_state: int) -> int:
+    """LDS the epilogue's reductions need inside the operand stages: the per-wave row states [wn][bm] and the
+    column states [max(wm, shares)][bn] side by side (each followed by a flag), and for phase 2 of a per-row
+    reduction one state per thread."""
+    need = 0
+    if row_state:
+        need += t.wn * t.bm * row_state * 4 + 16
+    if col_state:
+        need += max(t.wm, max(1, t.wm * t.wn * 64 // t.bn)) * t.bn * col_state * 4 + 16
+    return max(need, t.wm * t.wn * 64 * row_state * 4)
 
 
 _BINARY = {
@@ -244,6 +257,7 @@ class Codegen:
         hoisted = [n for n in need if not self.var_m[n]]
         inner = [n for n in need if self.var_m[n]]
 
+        aux_nodes = [n for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "aux"]
         e("template <class Cfg, class Tile, bool FAST>")
         e("static EVT_DEV void tile(const Params& p, const Tile& t, const evt::GemmArgs& g, "
           "const evt::f32x16 (&acc)[Cfg::MI][Cfg::NI]) {")
@@ -263,16 +277,14 @@ class Codegen:
                 e(f"cst[ni][{r.state_offset}] = {_IDENTITY[r.kind]};")
             e.dedent()
             e("}")
-        aux_nodes = [n for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "aux"]
         # check-free path: wave-uniform row base (scalar registers) + one per-lane offset per tensor
         for k in [ir.nodes[n].slot for n in aux_nodes] + [s_.slot for s_ in tile_stores]:
-            ct = DTYPE_CTYPES[ir.slots[k].dtype]
-            cq = "const " if ir.slots[k].role == "load" else ""
-            e(f"[[maybe_unused]] {cq}{ct}* ub_{k} = nullptr;")
-            e(f"[[maybe_unused]] uint32_t lo_{k} = 0;")
+            e(f"[[maybe_unused]] __amdgpu_buffer_rsrc_t rs_{k};   // this wave's corner of the tile (scalar registers)")
+            e(f"[[maybe_unused]] uint32_t vo_{k} = 0;              // this lane's byte offset inside a row")
+            e(f"[[maybe_unused]] const uint32_t rp_{k} = (uint32_t)p.t{k}_sm * (uint32_t)sizeof(*p.t{k});   // row pitch in bytes")
             e("if constexpr (FAST) {")
-            e(f"  ub_{k} = p.t{k} + {self.slot_off(k)} + (int64_t)t.row_u * p.t{k}_sm + t.col_u;")
-            e(f"  lo_{k} = (uint32_t)(t.row_l * (int)p.t{k}_sm + t.col_l);")
+            e(f"  rs_{k} = evt::make_rsrc((const char*)(p.t{k} + {self.slot_off(k)} + (int64_t)t.row_u * p.t{k}_sm + t.col_u));")
+            e(f"  vo_{k} = (uint32_t)(t.row_l * (int)p.t{k}_sm + t.col_l) * (uint32_t)sizeof(*p.t{k});")
             e("}")
         # With a cross-workgroup reduction in the same epilogue, the arrival ticket has to wait until this wave's
         # earlier stores are acknowledged; the output-tile values of a small wave tile are therefore kept in
@@ -280,7 +292,8 @@ class Codegen:
         defer = bool(tile_stores) and bool(row_reds or col_reds)
         e(f"constexpr bool DEFER = {'true' if defer else 'false'} && MI * NI <= 4;")
         for s_ in tile_stores:
-            e(f"[[maybe_unused]] float sv_{s_.slot}[DEFER ? MI : 1][16][NI];")
+            # kept in the storage type (rounded once, as a direct store would): half the registers for 16-bit outputs
+            e(f"[[maybe_unused]] typename evt::StorageRow<{DTYPE_CTYPES[ir.slots[s_.slot].dtype]}, NI>::type sv_{s_.slot}[DEFER ? MI : 1][16];")
         if any(r.kind == "welford" for r in row_reds):
             e("const float wcnt = (float)t.wave_cols();")
             e("const float wrcnt = wcnt > 0.f ? 1.f / wcnt : 0.f;")
@@ -306,7 +319,7 @@ class Codegen:
             e("const bool rok = t.row_ok(row);")
             for name in aux_nodes:
                 k = ir.nodes[name].slot
-                e(f"if constexpr (FAST) evt::row_load<Tile>(ub_{k} + (int64_t)Tile::row_step(mb + mo, v) * p.t{k}_sm, lo_{k}, "
+                e(f"if constexpr (FAST) evt::row_load<Tile>(rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mb + mo, v) * rp_{k}, "
                   f"rb_{_cname(name)}[mo][v]);")
                 e(f"else evt::aux_load<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
                   f"p.t{k}_sn, p.t{k}_vec, rok, rb_{_cname(name)}[mo][v]);")
@@ -338,7 +351,7 @@ class Codegen:
             else:
                 arr = _cname(src)
             e("if constexpr (DEFER) {")
-            e(f"  #pragma unroll\n  for (int ni = 0; ni < NI; ++ni) sv_{k}[mi][v][ni] = {arr}[ni];")
+            e(f"  #pragma unroll\n  for (int ni = 0; ni < NI; ++ni) sv_{k}[mi][v][ni] = evt::to_storage<{DTYPE_CTYPES[ir.slots[k].dtype]}>({arr}[ni]);")
             e("} else {")
             e.indent()
             self.emit_tile_store(e, k, arr)
@@ -368,9 +381,9 @@ class Codegen:
         e.dedent()
         e("}")
         if row_reds:
-            e("const bool row_last = evt::row_reduce_publish<Cfg, Epi>(p, t, g);")
+            e("const int row_ticket = evt::row_reduce_publish<Cfg, Epi>(p, t, g);")
         if col_reds:
-            e("const bool col_last = evt::col_reduce_publish<Cfg, Epi>(p, t, g, cst);")
+            e("const int col_ticket = evt::col_reduce_publish<Cfg, Epi>(p, t, g, cst);")
         if defer:
             e("if constexpr (DEFER) {")
             e.indent()
@@ -383,7 +396,9 @@ class Codegen:
             e("const int row = t.row(mi, v);")
             e("const bool rok = t.row_ok(row);")
             for s_ in tile_stores:
-                self.emit_tile_store(e, s_.slot, f"sv_{s_.slot}[mi][v]")
+                e(f"float dv_{s_.slot}[NI];")
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) dv_{s_.slot}[ni] = evt::from_storage(sv_{s_.slot}[mi][v][ni]);")
+                self.emit_tile_store(e, s_.slot, f"dv_{s_.slot}")
             e("(void)row; (void)rok;")
             e.dedent()
             e("}")
@@ -391,6 +406,11 @@ class Codegen:
             e("}")
             e.dedent()
             e("}")
+        # the deferred stores above travel while the arrival tickets do
+        if row_reds:
+            e("const bool row_last = evt::row_reduce_arrived<Cfg, Epi>(t, g, row_ticket);")
+        if col_reds:
+            e("const bool col_last = evt::col_reduce_arrived<Cfg, Epi>(t, g, col_ticket);")
         if row_reds:
             e("if (row_last) evt::row_reduce_complete<Cfg, Epi>(p, t, g);")
         if col_reds:
@@ -401,7 +421,7 @@ class Codegen:
 
     def emit_tile_store(self, e: _Emitter, k: int, arr: str):
         """Store the NI values `arr` of row (mi, v) to tile slot k (inside the row loops)."""
-        e(f"if constexpr (FAST) evt::row_store<Tile>(ub_{k} + (int64_t)Tile::row_step(mi, v) * p.t{k}_sm, lo_{k}, {arr});")
+        e(f"if constexpr (FAST) evt::row_store<Tile, {DTYPE_CTYPES[self.ir.slots[k].dtype]}>(rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mi, v) * rp_{k}, {arr});")
         e(f"else evt::aux_store<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
           f"p.t{k}_sn, p.t{k}_vec, rok, {arr});")
 
@@ -533,15 +553,12 @@ class Codegen:
         e.dedent()
         e("};")
         b = lambda x: "true" if x else "false"  # noqa: E731
+        tile_io = any((sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux") for sl in ir.slots)
         e(f"using Cfg = evt::GemmCfg<{t.bm}, {t.bn}, {t.bk}, {t.wm}, {t.wn}, {b(sp.a_kc)}, {b(sp.b_kc)}, "
-          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}, {t.pipe}>;")
+          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}, {t.pipe}, {b(tile_io)}>;")
         e(f"constexpr int kNumTensors = {len(ir.slots)};")
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
-        red_lds = 0
-        if ir.row_state:
-            red_lds += t.wn * t.bm * ir.row_state * 4 + 16
-        if ir.col_state:
-            red_lds += max(t.wm, max(1, t.wm * t.wn * 64 // t.bn)) * t.bn * ir.col_state * 4 + 16
+        red_lds = reduction_lds_bytes(t, ir.row_state, ir.col_state)
         e(f"static_assert(Cfg::LDS_BYTES >= {red_lds}, \"reduction exchange area exceeds the operand LDS\");")
         e("")
         e("// EVT_TWO_KERNEL_REDUCE=1 forces the separate finalize kernel for every cross-tile reduction")
@@ -648,8 +665,8 @@ class Codegen:
         tile_slots = [k for k, sl in enumerate(ir.slots)
                       if (sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux")]
         cond = " && ".join(
-            [f"(p.t{k}_vec & 1) && (!(Cfg::INTERLEAVE && sizeof(*p.t{k}) == 2 && (Cfg::NI == 2 || Cfg::NI == 4)) || (p.t{k}_vec & 2))"
-             f" && p.t{k}_sm >= 0 && p.t{k}_sm < (1 << 28)"
+            [f"(p.t{k}_vec & 1) && (!(Cfg::ADJACENT && sizeof(*p.t{k}) == 2 && (Cfg::NI == 2 || Cfg::NI == 4 || Cfg::NI == 8)) || (p.t{k}_vec & 2))"
+             f" && p.t{k}_sm >= 0 && p.t{k}_sm < (1 << 20)"
              for k in tile_slots]) or "true"
         e(f"p.fast = ({cond}) ? 1 : 0;")
         e("return EVT_OK;")

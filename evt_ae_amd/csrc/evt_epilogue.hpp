@@ -76,6 +76,17 @@ EVT_DEV void st_f32(T* p, int64_t off, float v) { p[off] = (T)v; }
 template <>
 EVT_DEV void st_f32<bool>(bool* p, int64_t off, float v) { p[off] = (v != 0.f); }
 
+// a value as its store would round it, and back (exact): what st_f32 writes for v equals what it writes for
+// from_storage(to_storage<T>(v))
+template <class T>
+EVT_DEV T to_storage(float v) { return (T)v; }
+template <>
+EVT_DEV bool to_storage<bool>(float v) { return v != 0.f; }
+template <class T>
+EVT_DEV float from_storage(T v) { return (float)v; }
+template <>
+EVT_DEV float from_storage<bool>(bool v) { return v ? 1.f : 0.f; }
+
 // ---------------------------------------------------------------------------
 // Where this lane's accumulator elements live in the output.
 // acc[mi][ni][v] is element (row(mi, v), col(ni)).
@@ -85,7 +96,7 @@ template <class Cfg, bool FULL_>
 struct TileCtx {
   static constexpr bool FULL = FULL_;
   static constexpr int MI = Cfg::MI, NI = Cfg::NI;
-  static constexpr bool INTERLEAVE = Cfg::INTERLEAVE;
+  static constexpr bool INTERLEAVE = Cfg::ADJACENT;   // this lane's NI columns are adjacent
   static constexpr int COL_STEP = INTERLEAVE ? 1 : 32;
   int M, N, L;
   int batch, tile_m, tile_n, tiles_m, tiles_n;
@@ -105,7 +116,9 @@ struct TileCtx {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     wm = wave / Cfg::WN; wn = wave % Cfg::WN;
     row_u = m0 + wm * Cfg::TM; row_l = 4 * (lane >> 5);
-    col_u = n0 + wn * Cfg::TN; col_l = INTERLEAVE ? (lane & 31) * NI : (lane & 31);
+    col_u = n0 + wn * Cfg::TN;
+    if constexpr (Cfg::REGROUP && NI == 2) col_l = 8 * ((lane & 31) >> 2) + ((lane & 1) << 2) + (lane & 2);   // see regroup_columns
+    else col_l = INTERLEAVE ? (lane & 31) * NI : (lane & 31);
     row0 = row_u + row_l;
     col0 = col_u + col_l;
     smem = smem_; workspace = g.workspace;
@@ -134,16 +147,22 @@ struct TileCtx {
 //          n (and aligned for the interleaved vector access): no bound checks,
 //          no flag tests -- straight-line code the scheduler can batch.
 //   else   `flags` bit 0: unit stride along n; bit 1: aligned so the NI
-//          adjacent elements of an interleaved lane move as one access.
+//          adjacent elements of an interleaved lane move as one access
+//          (4, 8 or 16 bytes for NI = 2, 4, 8 columns of a 16-bit type).
 template <bool FAST, class T, class Tile>
 EVT_DEV void aux_load(const Tile& t, const T* p, int64_t off, int64_t sn, int flags, bool rok,
                       T (&out)[Tile::NI]) {
   constexpr int NI = Tile::NI;
   const T* rp = p + off;
-  constexpr bool kVec = Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4);
+  constexpr bool kVec = Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4 || NI == 8);
   if constexpr (kVec) {
     if (FAST || ((flags & 2) && rok && t.col0 + NI <= t.N)) {
-      if constexpr (NI == 4) {
+      if constexpr (NI == 8) {
+        const u32x4 raw = *(const u32x4*)rp;
+        const T* e = (const T*)&raw;
+#pragma unroll
+        for (int ni = 0; ni < 8; ++ni) out[ni] = e[ni];
+      } else if constexpr (NI == 4) {
         const u32x2 raw = *(const u32x2*)rp;
         const T* e = (const T*)&raw;
 #pragma unroll
@@ -174,13 +193,15 @@ EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, 
                        const float (&val)[Tile::NI]) {
   constexpr int NI = Tile::NI;
   T* rp = p + off;
-  constexpr bool kVec = Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4);
+  constexpr bool kVec = Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4 || NI == 8);
   if constexpr (kVec) {
     if (FAST || ((flags & 2) && rok && t.col0 + NI <= t.N)) {
       T e[NI];
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) e[ni] = (T)val[ni];
-      if constexpr (NI == 4) {
+      if constexpr (NI == 8) {
+        *(u32x4*)rp = *(const u32x4*)e;
+      } else if constexpr (NI == 4) {
         *(u32x2*)rp = *(const u32x2*)e;
       } else {
         *(uint32_t*)rp = *(const uint32_t*)e;
@@ -202,43 +223,94 @@ EVT_DEV void aux_store(const Tile& t, T* p, int64_t off, int64_t sn, int flags, 
   }
 }
 
-// Check-free access to one accumulator row of a unit-stride tensor: `rowp` is
-// wave-uniform (a scalar-register pointer the compiler advances with scalar
-// arithmetic), `lo` is this lane's element offset inside the row, computed once
-// per tile -- no per-row 64-bit vector address arithmetic.
+// Check-free access to one accumulator row of a unit-stride tensor, through buffer instructions: `rs` is a
+// buffer resource whose base is this wave's corner of the tile (scalar registers), `voff` this lane's byte offset
+// inside a row (one register per tensor, the same for every row) and `soff` the row's byte offset from that corner
+// (scalar arithmetic) -- no per-row vector address arithmetic.  The bytes a lane moves per row: NI adjacent
+// 16-bit elements as one access of 4, 8 or 16 bytes, anything else element by element.
 template <class Tile, class T>
-EVT_DEV void row_load(const T* rowp, uint32_t lo, T (&out)[Tile::NI]) {
+constexpr bool row_is_vector() {
+  return Tile::INTERLEAVE && sizeof(T) == 2 && (Tile::NI == 2 || Tile::NI == 4 || Tile::NI == 8);
+}
+template <class T>
+EVT_DEV T buffer_load_elem(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+  if constexpr (sizeof(T) == 4) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(rs, voff, soff, 0));
+  else if constexpr (sizeof(T) == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b16(rs, voff, soff, 0));
+  else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b8(rs, voff, soff, 0));
+}
+template <class Tile, class T>
+EVT_DEV void row_load(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, T (&out)[Tile::NI]) {
   constexpr int NI = Tile::NI;
-  const char* base = (const char*)rowp;
-  if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && NI == 4) {
-    const u32x2 raw = *(const u32x2*)(base + lo * 2u);
+  if constexpr (row_is_vector<Tile, T>() && NI == 8) {
+    const u32x4 raw = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
+    const T* e = (const T*)&raw;
+#pragma unroll
+    for (int ni = 0; ni < 8; ++ni) out[ni] = e[ni];
+  } else if constexpr (row_is_vector<Tile, T>() && NI == 4) {
+    const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(rs, voff, soff, 0);
     const T* e = (const T*)&raw;
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) out[ni] = e[ni];
-  } else if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && NI == 2) {
-    const uint32_t raw = *(const uint32_t*)(base + lo * 2u);
+  } else if constexpr (row_is_vector<Tile, T>() && NI == 2) {
+    const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b32(rs, voff, soff, 0);
     const T* e = (const T*)&raw;
     out[0] = e[0]; out[1] = e[1];
   } else {
 #pragma unroll
-    for (int ni = 0; ni < NI; ++ni) out[ni] = *(const T*)(base + (lo + (uint32_t)(ni * Tile::COL_STEP)) * (uint32_t)sizeof(T));
+    for (int ni = 0; ni < NI; ++ni)
+      out[ni] = buffer_load_elem<T>(rs, voff + (uint32_t)(ni * Tile::COL_STEP * (int)sizeof(T)), soff);
   }
 }
 
+// NI elements of a 16-bit type in NI / 2 registers
+template <class T, int NI>
+struct PackOf {
+  typedef T type __attribute__((ext_vector_type(NI)));
+};
+// NI values of one row held in their storage type until a deferred store: a packed vector for 16-bit types with an
+// even count (two per register), a plain array otherwise; both are indexed [ni].
+template <class T, int NI, bool PACK = (sizeof(T) == 2 && NI % 2 == 0)>
+struct StorageRow {
+  struct type {
+    T e[NI];
+    EVT_DEV T& operator[](int i) { return e[i]; }
+    EVT_DEV const T& operator[](int i) const { return e[i]; }
+  };
+};
+template <class T, int NI>
+struct StorageRow<T, NI, true> {
+  typedef typename PackOf<T, NI>::type type;
+};
+
+// Output tiles are written once and not read again by this kernel: their stores carry the device-scope,
+// non-temporal cache policy (sc1 nt), which sends the data on to memory as it is written instead of leaving it
+// dirty in the L2 until the write-back at the end of the kernel -- the write then runs under the kernel's remaining
+// work instead of behind it (measured on the attention-score product: 15.1 -> 10.9 us per launch).
+constexpr int kStoreStreaming = 16 | 2;   // sc1 | nt
+template <class T>
+EVT_DEV void buffer_store_elem(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, float v) {
+  if constexpr (sizeof(T) == 4) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, (T)v), rs, voff, soff, kStoreStreaming);
+  } else if constexpr (sizeof(T) == 2) {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, (T)v), rs, voff, soff, kStoreStreaming);
+  } else {
+    __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(v != 0.f), rs, voff, soff, kStoreStreaming);   // bool
+  }
+}
 template <class Tile, class T>
-EVT_DEV void row_store(T* rowp, uint32_t lo, const float (&val)[Tile::NI]) {
+EVT_DEV void row_store(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, const float (&val)[Tile::NI]) {
   constexpr int NI = Tile::NI;
-  char* base = (char*)rowp;
-  if constexpr (Tile::INTERLEAVE && sizeof(T) == 2 && (NI == 2 || NI == 4)) {
+  if constexpr (row_is_vector<Tile, T>()) {
     T e[NI];
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) e[ni] = (T)val[ni];
-    if constexpr (NI == 4) *(u32x2*)(base + lo * 2u) = *(const u32x2*)e;
-    else *(uint32_t*)(base + lo * 2u) = *(const uint32_t*)e;
+    if constexpr (NI == 8) __builtin_amdgcn_raw_buffer_store_b128(*(const u32x4*)e, rs, voff, soff, kStoreStreaming);
+    else if constexpr (NI == 4) __builtin_amdgcn_raw_buffer_store_b64(*(const u32x2*)e, rs, voff, soff, kStoreStreaming);
+    else __builtin_amdgcn_raw_buffer_store_b32(*(const uint32_t*)e, rs, voff, soff, kStoreStreaming);
   } else {
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
-      st_f32<T>((T*)(base + (lo + (uint32_t)(ni * Tile::COL_STEP)) * (uint32_t)sizeof(T)), 0, val[ni]);
+      buffer_store_elem<T>(rs, voff + (uint32_t)(ni * Tile::COL_STEP * (int)sizeof(T)), soff, val[ni]);
   }
 }
 
@@ -312,37 +384,43 @@ EVT_DEV void rand8(uint64_t seed, uint32_t offset, uint32_t salt, int64_t e0, in
 // ---------------------------------------------------------------------------
 template <int STEP>
 EVT_DEV float half_wave_xchg(float x) {
+  static_assert(STEP >= 0 && STEP <= 3, "steps 0..3 stay inside a row of 16 lanes");
   const int xi = __builtin_bit_cast(int, x);
   int r;
   if constexpr (STEP == 0) r = __builtin_amdgcn_mov_dpp(xi, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
   else if constexpr (STEP == 1) r = __builtin_amdgcn_mov_dpp(xi, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
   else if constexpr (STEP == 2) r = __builtin_amdgcn_mov_dpp(xi, 0x141, 0xf, 0xf, true);  // row_half_mirror
-  else if constexpr (STEP == 3) r = __builtin_amdgcn_mov_dpp(xi, 0x140, 0xf, 0xf, true);  // row_mirror
-  else r = __builtin_amdgcn_ds_swizzle(xi, 0x401F);                                       // lane ^ 16
+  else r = __builtin_amdgcn_mov_dpp(xi, 0x140, 0xf, 0xf, true);                           // row_mirror
   return __builtin_bit_cast(float, r);
+}
+// Last step, between the two rows of 16 lanes of a half: v_permlane16_swap exchanges the odd rows of its first
+// operand with the even rows of its second, so with both equal to x the operands end up holding the even and the
+// odd row of each pair in every lane -- a VALU instruction, where ds_swizzle goes through the LDS crossbar and
+// costs its latency once per accumulator row.  (Written as assembly, with the two wait states the instruction
+// needs after a VALU write of its operands and before a VALU read of its results.)
+EVT_DEV void row_pair_split(float x, float& even_row, float& odd_row) {
+  even_row = x;
+  odd_row = x;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(even_row), "+v"(odd_row));
 }
 
 EVT_DEV float half_wave_sum(float x) {
-#ifdef EVT_ABLATE_ROWRED
-  return x;
-#endif
   x += half_wave_xchg<0>(x);
   x += half_wave_xchg<1>(x);
   x += half_wave_xchg<2>(x);
   x += half_wave_xchg<3>(x);
-  x += half_wave_xchg<4>(x);
-  return x;
+  float a, b;
+  row_pair_split(x, a, b);
+  return a + b;
 }
 EVT_DEV float half_wave_max(float x) {
-#ifdef EVT_ABLATE_ROWRED
-  return x;
-#endif
   x = fmaxf(x, half_wave_xchg<0>(x));
   x = fmaxf(x, half_wave_xchg<1>(x));
   x = fmaxf(x, half_wave_xchg<2>(x));
   x = fmaxf(x, half_wave_xchg<3>(x));
-  x = fmaxf(x, half_wave_xchg<4>(x));
-  return x;
+  float a, b;
+  row_pair_split(x, a, b);
+  return fmaxf(a, b);
 }
 
 // ---------------------------------------------------------------------------
@@ -426,40 +504,49 @@ EVT_DEV float ld_device(const float* p) {
   return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Count this workgroup in at `counter`; true (in every thread) for the
-// workgroup that arrives last of `expected`.  Every thread's partials were
-// stored with st_device before the call; the wait below lets them complete
-// before the ticket is taken, so the last arriver reads all of them.
-EVT_DEV bool arrive_last(int* counter, int expected, int* smem_flag) {
+// Count this workgroup in at `counter`.  Every thread's partials were stored
+// with st_device before the call; the wait below lets them complete before
+// the ticket is taken, so the workgroup that draws the last ticket reads all
+// of them.  In two halves, so that the caller can issue independent stores
+// while the ticket travels: arrive_begin returns the ticket (meaningful in
+// thread 0, -1 when the caller passed no counter), arrive_end tells every
+// thread whether this workgroup arrived last of `expected`.
+EVT_DEV int arrive_begin(int* counter) {
   __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0): my device-scope stores have been acknowledged
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    *smem_flag = ticket;
-  }
+  int ticket = -1;
+  if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return ticket;
+}
+EVT_DEV bool arrive_end(int ticket, int expected, int* smem_flag) {
+  if (threadIdx.x == 0) *smem_flag = ticket;
   __syncthreads();
   return *smem_flag == expected - 1;
 }
+EVT_DEV bool arrive_last(int* counter, int expected, int* smem_flag) {
+  return arrive_end(arrive_begin(counter), expected, smem_flag);
+}
 
-// Per-row reductions: combine the per-wave states left in LDS by the tile
-// visitor across the WN waves.  With one tile along N the result is final;
-// otherwise it is this tile's partial and phase 2 combines the partials in
-// tile order -- in the last workgroup of the row block to arrive (few tiles) or
-// in the finalize kernel (many tiles).
-//   LDS layout: state[wn][local_row][ROW_STATE] floats at smem, then one flag.
-// Phase 1 of a per-row reduction: combine the waves' row states in LDS and
-// either finalize (one tile spans the row) or publish this tile's partials.
-// Returns true when phase 2 runs in this kernel and this workgroup is the last
-// of its row block to arrive: it must then call row_reduce_complete.  Split in
-// two so the caller can issue its output-tile stores in between: the arrival
-// ticket has to wait for this wave's earlier stores to be acknowledged, and
-// 64 KB of tile stores in front of it cost microseconds.
+// Per-row reductions.  The tile visitor leaves one state per (wave column,
+// row) in LDS: state[wn][local_row][ROW_STATE] floats at smem, then one flag.
+// Phase 1 (row_reduce_publish): combine the WN waves' states; with one tile
+// along N the result is final, otherwise it is this tile's partial, written to
+// the workspace.  When phase 2 runs inside this kernel the workgroup also
+// draws its arrival ticket here.  The caller then issues its output-tile
+// stores (the ticket had to wait for this wave's earlier stores to be
+// acknowledged, and 64 KB of tile stores in front of it cost microseconds;
+// behind it they travel together with the ticket), asks row_reduce_arrived
+// whether it was the last workgroup of its row block and, if so, runs
+// row_reduce_complete.
+template <class Epi>
+EVT_DEV bool row_phase2_here(const GemmArgs& g) {
+  return Epi::ROW_STATE > 0 && row_uses_workspace(g) && g.row_inkernel;
+}
 template <class Cfg, class Epi, class Tile>
-EVT_DEV bool row_reduce_publish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
+EVT_DEV int row_reduce_publish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
   constexpr int RS = Epi::ROW_STATE;
   if constexpr (RS > 0) {
     const float* lds = (const float*)t.smem;
-    int* flag = (int*)(t.smem + Cfg::WN * Cfg::BM * RS * 4);
     const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     float* part = (float*)(t.workspace + wl.counter_bytes);
     __syncthreads();
@@ -479,39 +566,70 @@ EVT_DEV bool row_reduce_publish(const typename Epi::Params& p, const Tile& t, co
         for (int c = 0; c < RS; ++c) st_device(dst + c, st[c]);
       }
     }
-    if (!row_uses_workspace(g) || !g.row_inkernel) return false;
-    int* counter = (int*)t.workspace + fold_key(g, t.batch) * t.tiles_m + t.tile_m;
-    return arrive_last(counter, t.tiles_n * g.row_fold_count, flag);
+    if (!row_phase2_here<Epi>(g)) return -1;
+    return arrive_begin((int*)t.workspace + fold_key(g, t.batch) * t.tiles_m + t.tile_m);
+  } else {
+    return -1;
+  }
+}
+template <class Cfg, class Epi, class Tile>
+EVT_DEV bool row_reduce_arrived(const Tile& t, const GemmArgs& g, int ticket) {
+  if constexpr (Epi::ROW_STATE > 0) {
+    if (!row_phase2_here<Epi>(g)) return false;
+    return arrive_end(ticket, t.tiles_n * g.row_fold_count, (int*)(t.smem + Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4));
   } else {
     return false;
   }
 }
 
-// Phase 2 in the last workgroup of a row block: fold the partials in tile order.
+// Phase 2 in the last workgroup of a row block.  SHARES threads per row each
+// fold every SHARES-th partial (batches in fold order, tiles in tile order;
+// their loads are in flight together), then LDS combines the shares in order:
+// the combination tree depends on the problem and the tile only, so the result
+// is the same whichever workgroup arrives last.
 template <class Cfg, class Epi, class Tile>
 EVT_DEV void row_reduce_complete(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
   constexpr int RS = Epi::ROW_STATE;
   if constexpr (RS > 0) {
+    constexpr int SHARES = Cfg::THREADS >= Cfg::BM ? Cfg::THREADS / Cfg::BM : 1;
+    constexpr int ROWS_PER_PASS = Cfg::THREADS >= Cfg::BM ? Cfg::BM : Cfg::THREADS;
+    static_assert(SHARES * ROWS_PER_PASS * RS * 4 <= Cfg::LDS_BYTES, "share exchange area exceeds the operand LDS");
+    float* lds = (float*)t.smem;
     const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     const float* part = (const float*)(t.workspace + wl.counter_bytes);
     const int key = fold_key(g, t.batch);
     int* counter = (int*)t.workspace + key * t.tiles_m + t.tile_m;
-    for (int lr = t.tid; lr < Cfg::BM; lr += Cfg::THREADS) {
+    const int share = t.tid / ROWS_PER_PASS, lr0 = t.tid % ROWS_PER_PASS;
+    const int nq = t.tiles_n * g.row_fold_count;
+    for (int base = 0; base < Cfg::BM; base += ROWS_PER_PASS) {
+      const int lr = base + lr0;
       const int row = t.m0 + lr;
-      if (row >= t.M) continue;
+      const bool live = share < SHARES && lr < Cfg::BM && row < t.M;
       float st[RS];
       Epi::row_identity(st);
-      // batches in fold order, tiles in tile order: the same sum whichever workgroup arrives last
-      for (int f = 0; f < g.row_fold_count; ++f) {
-        const float* src = part + ((int64_t)fold_member(g, key, f) * t.tiles_n * t.M + row) * RS;
-        for (int j = 0; j < t.tiles_n; ++j) {
+      if (live) {
+#pragma unroll 4
+        for (int q = share; q < nq; q += SHARES) {
+          const int f = q / t.tiles_n, j = q - f * t.tiles_n;
+          const float* src = part + (((int64_t)fold_member(g, key, f) * t.tiles_n + j) * t.M + row) * RS;
           float o[RS];
 #pragma unroll
-          for (int c = 0; c < RS; ++c) o[c] = ld_device(src + (int64_t)j * t.M * RS + c);
+          for (int c = 0; c < RS; ++c) o[c] = ld_device(src + c);
           Epi::row_combine(st, o);
         }
       }
-      Epi::row_finalize(p, fold_member(g, key, 0), row, st);
+      if constexpr (SHARES > 1) {
+        __syncthreads();   // the exchange area is free (phase-1 states / the previous pass have been consumed)
+        if (share < SHARES) {
+#pragma unroll
+          for (int c = 0; c < RS; ++c) lds[(share * ROWS_PER_PASS + lr0) * RS + c] = st[c];
+        }
+        __syncthreads();
+        if (live && share == 0) {
+          for (int s2 = 1; s2 < SHARES; ++s2) Epi::row_combine(st, lds + (s2 * ROWS_PER_PASS + lr0) * RS);
+        }
+      }
+      if (live && share == 0) Epi::row_finalize(p, fold_member(g, key, 0), row, st);
     }
     if (t.tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -520,16 +638,24 @@ EVT_DEV void row_reduce_complete(const typename Epi::Params& p, const Tile& t, c
 
 // Per-column reductions.  `cs[ni][c]` holds this lane's state for column
 // col(ni) over all its rows.  LDS layout: state[wm][local_col][COL_STATE]
-// floats placed after the row-reduction area, then one flag.
+// floats placed after the row-reduction area, then one flag.  Same three steps
+// as for rows: publish (+ ticket), arrived, complete.
+template <class Epi>
+EVT_DEV bool col_phase2_here(const GemmArgs& g) {
+  return Epi::COL_STATE > 0 && col_uses_workspace(g) && g.col_inkernel;
+}
+template <class Cfg, class Epi>
+struct ColArea {
+  static constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
+  static constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
+  static constexpr int FLAG = ROW_AREA + (Cfg::WM > SHARES ? Cfg::WM : SHARES) * Cfg::BN * (Epi::COL_STATE > 0 ? Epi::COL_STATE : 1) * 4;
+};
 template <class Cfg, class Epi, class Tile>
-EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g,
+EVT_DEV int col_reduce_publish(const typename Epi::Params& p, const Tile& t, const GemmArgs& g,
                                float (&cs)[Tile::NI][Epi::COL_STATE > 0 ? Epi::COL_STATE : 1]) {
   constexpr int CS = Epi::COL_STATE;
   if constexpr (CS > 0) {
-    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
-    constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
-    float* lds = (float*)(t.smem + ROW_AREA);
-    int* flag = (int*)(t.smem + ROW_AREA + (Cfg::WM > SHARES ? Cfg::WM : SHARES) * Cfg::BN * CS * 4);
+    float* lds = (float*)(t.smem + ColArea<Cfg, Epi>::ROW_AREA);
     // the two halves of a wave hold different rows of the same columns
 #pragma unroll
     for (int ni = 0; ni < Tile::NI; ++ni) {
@@ -563,10 +689,18 @@ EVT_DEV bool col_reduce_publish(const typename Epi::Params& p, const Tile& t, co
         for (int c = 0; c < CS; ++c) st_device(dst + c, st[c]);
       }
     }
-    if (!col_uses_workspace(g) || !g.col_inkernel) return false;
+    if (!col_phase2_here<Epi>(g)) return -1;
     const int row_counters = (Epi::ROW_STATE > 0 && row_uses_workspace(g)) ? t.L * t.tiles_m : 0;
-    int* counter = (int*)t.workspace + row_counters + col_fold_key(g, t.batch) * t.tiles_n + t.tile_n;
-    return arrive_last(counter, t.tiles_m * g.col_fold_count, flag);
+    return arrive_begin((int*)t.workspace + row_counters + col_fold_key(g, t.batch) * t.tiles_n + t.tile_n);
+  } else {
+    return -1;
+  }
+}
+template <class Cfg, class Epi, class Tile>
+EVT_DEV bool col_reduce_arrived(const Tile& t, const GemmArgs& g, int ticket) {
+  if constexpr (Epi::COL_STATE > 0) {
+    if (!col_phase2_here<Epi>(g)) return false;
+    return arrive_end(ticket, t.tiles_m * g.col_fold_count, (int*)(t.smem + ColArea<Cfg, Epi>::FLAG));
   } else {
     return false;
   }
@@ -577,9 +711,8 @@ template <class Cfg, class Epi, class Tile>
 EVT_DEV void col_reduce_complete(const typename Epi::Params& p, const Tile& t, const GemmArgs& g) {
   constexpr int CS = Epi::COL_STATE;
   if constexpr (CS > 0) {
-    constexpr int ROW_AREA = Epi::ROW_STATE > 0 ? (Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4 + 16) : 0;
-    constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
-    float* lds = (float*)(t.smem + ROW_AREA);
+    constexpr int SHARES = ColArea<Cfg, Epi>::SHARES;
+    float* lds = (float*)(t.smem + ColArea<Cfg, Epi>::ROW_AREA);
     const WsLayout wl = ws_layout<Epi::ROW_STATE, Epi::COL_STATE>(g);
     const float* part = (const float*)(t.workspace + wl.counter_bytes + wl.row_bytes);
     const int row_counters = (Epi::ROW_STATE > 0 && row_uses_workspace(g)) ? t.L * t.tiles_m : 0;
@@ -748,9 +881,7 @@ EVT_DEV void combine_welford(float& n, float& mean, float& m2, float nb, float m
   n = nt;
 }
 
-// The fused kernel.  Interior tiles whose epilogue tensors are all unit-stride
-// (p.fast, decided on the host) take the check-free epilogue; everything else
-// takes the guarded one.
+// The fused kernel.
 #ifdef EVT_CLOCK_PROBE
 // Diagnostic build only: {main-loop shader cycles, main-loop 100 MHz ticks,
 // epilogue shader cycles, epilogue 100 MHz ticks} of workgroup 0.  The ratio
@@ -807,9 +938,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, type
     __syncthreads();
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch
   }
+  regroup_columns<Cfg>(acc);
 #ifdef EVT_CLOCK_PROBE
   const uint64_t probe_c1 = __builtin_amdgcn_s_memtime(), probe_r1 = __builtin_amdgcn_s_memrealtime();
 #endif
+  // interior tiles of an all-unit-stride epilogue (p.fast, decided on the host) take the check-free epilogue
   if (p.fast && (tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
     TileCtx<Cfg, true> t;
     t.init(g, batch, tm, tn, smem);

@@ -75,8 +75,9 @@ struct GemmArgs {
 };
 
 // Compile-time description of one kernel variant.
+//   TILE_IO_  the epilogue reads or writes full tensors: worth giving every lane adjacent output columns
 template <int BM_, int BN_, int BK_, int WM_, int WN_, bool A_KC_, bool B_KC_,
-          bool DMA_, int STAGES_, bool BF16_, int GROUP_M_, int PIPE_ = 0>
+          bool DMA_, int STAGES_, bool BF16_, int GROUP_M_, int PIPE_ = 0, bool TILE_IO_ = true>
 struct GemmCfg {
   // PIPE 0: ring of STAGES tiles, fragments fetched inside each k-tile.
   // PIPE 1: look-ahead ring (STAGES >= 3): tile kt+1 is made visible one
@@ -91,8 +92,17 @@ struct GemmCfg {
   // PIPE 3: ping-pong with one barrier per k-tile: the barrier between a
   //         group's read phase and its MFMA phase is dropped and wave
   //         priorities keep the two waves of a SIMD out of step.
+  // PIPE 4 + flags: PIPE 3 with options (Mainloop::PP_*):
+  //         1  group 0 meets the k-tile barrier inside its MFMA phase, a
+  //            quarter of its MFMAs still to issue, so the matrix pipe has work
+  //            while the barrier resolves and group 1 starts;
+  //         2  group 0 issues its global->LDS transfers between the LDS reads
+  //            of its read phase instead of between its MFMAs (with two stages:
+  //            instead of in one burst in front of the reads);
+  //         4  group 1 does the same (STAGES >= 3).
   static constexpr int PIPE = PIPE_;
-  static constexpr bool PINGPONG = PIPE_ == 2 || PIPE_ == 3;
+  static constexpr bool PINGPONG = PIPE_ >= 2;
+  static constexpr int PP_FLAGS = PIPE_ >= 4 ? PIPE_ - 4 : 0;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DMA = DMA_, BF16 = BF16_;
   static constexpr int STAGES = STAGES_, GROUP_M = GROUP_M_;
@@ -107,6 +117,12 @@ struct GemmCfg {
   // With a K-contiguous B tile the rows (= output columns) can be permuted for
   // free while loading, so every lane ends up owning NI adjacent columns.
   static constexpr bool INTERLEAVE = B_LDS_KC && (NI > 1);
+  // With a k-row B tile the transposing LDS read hands lane j column j of each 32-column block.  The blocks are
+  // then laid over the wave's columns in 4-column pieces (piece p of block f covers columns 4 (p NI + f) ...), and
+  // after the main loop the four lanes of a quad exchange accumulators so that every lane again owns NI adjacent
+  // columns (regroup_columns): the epilogue's vector accesses work for either operand layout.
+  static constexpr bool REGROUP = TILE_IO_ && !B_LDS_KC && (NI == 2 || NI == 4);
+  static constexpr bool ADJACENT = INTERLEAVE || REGROUP;   // a lane's NI columns are adjacent in the output
   static constexpr int A_BYTES = BM * BK * 2;
   static constexpr int B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
@@ -116,7 +132,8 @@ struct GemmCfg {
   static_assert(STAGES >= 1 && STAGES <= 8, "1..8 stages");
   static_assert(PIPE != 1 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
   static_assert(!PINGPONG || (DMA && STAGES >= 2 && WM * WN == 8), "ping-pong needs DMA, >= 2 stages, 8 waves");
-  static_assert(PIPE >= 0 && PIPE <= 3, "unknown pipeline");
+  static_assert(PIPE >= 0 && PIPE <= 11, "unknown pipeline");
+  static_assert(!(PP_FLAGS & 4) || STAGES >= 3, "group 1 can only issue in its read phase with three or more stages");
 };
 
 // ---------------------------------------------------------------------------
@@ -298,7 +315,9 @@ EVT_DEV void lds_pin(T& x) { asm volatile("" : "+v"(x)); }
 EVT_DEV uint32_t lds_addr(const char* p) { return (uint32_t)(uintptr_t)p; }
 
 // Per-lane LDS read addressing of MFMA operand fragments (32 rows x 16 k).
-template <int ROWS, int BK, bool LDS_KC, int NFRAG>
+//   PIECES  (k-row tiles only) > 0: fragment f takes its 32 rows in 8 pieces of 4, piece p = rows
+//           4 (p PIECES + f) ... of the wave's slice (GemmCfg::REGROUP); 0: rows 32 f ...
+template <int ROWS, int BK, bool LDS_KC, int NFRAG, int PIECES = 0>
 struct FragReader {
   static constexpr int CH = BK / 8;
   static constexpr int RC = ROWS / 8;
@@ -314,10 +333,10 @@ struct FragReader {
       // transposing read: each group of 16 lanes covers 4 k-rows x 16 rows
       const int u = lane >> 4, s = lane & 15;
       const int kl = 8 * (u >> 1) + (s >> 2);
-      const int i0 = wave_row_base + 16 * (u & 1) + 4 * (s & 3);
+      const int i0 = wave_row_base + (PIECES > 0 ? ((u & 1) * 4 + (s & 3)) * 4 * PIECES : 16 * (u & 1) + 4 * (s & 3));
 #pragma unroll
       for (int f = 0; f < NFRAG; ++f) {
-        const int i = i0 + f * 32;
+        const int i = i0 + f * (PIECES > 0 ? 4 : 32);
         off[f] = (kl * RC + ((i >> 3) ^ nc_swz<RC>(kl))) * 16 + (i & 7) * 2;
       }
     }
@@ -345,20 +364,20 @@ struct FragReader {
     u32x4 q[LDS_KC ? KSN * NFRAG : 1];
     u32x2 h[LDS_KC ? 1 : 2 * KSN * NFRAG];
   };
+  // number of LDS read instructions of one k-tile, and read number i of them (k-sub-step major)
+  static constexpr int NREADS = LDS_KC ? KSN * NFRAG : 2 * KSN * NFRAG;
+  EVT_DEV void issue_one(uint32_t lds, Tile& t, int i) const {
+    if constexpr (LDS_KC) {
+      const int ks = i / NFRAG, f = i % NFRAG;
+      t.q[i] = lds_read_b128(lds + off[ks] + f * (32 * CH * 16));
+    } else {
+      const int pr = i >> 1, ks = pr / NFRAG, f = pr % NFRAG;
+      t.h[i] = lds_read_tr16_b64(lds + off[f] + ks * (16 * RC * 16) + (i & 1) * (4 * RC * 16));
+    }
+  }
   EVT_DEV void issue(uint32_t lds, Tile& t) const {
 #pragma unroll
-    for (int ks = 0; ks < KSN; ++ks) {
-#pragma unroll
-      for (int f = 0; f < NFRAG; ++f) {
-        if constexpr (LDS_KC) {
-          t.q[ks * NFRAG + f] = lds_read_b128(lds + off[ks] + f * (32 * CH * 16));
-        } else {
-          const uint32_t p = lds + off[f] + ks * (16 * RC * 16);
-          t.h[2 * (ks * NFRAG + f)] = lds_read_tr16_b64(p);
-          t.h[2 * (ks * NFRAG + f) + 1] = lds_read_tr16_b64(p + 4 * RC * 16);
-        }
-      }
-    }
+    for (int i = 0; i < NREADS; ++i) issue_one(lds, t, i);
   }
   EVT_DEV void pin(Tile& t) const {
     if constexpr (LDS_KC) {
@@ -414,6 +433,46 @@ EVT_DEV void tile_coords(int pid, int nblocks, int tiles_m, int tiles_n, int& ba
   tn = in / gm;
 }
 
+// GemmCfg::REGROUP: lane c of a quad holds column c of NI four-column pieces (piece f in acc[.][f]); afterwards
+// it holds NI adjacent columns in acc[.][0 .. NI-1].  NI = 4: a 4 x 4 transpose inside the quad, lane c ends up
+// with piece c.  NI = 2: one exchange with the neighbouring lane; even lanes end up with columns c, c + 1 of piece
+// 0, odd lanes with columns c - 1, c of piece 1 (TileCtx::init has the matching column offsets).
+EVT_DEV float quad_xchg1(float x) {   // value of lane ^ 1
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xf, 0xf, true));
+}
+EVT_DEV float quad_xchg2(float x) {   // value of lane ^ 2
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x4E, 0xf, 0xf, true));
+}
+template <class Cfg>
+EVT_DEV void regroup_columns(f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  if constexpr (Cfg::REGROUP) {
+    const int lane = threadIdx.x & 63;
+    const bool b0 = lane & 1, b1 = lane & 2;
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+#pragma unroll
+        for (int f = 0; f < Cfg::NI; f += 2) {   // 2 x 2 transposes between lanes c, c ^ 1 on pieces (f, f + 1)
+          const float e0 = acc[mi][f][v], e1 = acc[mi][f + 1][v];
+          const float got = quad_xchg1(b0 ? e0 : e1);
+          acc[mi][f][v] = b0 ? got : e0;
+          acc[mi][f + 1][v] = b0 ? e1 : got;
+        }
+        if constexpr (Cfg::NI == 4) {            // and between lanes c, c ^ 2 on pieces (f, f + 2)
+#pragma unroll
+          for (int f = 0; f < 2; ++f) {
+            const float e0 = acc[mi][f][v], e1 = acc[mi][f + 2][v];
+            const float got = quad_xchg2(b1 ? e0 : e1);
+            acc[mi][f][v] = b1 ? got : e0;
+            acc[mi][f + 2][v] = b1 ? e1 : got;
+          }
+        }
+      }
+    }
+  }
+}
+
 // The main loop: acc[mi][ni] += A_tile * B_tile over all k-tiles.
 template <class Cfg>
 struct Mainloop {
@@ -421,7 +480,7 @@ struct Mainloop {
   using OpB = Operand<Cfg::BN, Cfg::BK, Cfg::B_KC, Cfg::DMA, Cfg::THREADS,
                       Cfg::INTERLEAVE ? Cfg::NI : 0, Cfg::TN>;
   using RdA = FragReader<Cfg::BM, Cfg::BK, Cfg::A_LDS_KC, Cfg::MI>;
-  using RdB = FragReader<Cfg::BN, Cfg::BK, Cfg::B_LDS_KC, Cfg::NI>;
+  using RdB = FragReader<Cfg::BN, Cfg::BK, Cfg::B_LDS_KC, Cfg::NI, Cfg::REGROUP ? Cfg::NI : 0>;
   static constexpr int LPS = OpA::NLOAD + OpB::NLOAD;   // DMA ops per thread per stage
 
   // One k-tile: KS sub-steps of MI x NI MFMAs.  Fragments of sub-step ks+1
@@ -432,28 +491,19 @@ struct Mainloop {
     const char* la = lds;
     const char* lb = lds + Cfg::A_BYTES;
     u32x4 af[2][Cfg::MI], bf[2][Cfg::NI];
-#ifndef EVT_ABLATE_LDS_READ
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi) af[0][mi] = ra.read(la, mi, 0);
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni) bf[0][ni] = rb.read(lb, ni, 0);
-#else
-#pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi) af[0][mi] = af[1][mi] = u32x4{(uint32_t)threadIdx.x, 1u, 2u, 3u};
-#pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni) bf[0][ni] = bf[1][ni] = u32x4{5u, (uint32_t)threadIdx.x, 7u, 8u};
-#endif
 #pragma unroll
     for (int ks = 0; ks < Cfg::KS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-#ifndef EVT_ABLATE_LDS_READ
       if (ks + 1 < Cfg::KS) {
 #pragma unroll
         for (int mi = 0; mi < Cfg::MI; ++mi) af[nxt][mi] = ra.read(la, mi, ks + 1);
 #pragma unroll
         for (int ni = 0; ni < Cfg::NI; ++ni) bf[nxt][ni] = rb.read(lb, ni, ks + 1);
       }
-#endif
 #pragma unroll
       for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
@@ -611,50 +661,79 @@ struct Mainloop {
     typename RdB::Tile b;
   };
   static constexpr int PP_NM = Cfg::KS * Cfg::MI * Cfg::NI;   // MFMAs per C phase
-  static constexpr bool PP_G0_ISSUES_IN_C = Cfg::STAGES >= 3;
-  // R phase: all fragments of the tile at `lds` are in registers on return
-  static EVT_DEV void pp_read(TileFrags& f, const char* lds, const RdA& ra, const RdB& rb) {
-    ra.issue(lds_addr(lds), f.a);
-    rb.issue(lds_addr(lds + Cfg::A_BYTES), f.b);
-    lds_wait_all();
-    ra.pin(f.a);
-    rb.pin(f.b);
-  }
-  // transfer c (of LPS) goes behind MFMA number (c * PP_NM) / LPS
-  template <int M>
-  static EVT_DEV void pp_pin_order() {
-    if constexpr (M < PP_NM) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      constexpr int n = ((M + 1) * LPS + PP_NM - 1) / PP_NM - (M * LPS + PP_NM - 1) / PP_NM;
-      if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x020, n, 0);
-      pp_pin_order<M + 1>();
-    }
-  }
-  // C phase; with ISSUE the transfers of k-tile `nk` into stage `ds` are spread between the MFMAs
-  template <bool ISSUE, int PRIO = 1>
-  static EVT_DEV void pp_mma(const TileFrags& f, const RdA& ra, const RdB& rb, f32x16 (&acc)[Cfg::MI][Cfg::NI],
-                             const OpA& a, const OpB& b, int nk, char* ds, int wave) {
+  static constexpr bool PP_MIDC = (Cfg::PP_FLAGS & 1) != 0;
+  static constexpr bool PP_G0_IN_R = (Cfg::PP_FLAGS & 2) != 0;
+  static constexpr bool PP_G1_IN_R = (Cfg::PP_FLAGS & 4) != 0;
+  static constexpr bool PP_G0_IN_C = !PP_G0_IN_R && Cfg::STAGES >= 3;
+  static constexpr int PP_REST = PP_MIDC ? (PP_NM / 4 > 0 ? PP_NM / 4 : 1) : 0;   // group 0's MFMAs behind the barrier
+  static constexpr int PP_NR = RdA::NREADS + RdB::NREADS;   // LDS reads per R phase
+  // R phase: all fragments of the tile at `lds` are in registers on return.  With ISSUE the transfers of
+  // k-tile `nk` into stage `ds` go between the reads (transfer c behind read number (c * PP_NR) / LPS): a wave
+  // that waits for LDS anyway absorbs the pacing of the texture path, and the MFMA phases stay pure.
+  template <bool ISSUE>
+  static EVT_DEV void pp_read(TileFrags& f, const char* lds, const RdA& ra, const RdB& rb,
+                              const OpA& a, const OpB& b, int nk, char* ds, int wave) {
     typename OpA::DmaTile da;
     typename OpB::DmaTile db;
     if constexpr (ISSUE) {
       da = a.dma_begin(nk);
       db = b.dma_begin(nk);
     }
-#ifndef EVT_NO_SETPRIO
+    const uint32_t la = lds_addr(lds), lb = lds_addr(lds + Cfg::A_BYTES);
+#pragma unroll
+    for (int i = 0; i < PP_NR; ++i) {
+      if (i < RdA::NREADS) ra.issue_one(la, f.a, i);
+      else rb.issue_one(lb, f.b, i - RdA::NREADS);
+      if constexpr (ISSUE) {
+#pragma unroll
+        for (int c = 0; c < LPS; ++c) {
+          if ((c * PP_NR) / LPS == i) {
+            if (c < OpA::NLOAD) a.dma_chunk(da, ds, wave, c);
+            else b.dma_chunk(db, ds + Cfg::A_BYTES, wave, c - OpA::NLOAD);
+          }
+        }
+      }
+    }
+    lds_wait_all();
+    ra.pin(f.a);
+    rb.pin(f.b);
+  }
+  // MFMAs [M, MEND) of a C phase, transfer c (of LPS) behind MFMA number (c * SPREAD) / LPS
+  template <int M, int MEND, int SPREAD>
+  static EVT_DEV void pp_pin_order() {
+    if constexpr (M < MEND) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      constexpr int n = ((M + 1) * LPS + SPREAD - 1) / SPREAD - (M * LPS + SPREAD - 1) / SPREAD;
+      if constexpr (n > 0 && M < SPREAD) __builtin_amdgcn_sched_group_barrier(0x020, n, 0);
+      pp_pin_order<M + 1, MEND, SPREAD>();
+    }
+  }
+  // MFMAs [M0, M1) of the C phase (numbered k-sub-step major); with ISSUE the transfers of k-tile `nk` into
+  // stage `ds` are spread between them
+  template <bool ISSUE, int PRIO, int M0, int M1>
+  static EVT_DEV void pp_mma(const TileFrags& f, const RdA& ra, const RdB& rb, f32x16 (&acc)[Cfg::MI][Cfg::NI],
+                             const OpA& a, const OpB& b, int nk, char* ds, int wave) {
+    static_assert(!ISSUE || M0 == 0, "transfers are spread from the first MFMA on");
+    typename OpA::DmaTile da;
+    typename OpB::DmaTile db;
+    if constexpr (ISSUE) {
+      da = a.dma_begin(nk);
+      db = b.dma_begin(nk);
+    }
     __builtin_amdgcn_s_setprio(PRIO);
-#endif
 #pragma unroll
     for (int ks = 0; ks < Cfg::KS; ++ks) {
 #pragma unroll
       for (int mi = 0; mi < Cfg::MI; ++mi) {
 #pragma unroll
         for (int ni = 0; ni < Cfg::NI; ++ni) {
+          const int m = (ks * Cfg::MI + mi) * Cfg::NI + ni;
+          if (m < M0 || m >= M1) continue;
           acc[mi][ni] = mfma32<Cfg::BF16>(ra.frag(f.a, mi, ks), rb.frag(f.b, ni, ks), acc[mi][ni]);
           if constexpr (ISSUE) {
-            const int m = (ks * Cfg::MI + mi) * Cfg::NI + ni;
 #pragma unroll
             for (int c = 0; c < LPS; ++c) {
-              if ((c * PP_NM) / LPS == m) {
+              if ((c * M1) / LPS == m) {
                 if (c < OpA::NLOAD) a.dma_chunk(da, ds, wave, c);
                 else b.dma_chunk(db, ds + Cfg::A_BYTES, wave, c - OpA::NLOAD);
               }
@@ -663,10 +742,8 @@ struct Mainloop {
         }
       }
     }
-    if constexpr (ISSUE) pp_pin_order<0>();
-#ifndef EVT_NO_SETPRIO
+    if constexpr (ISSUE) pp_pin_order<M0, M1, M1>();
     __builtin_amdgcn_s_setprio(0);
-#endif
   }
   // Transfers are issued for every T, also past the last k-tile: a tile index
   // beyond K reads as zeros through the buffer range check (no memory traffic)
@@ -702,25 +779,28 @@ struct Mainloop {
     const int grp = wave >> 2;
     if (grp == 0) {
       for (int T = 0; T < KT; ++T) {
-        if constexpr (!PP_G0_ISSUES_IN_C) pp_issue(T, stage, a, b, smem, wave);
-        pp_read(f, smem + stage * Cfg::STAGE_BYTES, ra, rb);
+        char* ds = pp_refill_stage(stage, smem);
+        if constexpr (!PP_G0_IN_C && !PP_G0_IN_R) pp_issue(T, stage, a, b, smem, wave);
+        pp_read<PP_G0_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, T + S - 1, ds, wave);
         if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
-        pp_mma<PP_G0_ISSUES_IN_C>(f, ra, rb, acc, a, b, T + S - 1, pp_refill_stage(stage, smem), wave);
+        pp_mma<PP_G0_IN_C, 1, 0, PP_NM - PP_REST>(f, ra, rb, acc, a, b, T + S - 1, ds, wave);
         wait_tiles<S - 2>();        // my share of tile T+1 has landed
         pp_barrier();               // ends phase 2T+1
+        if constexpr (PP_REST > 0) pp_mma<false, 3, PP_NM - PP_REST, PP_NM>(f, ra, rb, acc, a, b, 0, ds, wave);
         stage = stage + 1 == S ? 0 : stage + 1;
       }
     } else {
-      pp_issue(0, 0, a, b, smem, wave);
+      if constexpr (!PP_G1_IN_R) pp_issue(0, 0, a, b, smem, wave);
       for (int T = 0; T < KT; ++T) {
-        if (T > 0) pp_mma<true, 2>(f, ra, rb, acc, a, b, T + S - 1, pp_refill_stage(stage, smem), wave);   // C(T-1)
+        char* ds = pp_refill_stage(stage, smem);
+        if (T > 0) pp_mma<!PP_G1_IN_R, 2, 0, PP_NM>(f, ra, rb, acc, a, b, T + S - 1, ds, wave);   // C(T-1)
         if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
-        pp_read(f, smem + stage * Cfg::STAGE_BYTES, ra, rb);
+        pp_read<PP_G1_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, T + S - 1, ds, wave);
         wait_tiles<S - 2>();        // my share of tile T+1 has landed
         pp_barrier();               // ends phase 2T+1
         stage = stage + 1 == S ? 0 : stage + 1;
       }
-      if (KT > 0) pp_mma<false>(f, ra, rb, acc, a, b, 0, smem, wave);   // C(KT-1)
+      if (KT > 0) pp_mma<false, 2, 0, PP_NM>(f, ra, rb, acc, a, b, 0, smem, wave);   // C(KT-1)
     }
     wait_vmcnt<0>();                // the zero-fill transfers past the last tile have landed
   }
@@ -788,17 +868,13 @@ struct Mainloop {
         } else {
           wait_vmcnt<0>();
         }
-#ifndef EVT_ABLATE_BARRIER
         __syncthreads();   // tile kt visible to all waves; everyone left tile kt-1
-#endif
         const int nk = kt + Cfg::STAGES - 1;
         if (nk < KT) {
           int ns = stage + Cfg::STAGES - 1;
           if (ns >= Cfg::STAGES) ns -= Cfg::STAGES;
-#ifndef EVT_ABLATE_DMA
           a.dma(nk, smem + ns * Cfg::STAGE_BYTES, wave);
           b.dma(nk, smem + ns * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
-#endif
         }
         compute(smem + stage * Cfg::STAGE_BYTES, ra, rb, acc);
         stage = (stage + 1 == Cfg::STAGES) ? 0 : stage + 1;
