@@ -60,6 +60,8 @@ def reduction_lds_bytes(t: "TileConfig", row_state: int, col_state: int) -> int:
         need += t.wn * t.bm * row_state * 4 + 16
     if col_state:
         need += max(t.wm, max(1, t.wm * t.wn * 64 // t.bn)) * t.bn * col_state * 4 + 16
+    if row_state:   # + per wave and half one float per row: a row's first-pass result on its way back to its lanes
+        need = (need + 15) // 16 * 16 + t.wm * t.wn * 2 * (t.bm // t.wm // 2) * 4
     return max(need, t.wm * t.wn * 64 * row_state * 4)
 
 
@@ -294,9 +296,19 @@ class Codegen:
         for s_ in tile_stores:
             # kept in the storage type (rounded once, as a direct store would): half the registers for 16-bit outputs
             e(f"[[maybe_unused]] typename evt::StorageRow<{DTYPE_CTYPES[ir.slots[s_.slot].dtype]}, NI>::type sv_{s_.slot}[DEFER ? MI : 1][16];")
+        # per-row reductions work on all rows of the wave tile at once (evt::rows_*): the loops below only collect
+        # the values
+        # With one 32-row block per wave (MI = 1) each row is reduced as it is produced (ROW_BY_ROW), which runs under
+        # the row's stores; larger wave tiles collect the values and reduce all rows together afterwards
+        e("constexpr bool ROW_BY_ROW = MI == 1;")
+        for r in row_reds:
+            if r.kind in ("sum", "max"):
+                e(f"[[maybe_unused]] float rp_{_cname(r.name)}[16 * MI];")
+            else:
+                e(f"[[maybe_unused]] float rx_{_cname(r.name)}[ROW_BY_ROW ? 1 : 16 * MI][NI];")
         if any(r.kind == "welford" for r in row_reds):
-            e("const float wcnt = (float)t.wave_cols();")
-            e("const float wrcnt = wcnt > 0.f ? 1.f / wcnt : 0.f;")
+            e("[[maybe_unused]] const float wcnt = (float)t.wave_cols();")
+            e("[[maybe_unused]] const float wrcnt = wcnt > 0.f ? 1.f / wcnt : 0.f;")
         # rows are processed in batches of MB x 16: the full-tensor loads of a batch are all issued before its
         # arithmetic and stores (loads do not move above stores by themselves), so a batch costs one round trip
         # to HBM; two 32-row blocks per batch keep the staging registers bounded on the largest wave tiles
@@ -358,10 +370,26 @@ class Codegen:
             e.dedent()
             e("}")
         if row_reds:
+            e("if constexpr (ROW_BY_ROW) {")
+            e.indent()
             e(f"float rst[{ir.row_state}];")
             for r in row_reds:
                 self.emit_row_reduce(e, r)
             e(f"evt::row_state_to_lds<Cfg, {ir.row_state}>(t, mi, v, rst);")
+            e.dedent()
+            e("} else {")
+            e.indent()
+        for r in row_reds:
+            c, x = _cname(r.name), self.ref(r.input)
+            if r.kind == "sum":
+                e(f"{{ float a = 0.f;\n#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) a += t.col_ok(ni) ? {x} : 0.f;\nrp_{c}[mi * 16 + v] = a; }}")
+            elif r.kind == "max":
+                e(f"{{ float a = -INFINITY;\n#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) a = t.col_ok(ni) ? fmaxf(a, {x}) : a;\nrp_{c}[mi * 16 + v] = a; }}")
+            else:
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) rx_{c}[mi * 16 + v][ni] = {x};")
+        if row_reds:
+            e.dedent()
+            e("}")
         for r in col_reds:
             x = lambda: self.ref(r.input)  # noqa: E731
             o = r.state_offset
@@ -381,6 +409,21 @@ class Codegen:
         e.dedent()
         e("}")
         if row_reds:
+            e("if constexpr (!ROW_BY_ROW) {")
+            e.indent()
+        for r in row_reds:
+            c, o = _cname(r.name), r.state_offset
+            if r.kind in ("sum", "max"):
+                e(f"evt::rows_simple<Cfg, {ir.row_state}, {'true' if r.kind == 'max' else 'false'}>(t, rp_{c}, {o});")
+            elif r.kind == "maxsumexp":
+                e(f"evt::rows_maxsumexp<Cfg, {ir.row_state}, {ir.col_state}>(t, rx_{c}, {o});")
+            elif r.kind == "welford":
+                e(f"evt::rows_welford<Cfg, {ir.row_state}, {ir.col_state}>(t, rx_{c}, {o});")
+            else:
+                raise NotImplementedError(r.kind)
+        if row_reds:
+            e.dedent()
+            e("}")
             e("const int row_ticket = evt::row_reduce_publish<Cfg, Epi>(p, t, g);")
         if col_reds:
             e("const int col_ticket = evt::col_reduce_publish<Cfg, Epi>(p, t, g, cst);")

@@ -847,7 +847,8 @@ inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hip
   return (int)hipGetLastError();
 }
 
-// Write one per-wave row state into the LDS exchange area (lane 0 of each half).
+// Write one per-wave row state into the LDS exchange area (lane 0 of each half): for wave tiles of one 32-row
+// block, whose rows are reduced one by one with half_wave_sum / half_wave_max.
 template <class Cfg, int RS, class Tile>
 EVT_DEV void row_state_to_lds(const Tile& t, int mi, int v, const float (&st)[RS]) {
   if ((t.lane & 31) == 0) {
@@ -855,6 +856,171 @@ EVT_DEV void row_state_to_lds(const Tile& t, int mi, int v, const float (&st)[RS
 #pragma unroll
     for (int c = 0; c < RS; ++c) lds[c] = st[c];
   }
+}
+
+// ---------------------------------------------------------------------------
+// Per-row reductions of a wave tile, all rows at once.
+//
+// A lane holds one partial per accumulator row it owns (R = 16 MI rows, index r = 16 mi + v); each row is spread
+// over the 32 lanes of a half wave.  Instead of one 5-step butterfly per row (160 cross-lane operations per 32
+// rows, every lane ending up with every total) the rows are reduced together: at each step a lane hands the
+// partner half of its registers and keeps the other half, so the work halves with the lanes involved -- 31
+// exchanges for 32 rows -- and lane j ends up with the total of row j alone.  Steps, by the lane bit that tells the
+// partners apart: bit 4 v_permlane16_swap, bit 3 row_mirror, bit 2 row_half_mirror, bit 1 / bit 0 quad_perm.
+// After the steps x[e], e < R / 32, holds the total of row (lane & 31) * R / 32 + e.  (Wave tiles of a single
+// 32-row block reduce row by row instead, see row_state_to_lds.)
+// ---------------------------------------------------------------------------
+template <bool MAX>
+EVT_DEV float red_op(float a, float b) { return MAX ? fmaxf(a, b) : a + b; }
+
+template <int N, bool MAX>
+EVT_DEV void rows_step_swap16(float* x) {   // even rows of 16 lanes keep x[i], odd ones x[i + N/2]
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i) {
+    float a = x[i], b = x[i + N / 2];
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    x[i] = red_op<MAX>(a, b);
+  }
+}
+template <int N, int CTRL, int BIT, bool MAX>
+EVT_DEV void rows_step_dpp(float* x, int lane) {
+  const bool up = (lane >> BIT) & 1;
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i) {
+    const float keep = up ? x[i + N / 2] : x[i];
+    const float send = up ? x[i] : x[i + N / 2];
+    const float got = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), CTRL, 0xf, 0xf, true));
+    x[i] = red_op<MAX>(keep, got);
+  }
+}
+template <int R, bool MAX>
+EVT_DEV void rows_reduce(float (&x)[R], int lane) {
+  static_assert(R == 32 || R == 64 || R == 128, "two or more 32-row blocks per wave tile");
+  rows_step_swap16<R, MAX>(x);
+  rows_step_dpp<R / 2, 0x140, 3, MAX>(x, lane);    // row_mirror
+  rows_step_dpp<R / 4, 0x141, 2, MAX>(x, lane);    // row_half_mirror
+  rows_step_dpp<R / 8, 0x4E, 1, MAX>(x, lane);     // quad_perm [2,3,0,1]
+  rows_step_dpp<R / 16, 0xB1, 0, MAX>(x, lane);    // quad_perm [1,0,3,2]
+}
+// rows (of this lane's half) whose totals the lane holds after rows_reduce, and which
+template <int R>
+constexpr int rows_owned() { return R / 32; }
+template <int R>
+EVT_DEV int row_owned(int lane, int e) { return (lane & 31) * (R / 32) + e; }
+
+// LDS areas of the epilogue's reductions inside the operand stages: row states [wn][bm][RS] + flag, column states
+// [max(wm, shares)][bn][CS] + flag, then per wave and half R floats through which a row's first-pass result (its
+// maximum, its mean) goes back to all the lanes that hold the row.
+template <class Cfg, int RS, int CS>
+struct RedAreas {
+  static constexpr int ROW_AREA = RS > 0 ? (Cfg::WN * Cfg::BM * RS * 4 + 16) : 0;
+  static constexpr int SHARES = Cfg::THREADS / Cfg::BN > 0 ? Cfg::THREADS / Cfg::BN : 1;
+  static constexpr int COL_AREA = CS > 0 ? ((Cfg::WM > SHARES ? Cfg::WM : SHARES) * Cfg::BN * CS * 4 + 16) : 0;
+  static constexpr int BACK = (ROW_AREA + COL_AREA + 15) / 16 * 16;
+  static constexpr int BACK_BYTES = Cfg::WAVES * 2 * 16 * Cfg::MI * 4;
+};
+
+// Hand the first-pass result of every row back to all lanes of its half: owners write, everybody reads.
+template <class Cfg, int R>
+EVT_DEV void rows_broadcast(char* area, int lane, int wave, const float (&own)[rows_owned<R>()], float (&all)[R]) {
+  float* slot = (float*)area + (wave * 2 + (lane >> 5)) * R;
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) slot[row_owned<R>(lane, e)] = own[e];
+  // same wave: LDS operations complete in order, no barrier needed
+#pragma unroll
+  for (int r = 0; r < R; r += 4) {
+    const float4 q = *(const float4*)(slot + r);
+    all[r] = q.x; all[r + 1] = q.y; all[r + 2] = q.z; all[r + 3] = q.w;
+  }
+}
+
+// Store component c of the row state of every row this lane owns: state[wn][local row][RS] at smem.
+template <class Cfg, int RS, class Tile>
+EVT_DEV void rows_state_store(const Tile& t, int c, const float (&own)[rows_owned<16 * Cfg::MI>()]) {
+  constexpr int R = 16 * Cfg::MI;
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) {
+    const int r = row_owned<R>(t.lane, e);
+    const int lrow = t.row0 - t.m0 + (r >> 4) * 32 + 8 * ((r & 15) >> 2) + (r & 3);
+    ((float*)t.smem)[(t.wn * Cfg::BM + lrow) * RS + c] = own[e];
+  }
+}
+
+// The four kinds of per-row reduction over this wave's columns; results go to components [o ...] of the rows'
+// states in LDS.  The two-pass kinds take the values `x[r][ni]` (r = 16 mi + v) and mask them by column validity.
+template <class Cfg, int RS, bool MAX, class Tile>
+EVT_DEV void rows_simple(const Tile& t, float (&part)[16 * Cfg::MI], int o) {   // part[r]: this lane's columns of row r
+  constexpr int R = 16 * Cfg::MI;
+  rows_reduce<R, MAX>(part, t.lane);
+  float own[rows_owned<R>()];
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) own[e] = part[e];
+  rows_state_store<Cfg, RS>(t, o, own);
+}
+template <class Cfg, int RS, int CS, class Tile>
+EVT_DEV void rows_maxsumexp(const Tile& t, const float (&x)[16 * Cfg::MI][Cfg::NI], int o) {
+  constexpr int R = 16 * Cfg::MI;
+  float part[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float a = -INFINITY;
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) a = t.col_ok(ni) ? fmaxf(a, x[r][ni]) : a;
+    part[r] = a;
+  }
+  rows_reduce<R, true>(part, t.lane);
+  float mx[rows_owned<R>()];
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) mx[e] = part[e];
+  float m[R];
+  rows_broadcast<Cfg, R>(t.smem + RedAreas<Cfg, RS, CS>::BACK, t.lane, t.wm * Cfg::WN + t.wn, mx, m);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float a = 0.f;
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) a += t.col_ok(ni) ? op_exp(x[r][ni] - m[r]) : 0.f;
+    part[r] = a;
+  }
+  rows_reduce<R, false>(part, t.lane);
+  float se[rows_owned<R>()];
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) se[e] = part[e];
+  rows_state_store<Cfg, RS>(t, o, mx);
+  rows_state_store<Cfg, RS>(t, o + 1, se);
+}
+template <class Cfg, int RS, int CS, class Tile>
+EVT_DEV void rows_welford(const Tile& t, const float (&x)[16 * Cfg::MI][Cfg::NI], int o) {
+  constexpr int R = 16 * Cfg::MI;
+  const float cnt = (float)t.wave_cols();
+  const float rcnt = cnt > 0.f ? 1.f / cnt : 0.f;
+  float part[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float a = 0.f;
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) a += t.col_ok(ni) ? x[r][ni] : 0.f;
+    part[r] = a;
+  }
+  rows_reduce<R, false>(part, t.lane);
+  float mean[rows_owned<R>()], n[rows_owned<R>()];
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) { mean[e] = part[e] * rcnt; n[e] = cnt; }
+  float m[R];
+  rows_broadcast<Cfg, R>(t.smem + RedAreas<Cfg, RS, CS>::BACK, t.lane, t.wm * Cfg::WN + t.wn, mean, m);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float a = 0.f;
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni) { const float d = x[r][ni] - m[r]; a += t.col_ok(ni) ? d * d : 0.f; }
+    part[r] = a;
+  }
+  rows_reduce<R, false>(part, t.lane);
+  float m2[rows_owned<R>()];
+#pragma unroll
+  for (int e = 0; e < rows_owned<R>(); ++e) m2[e] = part[e];
+  rows_state_store<Cfg, RS>(t, o, n);
+  rows_state_store<Cfg, RS>(t, o + 1, mean);
+  rows_state_store<Cfg, RS>(t, o + 2, m2);
 }
 
 // ---------------------------------------------------------------------------
