@@ -65,6 +65,39 @@ def reduction_lds_bytes(t: "TileConfig", row_state: int, col_state: int) -> int:
     return max(need, t.wm * t.wn * 64 * row_state * 4)
 
 
+STATIC_SCRATCH_BYTES = 1 << 20
+
+
+def emit_static_scratch(e: "_Emitter") -> None:
+    """File-scope device array that takes the workspace's place in `evt_launch_static`, and the per-device
+    look-up of its address (each GPU that loads the module holds its own copy)."""
+    e("// ---- evt_launch_static: the entry point that allocates nothing ------------------------------------------")
+    e("namespace {")
+    e(f"constexpr int64_t kScratchBytes = {STATIC_SCRATCH_BYTES};")
+    e("static __device__ __align__(256) unsigned char scratch[kScratchBytes];")
+    e("constexpr int kMaxDevices = 64;")
+    e("void* scratch_address[kMaxDevices];   // device address of `scratch` on each GPU, looked up on first use")
+    e("std::mutex scratch_mutex;")
+    e("// `scratch` names a host-side stand-in; kernels, fills and copies take the address this returns")
+    e("int scratch_on_current_device(void** out) {")
+    e("  int dev = -1;")
+    e("  const hipError_t e0 = hipGetDevice(&dev);")
+    e("  if (e0 != hipSuccess) return (int)e0;")
+    e("  if (dev < 0 || dev >= kMaxDevices) return EVT_ERR_RANGE;")
+    e("  std::lock_guard<std::mutex> lock(scratch_mutex);")
+    e("  if (!scratch_address[dev]) {")
+    e("    void* ptr = nullptr;")
+    e("    const hipError_t e1 = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));")
+    e("    if (e1 != hipSuccess) return (int)e1;")
+    e("    if (!ptr) return EVT_ERR_WORKSPACE;")
+    e("    scratch_address[dev] = ptr;")
+    e("  }")
+    e("  *out = scratch_address[dev];")
+    e("  return EVT_OK;")
+    e("}")
+    e("}  // namespace")
+
+
 _BINARY = {
     "add": "({a} + {b})", "sub": "({a} - {b})", "mul": "({a} * {b})",
     "div": "__fdividef({a}, {b})", "max": "fmaxf({a}, {b})", "min": "fminf({a}, {b})",
@@ -555,6 +588,7 @@ class Codegen:
         return {
             "abi": 3,
             "name": self.name,
+            "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
             "tile": asdict(t),
             "a_k_contiguous": self.spec.a_kc,
             "b_k_contiguous": self.spec.b_kc,
@@ -579,6 +613,7 @@ class Codegen:
         e('#include "evt_epilogue.hpp"')
         e('#include "evt_amd.h"')
         e("#include <stdlib.h>")
+        e("#include <mutex>")
         e("")
         e("namespace {")
         e("struct Epi {")
@@ -733,18 +768,40 @@ class Codegen:
         e("  hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ws, bytes / 4);")
         e("  return (int)hipGetLastError();")
         e("}")
-        e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
-        e("  evt::GemmArgs g; Epi::Params p;")
-        e("  const int rc = fill(a, g, p);")
-        e("  if (rc != EVT_OK) return rc;")
-        e("  const int64_t need = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
-        e("  if (need > 0 && (!ws || ws_bytes < need || ((uintptr_t)ws & 15))) return EVT_ERR_WORKSPACE;   // 16-byte aligned")
+        e("static int enqueue(evt::GemmArgs& g, const Epi::Params& p, void* ws, void* stream) {")
         e("  g.workspace = (char*)ws;")
         e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L * g.splits);")
         e("  hipLaunchKernelGGL((evt::evt_gemm_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  const int err = (int)hipGetLastError();")
         e("  if (err != 0) return err;")
         e("  return evt::launch_finalize<Epi>(p, g, (hipStream_t)stream);")
+        e("}")
+        e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
+        e("  evt::GemmArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  const int64_t need = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
+        e("  if (need > 0 && (!ws || ws_bytes < need || ((uintptr_t)ws & 15))) return EVT_ERR_WORKSPACE;   // 16-byte aligned")
+        e("  return enqueue(g, p, ws, stream);")
+        e("}")
+        emit_static_scratch(e)
+        e('extern "C" int evt_launch_static(const EvtArgs* a, void* stream) {')
+        e("  evt::GemmArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  const int64_t need = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
+        e("  if (need > kScratchBytes) return EVT_ERR_SCRATCH;   // this problem's partial results do not fit the static array")
+        e("  void* ws = nullptr;")
+        e("  if (need > 0) {")
+        e("    const int rs = scratch_on_current_device(&ws);")
+        e("    if (rs != EVT_OK) return rs;")
+        e("    // the array keeps the last call's contents, and another problem size lays its counters out elsewhere:")
+        e("    // everything this launch uses starts at zero (a fill kernel, not a memset node)")
+        e("    hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ws, (need + 3) / 4);")
+        e("    const int ef = (int)hipGetLastError();")
+        e("    if (ef != 0) return ef;")
+        e("  }")
+        e("  return enqueue(g, p, ws, stream);")
         e("}")
         if self.clock_probe:
             e("// out[0..3] = main-loop shader cycles, main-loop 100 MHz ticks, epilogue shader cycles, epilogue ticks")
@@ -961,6 +1018,7 @@ class RowCodegen(Codegen):
         return {
             "abi": 3,
             "name": self.name,
+            "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
             "anchor": sp.op,
             "row": {"chunks": sp.ch, "lanes_per_row": sp.lpr * sp.wpr, "waves_per_row": sp.wpr, "max_n": sp.max_n},
             "element": sp.elt,
@@ -989,6 +1047,7 @@ class RowCodegen(Codegen):
         e('#include "evt_rowwise.hpp"')
         e('#include "evt_amd.h"')
         e("#include <stdlib.h>")
+        e("#include <mutex>")
         e("")
         e("namespace {")
         e("struct Epi {")
@@ -1092,6 +1151,7 @@ class RowCodegen(Codegen):
         e("  (void)ws; (void)bytes; (void)stream;      // no counters: every partial is written before it is read")
         e("  return EVT_OK;")
         e("}")
+        e("static int enqueue(evt::RowArgs& g, const Epi::Params& p, unsigned grid, void* ws, void* stream);")
         e('extern "C" int evt_launch(const EvtArgs* a, void* ws, int64_t ws_bytes, void* stream) {')
         e("  evt::RowArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
@@ -1099,6 +1159,24 @@ class RowCodegen(Codegen):
         e("  const unsigned grid = grid_for(g);")
         e("  const int64_t need = (int64_t)grid * Epi::COL_STATE * g.N * 4;")
         e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
+        e("  return enqueue(g, p, grid, ws, stream);")
+        e("}")
+        emit_static_scratch(e)
+        e('extern "C" int evt_launch_static(const EvtArgs* a, void* stream) {')
+        e("  evt::RowArgs g; Epi::Params p;")
+        e("  const int rc = fill(a, g, p);")
+        e("  if (rc != EVT_OK) return rc;")
+        e("  const unsigned grid = grid_for(g);")
+        e("  const int64_t need = (int64_t)grid * Epi::COL_STATE * g.N * 4;")
+        e("  if (need > kScratchBytes) return EVT_ERR_SCRATCH;")
+        e("  void* ws = nullptr;")
+        e("  if (need > 0) {   // partials only, each written before it is read: nothing to clear")
+        e("    const int rs = scratch_on_current_device(&ws);")
+        e("    if (rs != EVT_OK) return rs;")
+        e("  }")
+        e("  return enqueue(g, p, grid, ws, stream);")
+        e("}")
+        e("static int enqueue(evt::RowArgs& g, const Epi::Params& p, unsigned grid, void* ws, void* stream) {")
         e("  g.colws = (float*)ws;")
         e("  if (p.fast) hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, true>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  else hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, false>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")

@@ -60,7 +60,8 @@ class EvtArgs(ctypes.Structure):
                 ("tensors", EvtTensorArg * EVT_MAX_TENSORS), ("scalars", ctypes.c_float * EVT_MAX_SCALARS)]
 
 
-ERROR_NAMES = {-1: "EVT_ERR_BAD_ARGS", -2: "EVT_ERR_ALIGNMENT", -3: "EVT_ERR_WORKSPACE", -4: "EVT_ERR_RANGE"}
+ERROR_NAMES = {-1: "EVT_ERR_BAD_ARGS", -2: "EVT_ERR_ALIGNMENT", -3: "EVT_ERR_WORKSPACE", -4: "EVT_ERR_RANGE",
+               -5: "EVT_ERR_SCRATCH"}
 
 
 class KernelModule:
@@ -77,6 +78,8 @@ class KernelModule:
         self.lib.evt_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         self.lib.evt_launch.restype = ctypes.c_int
         self.lib.evt_launch.argtypes = [ctypes.POINTER(EvtArgs), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        self.lib.evt_launch_static.restype = ctypes.c_int
+        self.lib.evt_launch_static.argtypes = [ctypes.POINTER(EvtArgs), ctypes.c_void_p]
         if self.lib.evt_abi_version() != EVT_ABI_VERSION:
             raise RuntimeError(f"{path}: ABI version mismatch")
         if hasattr(self.lib, "evt_clock_probe_read"):      # diagnostic builds only
@@ -113,6 +116,15 @@ class KernelModule:
         if rc > 0:
             # same error class as the reference raises on a failed launch
             # (python/gtl/ops/reduce_apply_operation.py:157-158)
+            raise RuntimeError(f"HIP Error {rc} launching {self.path.name}")
+
+
+    def launch_static(self, args: EvtArgs, stream: int) -> None:
+        """evt_launch_static: partial results go to the module's own device array, nothing is allocated."""
+        rc = self.lib.evt_launch_static(ctypes.byref(args), ctypes.c_void_p(stream))
+        if rc < 0:
+            raise RuntimeError(f"evt_launch_static rejected the arguments: {ERROR_NAMES.get(rc, rc)} ({self.path.name})")
+        if rc > 0:
             raise RuntimeError(f"HIP Error {rc} launching {self.path.name}")
 
 
@@ -225,6 +237,9 @@ class LazyModule:
 
     def launch(self, args: EvtArgs, ws_ptr: int, ws_bytes: int, stream: int) -> None:
         self.ensure().launch(args, ws_ptr, ws_bytes, stream)
+
+    def launch_static(self, args: EvtArgs, stream: int) -> None:
+        self.ensure().launch_static(args, stream)
 
     def clock_probe_read(self):
         return self.ensure().clock_probe_read()

@@ -110,6 +110,14 @@ def register_all() -> List[jit.LazyModule]:
         with force_tile(tile):
             for cfg in W.CONFIGS:
                 W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, W.PIPELINE_SHAPES[cfg]))
+    from .codegen import TileConfig
+    with force_tile(TileConfig(*W.NO_ALLOC_TILE)):
+        for cfg, cases in W.NO_ALLOC_SHAPES.items():
+            for shapes in cases:
+                W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
+    cfg, shapes, tile = W.NO_ALLOC_TOO_BIG
+    with force_tile(TileConfig(*tile)):
+        W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
     for name, (cls, _) in W.REFERENCE_PATTERNS.items():
         g = torch.Generator(device="cpu").manual_seed(0)
         # shapes only: generate on CPU lazily is costly for the big patterns, so

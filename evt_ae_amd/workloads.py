@@ -201,6 +201,14 @@ def make_inputs(cfg: int, shapes: dict = None, seed: int = None) -> List[torch.T
     return fn(g, **(shapes or {}))
 
 
+# evt_launch_static against evt_launch: (config, first problem, a smaller second one) through one module; the
+# classifier's 6 MiB of partial results exceed the static array
+NO_ALLOC_TILE = (128, 128, 64, 2, 4, 2, True, 4, 2)
+NO_ALLOC_SHAPES = {3: (dict(M=1024, N=512, K=256), dict(M=384, N=256, K=128)),
+                   4: (dict(M=1024, N=512, K=256), dict(M=384, N=256, K=128))}
+NO_ALLOC_TOO_BIG = (5, dict(M=1024, N=131072, K=64), (256, 256, 64, 4, 2, 2, True, 4, 2))
+
+
 def pipeline_tiles():
     """Ping-pong main-loop variants (pipe 2: two barriers per k-tile, pipe 3:
     one) on every stage count / k-depth / wave grid they are instantiated with."""

@@ -39,6 +39,7 @@ extern "C" {
 #define EVT_ERR_ALIGNMENT (-2)     /* operand not aligned for this module       */
 #define EVT_ERR_WORKSPACE (-3)     /* workspace missing or too small            */
 #define EVT_ERR_RANGE (-4)         /* a dimension exceeds what the kernel holds */
+#define EVT_ERR_SCRATCH (-5)       /* evt_launch_static: the partial results of this problem exceed the static array */
 
 /* One epilogue tensor (load or store).  Element (l, m, n) of the logical
  * [L, M, N] iteration space lives at
@@ -152,6 +153,22 @@ int evt_workspace_init(void* workspace, int64_t bytes, void* stream);
  * `operation.run(arguments, stream=stream.cuda_stream)` (evt_fuser.py:546). */
 int evt_launch(const EvtArgs* args, void* workspace, int64_t workspace_bytes,
                void* stream);
+
+/* `evt_launch` for callers that cannot allocate device memory or be handed a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference (whose callers
+ * allocate and zero their reduction outputs per call, evt_fuser.py:217-225).
+ * The partial results, arrival counters and split-K tiles that `evt_launch`
+ * keeps in the caller's workspace live in a device array that is part of the
+ * module ("static_scratch_bytes" in the module spec: 1 MiB), which every GPU the module runs
+ * on holds from the first such call until the process ends; the call itself
+ * allocates nothing and frees nothing.  A problem whose workspace
+ * (evt_workspace_bytes) exceeds the array is refused with EVT_ERR_SCRATCH
+ * before anything is enqueued.  All calls on one GPU share that GPU's array,
+ * so calls that may overlap in time (different streams) race; each call
+ * clears what it needs on `stream` first (a fill kernel).  Inputs and outputs
+ * are passed as for `evt_launch`. */
+int evt_launch_static(const EvtArgs* args, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,8 +30,8 @@ def module():
 
 
 def test_header_declares_the_expected_entry_points():
-    assert declared_symbols() == ["evt_abi_version", "evt_launch", "evt_module_spec", "evt_workspace_bytes",
-                                  "evt_workspace_init"]
+    assert declared_symbols() == ["evt_abi_version", "evt_launch", "evt_launch_static", "evt_module_spec",
+                                  "evt_workspace_bytes", "evt_workspace_init"]
 
 
 def test_every_built_module_exports_the_abi():
