@@ -332,17 +332,135 @@ def cpu_baseline(torch, W, evt_oracle, cfgs, reps=3):
     return flops / secs / 1e12, torch.get_num_threads(), secs
 
 
-# L2<->fabric bytes per launch of the fused kernel, from two rocprofv3 --pmc runs of this script (FETCH_SIZE,
-# then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the 256 MiB streaming kernel
-# of --copy-calibration (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Keyed by (config, tile): a launch with another
-# tile has no measurement and reports null.  The summary of those runs is profiles/evt_gemm_kernel_bench_configs_1-5.md.
-MEASURED_TRAFFIC_BYTES = {
-    (1, "256x256x64_w2x4_s2_dma_g4_p3"): int((2.0 * 24738.0 + 32768) * 1024),
-    (2, "128x512x64_w4x2_s1_dma_g4"): int((2.0 * 4222.0 + 33024) * 1024),
-    (3, "128x256x64_w2x4_s3_dma_g4_p3"): int((2.0 * 74120.8 + 17610) * 1024),
-    (4, "256x128x64_w4x2_s3_dma_g4_p3"): int((2.0 * 73935.3 + 16524.2) * 1024),
-    (5, "256x256x64_w4x2_s2_dma_g4_p2"): int((2.0 * 69934.5 + 18432) * 1024),
-}
+class MfmaProbe:
+    """Builds / loads bench_mfma_probe.hip (a register-only MFMA loop, a measurement aid that sits beside this
+    script) and runs it on operand data of the caller's choice: what the matrix cores sustain on data like the
+    benchmark's, next to the published peak."""
+
+    SOURCE = ROOT / "bench_mfma_probe.hip"
+
+    def __init__(self):
+        import hashlib
+        from evt_ae_amd import jit
+        h = hashlib.sha256((self.SOURCE.read_text() + " ".join(jit.HIPCC_FLAGS)).encode()).hexdigest()[:20]
+        self.path = ROOT / "build" / f"bench_mfma_probe_{h}.so"
+        self._lib = None
+
+    def build(self, force=False):
+        import subprocess
+        from evt_ae_amd import jit
+        if force or not self.path.exists():
+            self.path.parent.mkdir(parents=True, exist_ok=True)
+            tmp = self.path.with_suffix(f".tmp{os.getpid()}.so")
+            proc = subprocess.run([jit.HIPCC, *jit.HIPCC_FLAGS, str(self.SOURCE), "-o", str(tmp)],
+                                  capture_output=True, text=True)
+            if proc.returncode != 0:
+                raise RuntimeError(f"hipcc failed for {self.SOURCE}:\n{proc.stderr[-4000:]}")
+            os.replace(tmp, self.path)
+        return self.path
+
+    def run(self, torch, operands, workgroups=256, iters=1 << 15, warm_launches=6):
+        """operands: contiguous CUDA fp16 tensor of >= 65536 elements.  Returns (TFLOP/s, shader MHz) of the last
+        of `warm_launches` + 1 back-to-back launches."""
+        import ctypes
+        if self._lib is None:
+            self.build()
+            self._lib = ctypes.CDLL(str(self.path), mode=ctypes.RTLD_LOCAL)
+            self._lib.evt_mfma_probe_launch.restype = ctypes.c_int
+            self._lib.evt_mfma_probe_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                        ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        if operands.dtype != torch.float16 or operands.numel() < 65536 or not operands.is_contiguous():
+            raise ValueError("operands: contiguous fp16 tensor of at least 65536 elements")
+        sink = torch.zeros(1024, dtype=torch.float32, device=operands.device)
+        clk = torch.zeros(2, dtype=torch.int64, device=operands.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(warm_launches + 1):
+            if i == warm_launches:
+                e0.record()
+            rc = self._lib.evt_mfma_probe_launch(operands.data_ptr(), sink.data_ptr(), clk.data_ptr(), workgroups, iters,
+                                                 ctypes.c_void_p(stream))
+            if rc != 0:
+                raise RuntimeError(f"HIP Error {rc} launching the MFMA probe")
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        cycles, ticks = (int(x) for x in clk.cpu())
+        flops = workgroups * 8 * iters * 8 * 32768.0
+        return flops / (ms * 1e-3) / 1e12, 100.0 * cycles / max(ticks, 1)
+
+
+# ---------------------------------------------------------------------------
+# HBM-side traffic of the fused kernels, from rocprofv3 counter runs of this script
+# ---------------------------------------------------------------------------
+# Two counter runs of this script (`rocprofv3 --pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, both with
+# --copy-calibration) leave one bench_counter_collection.csv each.  `bench.py --traffic-summary FETCH.csv WRITE.csv`
+# condenses them into TRAFFIC_FILE: per fused kernel (named by its GemmCfg<...> template arguments and grid size)
+# the mean KiB per dispatch of both counters, and the factor each counter needs so that the plain streaming kernel
+# of --copy-calibration reads its known size.  A bench run looks the dominant kernel up there; a kernel the file
+# does not hold (another tile, no counter run yet) reports "traffic": null.
+TRAFFIC_FILE = ROOT / "profiles" / "evt_gemm_kernel_hbm_traffic.txt"
+CALIBRATION_KIB = 64 * 4 * 1024      # the streaming kernel reads and writes 64 Mi fp32 values
+
+
+def kernel_key(source_text):
+    """The GemmCfg<...> instantiation a generated module launches, as rocprofv3 prints it in kernel names."""
+    import re
+    m = re.search(r"using Cfg = (evt::GemmCfg<[^>]*>);", source_text)
+    return m.group(1) if m else None
+
+
+def summarize_traffic(fetch_csv, write_csv, out_path=TRAFFIC_FILE):
+    import csv
+    import re
+    from collections import defaultdict
+    sums = {"FETCH_SIZE": defaultdict(list), "WRITE_SIZE": defaultdict(list)}
+    for path in (fetch_csv, write_csv):
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] not in sums:
+                    continue
+                name = r["Kernel_Name"]
+                m = re.search(r"evt_gemm_kernel<(evt::GemmCfg<[^>]*>)", name)
+                if m:
+                    key = (m.group(1), int(r["Grid_Size"]))
+                elif "neg_kernel_cuda" in name and int(r["Grid_Size"]) == 64 << 18:
+                    key = ("calibration", 0)
+                else:
+                    continue
+                sums[r["Counter_Name"]][key].append(float(r["Counter_Value"]))
+    mean = {c: {k: sum(v) / len(v) for k, v in d.items()} for c, d in sums.items()}
+    cal = ("calibration", 0)
+    if cal not in mean["FETCH_SIZE"] or cal not in mean["WRITE_SIZE"]:
+        sys.exit("bench.py: the counter files hold no dispatch of the --copy-calibration kernel")
+    lines = ["# written by `bench.py --traffic-summary`; KiB per dispatch, mean over the run's dispatches",
+             f"calibration known_kib={CALIBRATION_KIB} fetch_kib={mean['FETCH_SIZE'][cal]:.1f} "
+             f"write_kib={mean['WRITE_SIZE'][cal]:.1f} fetch_scale={CALIBRATION_KIB / mean['FETCH_SIZE'][cal]:.4f} "
+             f"write_scale={CALIBRATION_KIB / mean['WRITE_SIZE'][cal]:.4f}"]
+    for key in sorted(k for k in mean["FETCH_SIZE"] if k != cal and k in mean["WRITE_SIZE"]):
+        lines.append(f"kernel {key[0].replace(' ', '')} grid={key[1]} dispatches={len(sums['FETCH_SIZE'][key])} "
+                     f"fetch_kib={mean['FETCH_SIZE'][key]:.1f} write_kib={mean['WRITE_SIZE'][key]:.1f}")
+    Path(out_path).write_text("\n".join(lines) + "\n")
+    return lines
+
+
+def measured_traffic_bytes(key, path=TRAFFIC_FILE):
+    """HBM-side bytes per launch of the kernel `key`, scaled by the calibration; None when the file does not hold
+    the kernel, or holds it at several grid sizes (then the entry cannot be told apart from here)."""
+    if key is None or not Path(path).exists():
+        return None
+    scale, found = None, []
+    for ln in Path(path).read_text().splitlines():
+        if ln.startswith("#"):
+            continue
+        f = dict(kv.split("=", 1) for kv in ln.split()[1:] if "=" in kv)
+        if ln.startswith("calibration"):
+            scale = (float(f["fetch_scale"]), float(f["write_scale"]))
+        elif ln.startswith("kernel") and ln.split()[1] == key.replace(" ", ""):
+            found.append((float(f["fetch_kib"]), float(f["write_kib"])))
+    if scale is None or len(found) != 1:
+        return None
+    return int((scale[0] * found[0][0] + scale[1] * found[0][1]) * 1024)
 
 
 def main():
@@ -367,7 +485,13 @@ def main():
     ap.add_argument("--no-clock-probe", dest="clock_probe", action="store_false",
                     help="skip the diagnostic build of each kernel that reports the shader clock it ran at and "
                          "workgroup 0's main-loop / epilogue split (per_config[*].clock_probe, roofline.shader_mhz)")
+    ap.add_argument("--traffic-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
+                    help="no GPU work: condense the counter files of two rocprofv3 --pmc runs of this script "
+                         f"(FETCH_SIZE, WRITE_SIZE) into {TRAFFIC_FILE.relative_to(ROOT)} and exit")
     args = ap.parse_args()
+    if args.traffic_summary:
+        print("\n".join(summarize_traffic(*args.traffic_summary)))
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU (the fused GEMM+epilogue path has no cross-GPU exchange); "
                  "run with --gpus 1")
@@ -416,6 +540,8 @@ def main():
                                                                      case.sets[i % case.nsets][3][0],
                                                                      case.sets[i % case.nsets][3][1]), approximate="tanh"),
                                    max(20, args.steps // 4), 5)
+        if ms_unf_lib is not None:
+            best_unf = min(best_unf, ms_unf_lib)   # the speed-up is quoted against the fastest unfused form
         details[cfg] = {
             "workload": wl.name, "dims_MNKL": list(wl.dims), "tile": case.op.tile.tag(),
             "us": round(ms * 1e3, 2), "us_graph": None if ms_graph is None else round(ms_graph * 1e3, 2),
@@ -427,6 +553,7 @@ def main():
             "unfused_us_graph": None if ms_unf_graph is None else round(ms_unf_graph * 1e3, 2),
             "speedup_vs_unfused": round(best_unf / best, 3),
             "max_rel_err": parity, "normwise_err": normwise, "buffer_sets": case.nsets, "_ms": ms, "_best": best,
+            "_key": kernel_key(case.op.module.source),
         }
         if ms_unf_lib is not None:
             details[cfg]["unfused_addmm_gelu_us"] = round(ms_unf_lib * 1e3, 2)
@@ -467,17 +594,18 @@ def main():
     # like the benchmark's, and on zeros: the first is the practical MFMA ceiling for this data on this part
     mfma_only = None
     if args.clock_probe:
-        probe = jit.MfmaProbe()
+        probe = MfmaProbe()
         g = torch.Generator(device="cpu").manual_seed(0xE7A0)
         rnd = torch.randn(1 << 16, generator=g).half().cuda()
-        t_rnd, mhz_rnd = probe.run(rnd)
-        t_zero, mhz_zero = probe.run(torch.zeros_like(rnd))
+        t_rnd, mhz_rnd = probe.run(torch, rnd)
+        t_zero, mhz_zero = probe.run(torch, torch.zeros_like(rnd))
         mfma_only = {"normal_operands_tflops": round(t_rnd, 1), "normal_operands_shader_mhz": round(mhz_rnd),
                      "zero_operands_tflops": round(t_zero, 1), "zero_operands_shader_mhz": round(mhz_zero)}
         clock["frac_of_mfma_only_normal_operands"] = round(dom_tflops / t_rnd, 4)
         log(f"[bench] register-only MFMA loop: {mfma_only}")
+    traffic = measured_traffic_bytes(details[dom]["_key"])
     for d in details.values():
-        d.pop("_ms"); d.pop("_best")
+        d.pop("_ms"); d.pop("_best"); d.pop("_key")
     line = {
         "metric": "fused GEMM+epilogue TFLOP/s, % MI355X fp16 MFMA peak, speedup vs unfused",
         "value": round(flops / (step_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
@@ -490,7 +618,7 @@ def main():
                    "frac_mfma_peak": round(flops / (step_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS, 4)},
         "roofline": {"bound": "mfma", "achieved": round(dom_tflops, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(dom_tflops / PEAK_FP16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((dom, details[dom]["tile"])),
+                     "traffic": traffic,
                      "kernel": f"config {dom} ({details[dom]['workload']}, tile {details[dom]['tile']})",
                      "us": details[dom]["us"], **clock, "mfma_only": mfma_only},
         "cpu_baseline": cpu,

@@ -65,6 +65,7 @@ def reduction_lds_bytes(t: "TileConfig", row_state: int, col_state: int) -> int:
     return max(need, t.wm * t.wn * 64 * row_state * 4)
 
 
+ABI_VERSION = 4            # EVT_ABI_VERSION of include/evt_amd.h
 STATIC_SCRATCH_BYTES = 1 << 20
 
 
@@ -520,7 +521,7 @@ class Codegen:
                 r = self.ir.rng_scalar
                 e(f"float {c}[NI];")
                 e(f"evt::rand_row<Tile>((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r}]) | ((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r + 1}]) << 32), "
-                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u, "
+                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u + 16u * __builtin_bit_cast(uint32_t, p.s[{r + 3}]), "
                   f"{base} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, p.t{k}_sn, {c});")
             elif s.kind == "aux":
                 e(f"float {c}[NI];")
@@ -586,7 +587,7 @@ class Codegen:
     def module_spec(self) -> dict:
         t = self.spec.tile
         return {
-            "abi": 3,
+            "abi": ABI_VERSION,
             "name": self.name,
             "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
             "tile": asdict(t),
@@ -599,7 +600,7 @@ class Codegen:
             "tensors": [{"name": s.name, "role": s.role, "dtype": s.dtype, "kind": s.kind,
                          "domain": s.domain} for s in self.ir.slots],
             "num_scalars": len(self.ir.scalars),
-            # scalars[rng_scalars .. +3] = 32-bit patterns of (seed low, seed high, offset, unused) for rand_like
+            # scalars[rng_scalars .. +3] = 32-bit patterns of (seed low, seed high, offset, stream id) for rand_like
             "rng_scalars": self.ir.rng_scalar,
         }
 
@@ -639,16 +640,13 @@ class Codegen:
         red_lds = reduction_lds_bytes(t, ir.row_state, ir.col_state)
         e(f"static_assert(Cfg::LDS_BYTES >= {red_lds}, \"reduction exchange area exceeds the operand LDS\");")
         e("")
-        e("// EVT_TWO_KERNEL_REDUCE=1 forces the separate finalize kernel for every cross-tile reduction")
-        e("bool evt_two_kernel_reduce() {")
-        e("  static const bool v = [] { const char* s = getenv(\"EVT_TWO_KERNEL_REDUCE\"); return s && s[0] == '1'; }();")
-        e("  return v;")
-        e("}")
         e("int fill(const EvtArgs* a, evt::GemmArgs& g, Epi::Params& p) {")
         e.indent()
         e("if (!a || !a->A || !a->B) return EVT_ERR_BAD_ARGS;")
         e("if (a->num_tensors != kNumTensors || a->num_scalars != kNumScalars) return EVT_ERR_BAD_ARGS;")
         e("if (a->M <= 0 || a->N <= 0 || a->K <= 0 || a->L <= 0) return EVT_ERR_BAD_ARGS;")
+        e("if (a->split_k < 0 || (a->flags & ~EVT_FLAG_TWO_KERNEL_REDUCE)) return EVT_ERR_BAD_ARGS;")
+        e("const bool two_kernel_reduce = (a->flags & EVT_FLAG_TWO_KERNEL_REDUCE) != 0;")
         e("g.M = a->M; g.N = a->N; g.K = a->K; g.L = a->L;")
         e("g.A = (const char*)a->A; g.lda = a->lda; g.bsA = a->batch_stride_A;")
         e("g.B = (const char*)a->B; g.ldb = a->ldb; g.bsB = a->batch_stride_B;")
@@ -672,7 +670,7 @@ class Codegen:
                 e("  if (x.l_mod != 0 || x.l_div <= 1 || a->L % x.l_div) return EVT_ERR_BAD_ARGS;")
                 e("  g.row_fold_count = (int)x.l_div; }")
         e("// few partials: the last workgroup to arrive combines them; many: a finalize kernel does")
-        e("g.row_inkernel = (g.tiles_n * g.row_fold_count <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
+        e("g.row_inkernel = (g.tiles_n * g.row_fold_count <= evt::kMaxInKernelPartials && !two_kernel_reduce) ? 1 : 0;")
         e("g.col_fold_step = 1; g.col_fold_count = 1;")
         col_folds = {r.fold for r in ir.reduces.values() if r.axis == "col"} - {""}
         if col_folds:
@@ -682,15 +680,14 @@ class Codegen:
             e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
             e("  if (x.l_mod <= 0 || x.l_div != 1 || a->L % x.l_mod) return EVT_ERR_BAD_ARGS;")
             e("  g.col_fold_step = (int)x.l_mod; g.col_fold_count = a->L / (int)x.l_mod;")
-            e("  if ((int64_t)g.tiles_m * g.col_fold_count > evt::kMaxInKernelPartials || evt_two_kernel_reduce()) return EVT_ERR_RANGE; }")
-        e("g.col_inkernel = (g.tiles_m * g.col_fold_count <= evt::kMaxInKernelPartials && !evt_two_kernel_reduce()) ? 1 : 0;")
+            e("  if ((int64_t)g.tiles_m * g.col_fold_count > evt::kMaxInKernelPartials || two_kernel_reduce) return EVT_ERR_RANGE; }")
+        e("g.col_inkernel = (g.tiles_m * g.col_fold_count <= evt::kMaxInKernelPartials && !two_kernel_reduce) ? 1 : 0;")
         e("// Split-K: when the output tiles cannot fill the chip and K is long, several workgroups share a tile")
-        e("// (EVT_SPLIT_K=1 turns this off, EVT_SPLIT_K=n asks for n splits)")
+        e("// (EvtArgs.split_k: 0 = decide here, 1 = off, n = n splits)")
         e("g.splits = 1; g.k_chunk = (a->K + Cfg::BK - 1) / Cfg::BK * Cfg::BK;")
         if t.stages > 1:
             e("{")
-            e("  const char* env = getenv(\"EVT_SPLIT_K\");      // read per call: a caller may switch it between launches")
-            e("  const int want = env ? atoi(env) : 0;")
+            e("  const int want = a->split_k;")
             e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
               "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
             e("  const int kt = (a->K + Cfg::BK - 1) / Cfg::BK;")
@@ -971,7 +968,7 @@ class RowCodegen(Codegen):
             elif n.op == "load" and ir.slots[n.slot].kind == "rand":
                 k, r = n.slot, ir.rng_scalar
                 e(f"evt::rand8((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r}]) | ((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r + 1}]) << 32), "
-                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u, o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, {c});")
+                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u + 16u * __builtin_bit_cast(uint32_t, p.s[{r + 3}]), o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, {c});")
             elif n.op == "load" and name in self.hoisted:
                 e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
             elif n.op == "load":
@@ -1016,7 +1013,7 @@ class RowCodegen(Codegen):
     def module_spec(self) -> dict:
         sp = self.row_spec
         return {
-            "abi": 3,
+            "abi": ABI_VERSION,
             "name": self.name,
             "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
             "anchor": sp.op,

@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import ctypes
 import operator
+import itertools
 import os
 from contextlib import nullcontext
 from typing import Any, Dict, List, Optional, Sequence, Tuple
@@ -121,6 +122,19 @@ def _contig_strides(shape: Sequence[int]) -> Tuple[int, ...]:
 # ---------------------------------------------------------------------------
 
 
+_RAND_STREAM_IDS = itertools.count(1)
+
+
+def launch_switches() -> Tuple[int, int]:
+    """(EvtArgs.split_k, EvtArgs.flags) from the host's environment, read at
+    every call: EVT_SPLIT_K=1|n turns split-K off / asks for n splits,
+    EVT_TWO_KERNEL_REDUCE=1 finishes cross-tile reductions in the finalize
+    kernel.  The kernel modules themselves read no environment."""
+    split = os.environ.get("EVT_SPLIT_K")
+    flags = jit.EVT_FLAG_TWO_KERNEL_REDUCE if os.environ.get("EVT_TWO_KERNEL_REDUCE") == "1" else 0
+    return (max(0, int(split)) if split else 0), flags
+
+
 class FusedOpBase:
     """Callable placed in the fx graph.  `fused(*epilogue_inputs, A, B)` returns
     the list of partition outputs (reference: evt_fuser.py:62-279)."""
@@ -144,11 +158,28 @@ class FusedOpBase:
         self.slot_sources = epilogue_visitor.slot_sources      # slot -> ('input', idx) | ('output', store name)
         self.store_meta = epilogue_visitor.store_meta          # store name -> (shape, dtype)
         self._workspace = {}
-        # rand_like stream: 64-bit seed (torch's global seed at trace time unless set) and a 32-bit offset that
-        # advances by one per launch, so successive calls draw different numbers
-        self.rand_seed = int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF
+        # rand_like stream: 64-bit seed (torch's global seed at the time of the call unless `rand_seed` is set), a
+        # 32-bit offset that advances by one per launch, so successive calls draw different numbers, and a stream
+        # id of the op's own (process-wide count, in trace order) that goes into the generator's counter next to
+        # the slot index: two fused ops with rand_like tensors of equal shape draw unrelated numbers, as eager
+        # PyTorch does.  The offset is a launch argument: a captured HIP graph replays the mask it was captured with.
+        self._rand_seed: Optional[int] = None
+        self.rand_stream = next(_RAND_STREAM_IDS) & 0x0FFFFFFF
         self.rand_offset = 0
         self.last_rand_state: Optional[Tuple[int, int]] = None   # (seed, offset) the most recent launch used
+
+    @property
+    def rand_seed(self) -> int:
+        seed = torch.initial_seed() if self._rand_seed is None else self._rand_seed
+        return int(seed) & 0xFFFFFFFFFFFFFFFF
+
+    @rand_seed.setter
+    def rand_seed(self, value: Optional[int]) -> None:
+        self._rand_seed = value
+
+    def rand_salt(self, slot: int) -> int:
+        """Fourth counter word of the generator for rand_like slot `slot` of this op."""
+        return (slot + 16 * self.rand_stream) & 0xFFFFFFFF
 
     # -- to be provided by subclasses -----------------------------------------
     module: jit.KernelModule
@@ -173,6 +204,7 @@ class FusedOpBase:
         a.M, a.N, a.K, a.L = M, N, K, L
         a.A, a.lda, a.batch_stride_A = A.data_ptr(), lda, bsa
         a.B, a.ldb, a.batch_stride_B = B.data_ptr(), ldb, bsb
+        a.split_k, a.flags = launch_switches()
         keep = [A, B]
         self.fill_epilogue_arguments(a, keep, visitor_args, args)
         return a, keep
@@ -223,16 +255,17 @@ class FusedOpBase:
             # 32-bit patterns, not float values: written through an integer view of the scalar array
             bits = (ctypes.c_uint32 * jit.EVT_MAX_SCALARS).from_buffer(a, jit.EvtArgs.scalars.offset)
             r = self.ir.rng_scalar
-            bits[r], bits[r + 1] = self.rand_seed & 0xFFFFFFFF, (self.rand_seed >> 32) & 0xFFFFFFFF
-            bits[r + 2], bits[r + 3] = self.rand_offset & 0xFFFFFFFF, 0
-            self.last_rand_state = (self.rand_seed, self.rand_offset & 0xFFFFFFFF)
+            seed = self.rand_seed
+            bits[r], bits[r + 1] = seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF
+            bits[r + 2], bits[r + 3] = self.rand_offset & 0xFFFFFFFF, self.rand_stream
+            self.last_rand_state = (seed, self.rand_offset & 0xFFFFFFFF)
             self.rand_offset += 1
 
     def workspace_for(self, a: jit.EvtArgs, stream, device) -> Tuple[int, int]:
         """Device workspace for cross-workgroup reductions, one per stream,
         zero-filled once (launches leave it clean)."""
-        # the size depends on the problem (fixed per op) and on the split-K switch, which may change between calls
-        mode = os.environ.get("EVT_SPLIT_K")
+        # the size depends on the problem (fixed per op) and on the block's split-K / reduction switches
+        mode = (a.split_k, a.flags)
         cached = getattr(self, "_ws_bytes", None)
         if cached is None or cached[0] != mode:
             cached = self._ws_bytes = (mode, self.module.workspace_bytes(a))
@@ -473,6 +506,13 @@ class FusedGEMM(FusedOpBase):
     def operands(self, A, B):
         A = A.contiguous()
         B = B.contiguous()
+        if self.tile.dma:
+            # the global->LDS path moves 16-byte chunks: a contiguous view that starts at an odd storage offset is
+            # copied into a fresh (aligned) allocation instead of failing the launch, as eager would simply work
+            if A.data_ptr() & 15:
+                A = A.clone()
+            if B.data_ptr() & 15:
+                B = B.clone()
         return A, self.lda, 0, B, self.ldb, 0
 
     def anchor_eager(self, A, B):

@@ -98,21 +98,39 @@ def _freeze(x):
         return ("node", x.name)
     if isinstance(x, slice):
         return ("slice", x.start, x.stop, x.step)
+    if isinstance(x, (bool, int, float, complex)):
+        return (type(x).__name__, x)      # 1, 1.0 and True compare equal but promote differently
     return x
 
 
 _IMPURE = {"rand_like", "randn_like", "native_dropout", "bernoulli", "rand", "randn", "randint", "randperm",
            "normal", "uniform", "dropout"}
+# fresh storage on every call: two of these must stay two tensors (something may write into one later)
+_FACTORIES = {"empty", "empty_like", "empty_strided", "new_empty", "new_empty_strided", "new_zeros", "new_ones",
+              "new_full", "zeros", "ones", "full", "zeros_like", "ones_like", "full_like", "clone", "arange"}
+
+
+def _mergeable(node: Node) -> bool:
+    """A pure function of its operands: not random, not a factory, and no mutable / out-variant schema."""
+    name = target_name(node.target)
+    if name in _IMPURE or name in _FACTORIES or name.endswith("_"):
+        return False
+    schema = getattr(node.target, "_schema", None)
+    if schema is not None and getattr(schema, "is_mutable", False):
+        return False
+    return True
+
 
 
 def pass_cse(module: GraphModule, graph: Graph = None) -> GraphModule:
     """Common-subexpression elimination over pure call_function nodes: a node
     with the same target and the same (already merged) operands as an earlier
-    one is replaced by it.  Random ops never merge."""
+    one is replaced by it.  Random ops, factory ops and ops with a mutable schema
+    never merge, and Python scalars are keyed with their type."""
     graph = module.graph
     seen: Dict[tuple, Node] = {}
     for node in list(graph.nodes):
-        if node.op != "call_function" or target_name(node.target) in _IMPURE or node.meta.get("evt"):
+        if node.op != "call_function" or not _mergeable(node) or node.meta.get("evt"):
             continue
         try:
             key = (node.target, _freeze(node.args), _freeze(node.kwargs))

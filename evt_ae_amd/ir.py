@@ -206,7 +206,8 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
 
     `elem_strides` are the memory strides of the tensor (default: contiguous).
     Returns None when the mapping is not of that form (checked on the corners,
-    the unit steps and a few thousand random points)."""
+    the unit steps, a few thousand random points and every point of the lines
+    along l, m and n through six anchors)."""
     shape = coord.shape
     if elem_strides is None:
         elem_strides = []
@@ -243,6 +244,19 @@ def fit_strides(coord: Coord, L: int, M: int, N: int, elem_strides: Optional[Seq
     pn = rng.integers(0, N, npts)
     # always include the far corner
     pl[0], pm[0], pn[0] = L - 1, M - 1, N - 1
+    # ... and whole lines along each axis through a few anchors (the corners and two random points), so that a
+    # mapping that leaves the affine form only in a late column / row / batch cannot slip through the sample:
+    # O(L + M + N) points
+    anchors = [(0, 0, 0), (L - 1, M - 1, N - 1), (L - 1, 0, N - 1), (0, M - 1, 0),
+               (int(pl[1]), int(pm[1]), int(pn[1])), (int(pl[2]), int(pm[2]), int(pn[2]))]
+    ll, mm, nn = [pl], [pm], [pn]
+    for al, am, an in anchors:
+        for axis, size in ((0, L), (1, M), (2, N)):
+            line = np.arange(size, dtype=np.int64)
+            ll.append(line if axis == 0 else np.full(size, al, dtype=np.int64))
+            mm.append(line if axis == 1 else np.full(size, am, dtype=np.int64))
+            nn.append(line if axis == 2 else np.full(size, an, dtype=np.int64))
+    pl, pm, pn = np.concatenate(ll), np.concatenate(mm), np.concatenate(nn)
     want = offset(pl, pm, pn)
 
     def fits(st: Strides) -> bool:

@@ -22,7 +22,7 @@ import threading
 from pathlib import Path
 from typing import Dict, Optional
 
-from .codegen import KernelSpec, generate
+from .codegen import ABI_VERSION, KernelSpec, generate
 from .ir import EpilogueIR
 
 PKG_DIR = Path(__file__).resolve().parent
@@ -31,7 +31,7 @@ INCLUDE_DIR = PKG_DIR.parent / "include"
 KERNEL_DIR = Path(os.environ.get("EVT_KERNEL_DIR", PKG_DIR / "_kernels"))
 CACHE_FILE = KERNEL_DIR / "compiled_cache.db"
 
-EVT_ABI_VERSION = 3
+EVT_ABI_VERSION = ABI_VERSION
 EVT_MAX_TENSORS = 16
 EVT_MAX_SCALARS = 16
 
@@ -57,8 +57,11 @@ class EvtArgs(ctypes.Structure):
                 ("batch_div_A", ctypes.c_int64), ("batch_stride2_A", ctypes.c_int64),
                 ("batch_div_B", ctypes.c_int64), ("batch_stride2_B", ctypes.c_int64),
                 ("num_tensors", ctypes.c_int32), ("num_scalars", ctypes.c_int32),
+                ("split_k", ctypes.c_int32), ("flags", ctypes.c_int32),
                 ("tensors", EvtTensorArg * EVT_MAX_TENSORS), ("scalars", ctypes.c_float * EVT_MAX_SCALARS)]
 
+
+EVT_FLAG_TWO_KERNEL_REDUCE = 1
 
 ERROR_NAMES = {-1: "EVT_ERR_BAD_ARGS", -2: "EVT_ERR_ALIGNMENT", -3: "EVT_ERR_WORKSPACE", -4: "EVT_ERR_RANGE",
                -5: "EVT_ERR_SCRATCH"}
@@ -261,57 +264,3 @@ def registered_modules():
 
 def build_module(ir: EpilogueIR, spec: KernelSpec, force: bool = False) -> Path:
     return load_module(ir, spec).build(force)
-
-
-# ---------------------------------------------------------------------------
-# measurement aid: register-only MFMA loop (csrc/mfma_ceiling_probe.hip)
-# ---------------------------------------------------------------------------
-
-class MfmaProbe:
-    """Builds / loads the MFMA ceiling probe and runs it on operand data of the
-    caller's choice.  Used by bench.py to report what the matrix cores sustain
-    on data like the benchmark's, next to the published peak."""
-
-    SOURCE = CSRC_DIR / "mfma_ceiling_probe.hip"
-
-    def __init__(self):
-        text = self.SOURCE.read_text()
-        h = hashlib.sha256((text + " ".join(HIPCC_FLAGS)).encode()).hexdigest()[:20]
-        self.path = KERNEL_DIR / f"mfma_probe_{h}.so"
-        self._text = text
-        self._lib = None
-
-    def build(self, force: bool = False) -> Path:
-        if force or not self.path.exists():
-            compile_source(self._text, self.path)
-        return self.path
-
-    def run(self, operands, workgroups: int = 256, iters: int = 1 << 15, warm_launches: int = 6):
-        """operands: CUDA fp16 tensor of >= 65536 elements.  Returns (TFLOP/s, shader MHz)
-        of the last of `warm_launches` + 1 back-to-back launches."""
-        import torch
-        if self._lib is None:
-            self.build()
-            self._lib = ctypes.CDLL(str(self.path), mode=ctypes.RTLD_LOCAL)
-            self._lib.evt_mfma_probe_launch.restype = ctypes.c_int
-            self._lib.evt_mfma_probe_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
-                                                        ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
-        if operands.dtype != torch.float16 or operands.numel() < 65536 or not operands.is_contiguous():
-            raise ValueError("operands: contiguous fp16 tensor of at least 65536 elements")
-        sink = torch.zeros(1024, dtype=torch.float32, device=operands.device)
-        clk = torch.zeros(2, dtype=torch.int64, device=operands.device)
-        stream = torch.cuda.current_stream().cuda_stream
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for i in range(warm_launches + 1):
-            if i == warm_launches:
-                e0.record()
-            rc = self._lib.evt_mfma_probe_launch(operands.data_ptr(), sink.data_ptr(), clk.data_ptr(), workgroups, iters,
-                                                 ctypes.c_void_p(stream))
-            if rc != 0:
-                raise RuntimeError(f"HIP Error {rc} launching the MFMA probe")
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        cycles, ticks = (int(x) for x in clk.cpu())
-        flops = workgroups * 8 * iters * 8 * 32768.0
-        return flops / (ms * 1e-3) / 1e12, 100.0 * cycles / max(ticks, 1)

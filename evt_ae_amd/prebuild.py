@@ -144,7 +144,6 @@ def build_all(jobs: int = 8, force: bool = False, verbose: bool = True) -> List[
         for m, _ in zip(todo, pool.map(lambda mod: mod.build(force=force), todo)):
             if verbose:
                 print(f"[prebuild] built {m.name} -> {m.path.name}", flush=True)
-    jit.MfmaProbe().build(force)
     if verbose:
         print(f"[prebuild] done in {time.time() - t0:.1f}s", flush=True)
     return mods

@@ -28,9 +28,14 @@
 extern "C" {
 #endif
 
-#define EVT_ABI_VERSION 3
+#define EVT_ABI_VERSION 4
 #define EVT_MAX_TENSORS 16
 #define EVT_MAX_SCALARS 16
+
+/* EvtArgs.flags: finish every cross-tile reduction in the separate finalize
+ * kernel, also where the last workgroup to arrive could do it inside the GEMM
+ * kernel (a test switch: both forms give the same bits). */
+#define EVT_FLAG_TWO_KERNEL_REDUCE 1
 
 /* Error codes returned by evt_launch / evt_workspace_bytes (negative); a
  * positive value is a hipError_t reported by the runtime at launch. */
@@ -60,8 +65,8 @@ extern "C" {
  * A slot the module spec lists with kind "rand" (rand_like) has no storage:
  * `ptr` is ignored and the strides give the element index e that seeds the
  * generator -- the value is word (e & 3) of Philox4x32-10(counter = (e >> 2
- * as two words, offset, slot index), key = seed), mapped to [0, 1) as
- * (word >> 8) * 2^-24.  Takes the place of VisitorRand's {seed, offset}
+ * as two words, offset, slot index + 16 * stream id), key = seed), mapped to
+ * [0, 1) as (word >> 8) * 2^-24.  Takes the place of VisitorRand's {seed, offset}
  * arguments (visitor_load.hpp:79-151). */
 typedef struct EvtTensorArg {
   void* ptr;
@@ -116,10 +121,20 @@ typedef struct EvtArgs {
   int64_t batch_stride2_B;
   int32_t num_tensors;
   int32_t num_scalars;
+  /* Split-K of a GEMM module: 0 = the module decides (splits only when the
+   * output tiles cannot fill the chip, K is long and the output is small),
+   * 1 = never, n >= 2 = n splits (capped at the number of k-tiles).  The
+   * workspace size depends on it: pass the same value to evt_workspace_bytes
+   * and evt_launch.  Row-wise modules ignore it. */
+  int32_t split_k;
+  /* EVT_FLAG_* bits. */
+  int32_t flags;
   EvtTensorArg tensors[EVT_MAX_TENSORS];
   /* immediates of the epilogue, in module-spec order.  A module with a "rand"
    * slot reads four of them as 32-bit patterns, not as float values:
-   * scalars[rng_scalars + 0..2] = seed low word, seed high word, offset. */
+   * scalars[rng_scalars + 0..3] = seed low word, seed high word, offset,
+   * stream id (below 2^28; distinct per fused op, so that two ops whose
+   * rand_like tensors have equal shapes draw unrelated numbers). */
   float scalars[EVT_MAX_SCALARS];
 } EvtArgs;
 

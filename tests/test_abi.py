@@ -43,10 +43,10 @@ def test_every_built_module_exports_the_abi():
         for sym in declared_symbols():
             assert hasattr(lib, sym), f"{p.name} lacks {sym}"
         lib.evt_abi_version.restype = ctypes.c_int
-        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 3
+        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 4
         lib.evt_module_spec.restype = ctypes.c_char_p
         spec = json.loads(lib.evt_module_spec().decode())
-        assert spec["abi"] == 3
+        assert spec["abi"] == 4
         if "anchor" in spec:      # row-wise reduce-apply module
             assert spec["anchor"] in ("softmax", "softmax_backward", "layernorm", "layernorm_backward")
             assert spec["element"] in ("f16", "bf16", "f32") and spec["row"]["max_n"] >= 1

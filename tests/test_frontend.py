@@ -164,6 +164,35 @@ def test_random_patterns_lower_correctly():
     assert abs(keep - 0.3) < 5e-3
 
 
+def test_two_dropout_partitions_draw_unrelated_masks():
+    """Two fused ops whose rand_like tensors have the same shape (the hidden
+    dropouts of two layers) must not share a random stream: same seed, same
+    offset, same slot index, yet different masks -- every op mixes a stream id
+    of its own into the generator's counter.  And the seed is read when the op
+    is called, so torch.manual_seed after tracing still takes effect."""
+    g = torch.Generator().manual_seed(7)
+    h = lambda *s: (torch.randn(*s, generator=g) * 0.5).half()   # noqa: E731
+    inputs = [h(1024, 32), h(1024, 32), h(1024), h(512, 2, 1024)]
+    ops = []
+    for _ in range(2):
+        gm = W.fuse(W.Dropout1(), inputs)
+        (n,) = fused_nodes(gm)
+        ops.append((gm, n.target))
+    assert ops[0][1].rand_stream != ops[1][1].rand_stream
+    torch.manual_seed(1234)
+    masks = []
+    for gm, op in ops:
+        got = run_emulated(gm, inputs)
+        assert op.last_rand_state == (1234, 0)
+        masks.append([o for o in got if o.dtype == torch.bool][-1])
+    assert not torch.equal(masks[0], masks[1])
+    agree = (masks[0] == masks[1]).float().mean().item()      # independent masks with keep rate 0.3 agree on 58 %
+    assert abs(agree - (0.3 * 0.3 + 0.7 * 0.7)) < 1e-2
+    torch.manual_seed(99)                                      # after tracing: a new seed, new numbers
+    again = [o for o in run_emulated(ops[0][0], inputs) if o.dtype == torch.bool][-1]
+    assert ops[0][1].last_rand_state == (99, 1)
+
+
 def test_pass_decomposition_rewrites():
     """The reference's Decomposition replacements this path depends on
     (pass_decomposition.py:280-502): same values after the rewrite, the targeted
@@ -272,7 +301,7 @@ def test_row_anchor_patterns_trace(name):
     assert K == 1 and N == inputs[0].shape[-1] and L * M * N == inputs[0].numel()
     assert op.row_spec.max_n >= N and op.row_spec.lpr in (8, 16, 32, 64) and 1 <= op.row_spec.ch <= 16
     spec = op.module.spec
-    assert spec["abi"] == 3 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
+    assert spec["abi"] == 4 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
     assert op.num_anchor_inputs == {"softmax": 1, "softmax_backward": 2, "layernorm": 1, "layernorm_backward": 5}[kind]
     if kind == "layernorm":
         # eps travels as a scalar; mean and rstd are per-row stores

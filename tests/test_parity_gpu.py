@@ -111,6 +111,48 @@ def test_reductions_are_deterministic_and_workspace_reusable():
                 assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("cfg,shapes", [(3, None), (4, None), (3, W.SPLIT_K_SHAPES[3])],
+                         ids=["row_finalize", "column_finalize", "split_k"])
+def test_exchange_between_workgroups_holds_over_many_launches(cfg, shapes):
+    """Regression guard for the exchange of partial results between workgroups
+    inside one kernel (device-scope stores, the wait for their acknowledgement,
+    a relaxed arrival ticket, device-scope loads by the last arriver): 2000
+    back-to-back launches on one shared workspace -- config 3 at full size (the
+    last workgroup of a row block finishes the row statistics), config 4 at full
+    size (per-column sums) and a split-K shape (accumulator tiles exchanged) --
+    each compared bit for bit with the first launch; stops at the first mismatch."""
+    wl = W.CONFIGS[cfg]
+    inputs = W.make_inputs(cfg, shapes)
+    gm = W.fuse(wl.module(), [t.to("meta") for t in inputs])
+    (node,) = fused_nodes(gm)
+    op = node.target
+    placeholders = [n for n in gm.graph.nodes if n.op == "placeholder"]
+    args = [inputs[placeholders.index(a)].cuda() for a in node.args]
+    stream = torch.cuda.current_stream()
+    module = op.module.ensure()
+    batch, launches = 20, 2000
+    sets = []
+    for _ in range(batch + 1):
+        stores = op.allocate_outputs("cuda")
+        a, keep = op.build_arguments(stores, *args, block=op.new_argument_block())
+        sets.append((stores, a, keep))
+    ws_ptr, ws_bytes = op.workspace_for(sets[0][1], stream, "cuda")
+    assert ws_bytes > 0
+    module.launch(sets[batch][1], ws_ptr, ws_bytes, stream.cuda_stream)       # the reference launch
+    torch.cuda.synchronize()
+    first = sets[batch][0]
+    done = 1
+    while done < launches:
+        for stores, a, _ in sets[:batch]:
+            module.launch(a, ws_ptr, ws_bytes, stream.cuda_stream)
+        torch.cuda.synchronize()
+        for i, (stores, _, _) in enumerate(sets[:batch]):
+            for name, t in stores.items():
+                assert torch.equal(t.view(torch.uint8), first[name].view(torch.uint8)), \
+                    f"config {cfg}: launch {done + i} differs from the first in '{name}'"
+        done += batch
+
+
 PATTERN_ATOL = 2e-1   # the reference's own criterion (unittest/evt_fuser/mm.py:28, bmm.py:27)
 
 

@@ -32,7 +32,7 @@ def emulate_fused(op: FusedOpBase, *args):
             numel = 1
             for d in slot.shape:
                 numel *= d
-            loads[k] = torch.from_numpy(philox.uniform(op.rand_seed, op.rand_offset, k, numel))
+            loads[k] = torch.from_numpy(philox.uniform(op.rand_seed, op.rand_offset, op.rand_salt(k), numel))
     if op.ir.rng_scalar is not None:
         op.last_rand_state = (op.rand_seed, op.rand_offset & 0xFFFFFFFF)
         op.rand_offset += 1
@@ -77,6 +77,6 @@ def run_emulated(gm, inputs):
 
 
 def rand_slot(op: FusedOpBase) -> int:
-    """Index (= generator salt) of the op's single rand_like slot."""
+    """Generator salt (slot index + 16 x the op's stream id) of the op's single rand_like slot."""
     (k,) = [k for k, s in enumerate(op.ir.slots) if s.kind == "rand"]
-    return k
+    return op.rand_salt(k)
