@@ -86,7 +86,7 @@ def main():
     mods = []
     for cfg, t in tuners:
         for tile in t.candidates():
-            mods.append(jit.load_module(t.ir, KernelSpec(t.a_kc, t.b_kc, t.bf16, tile)))
+            mods.append(jit.load_module(t.ir, KernelSpec.for_problem(t.K, t.a_kc, t.b_kc, t.bf16, tile)))
     todo = [m for m in mods if not m.path.exists()]
     print(f"[tune] {len(mods)} candidate modules, {len(todo)} to compile", flush=True)
     with ThreadPoolExecutor(args.jobs) as pool:

@@ -16,7 +16,7 @@ import json
 import os
 import sqlite3
 from contextlib import contextmanager
-from dataclasses import asdict, fields
+from dataclasses import asdict, fields, replace
 from pathlib import Path
 from typing import List, Optional, Sequence, Tuple
 
@@ -128,6 +128,11 @@ class AutoTunerBase:
                            # two stages: 64 KB of LDS, so two such workgroups share a CU and one's epilogue runs
                            # under the other's main loop (measured 12-17 % faster than four stages on 128 x 128)
                            (128, 128, 64, 4, 2, 2, pipe), (128, 128, 64, 2, 4, 2, pipe)]
+            # options of the one-barrier ping-pong loop (pipe 4 + flags, see TileConfig.pipe)
+            for pipe in (5, 6, 7):
+                shapes += [(256, 256, 64, 4, 2, 2, pipe), (256, 256, 64, 2, 4, 2, pipe)]
+            for pipe in (5, 6, 7, 8, 10):
+                shapes += [(256, 128, 64, 4, 2, 3, pipe), (128, 256, 64, 2, 4, 3, pipe)]
             if self.N == 512:     # one tile spans the rows: row statistics complete inside the workgroup
                 shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0),
                            # 32 x 256 wave tiles: 8 columns per lane halve the cross-lane steps per element of a
@@ -143,11 +148,28 @@ class AutoTunerBase:
             t = TileConfig(bm, bn, bk, wm, wn, st, self.dma, 4, pipe)
             if self.fits(t) and t not in out:
                 out.append(t)
+        # many more tiles than CUs: workgroups that walk over 2, 4 or 8 tiles of a row block (ping-pong tiles
+        # with two or three stages; fits() knows the other conditions), as long as every CU still gets one
+        for t in list(out):
+            tiles_n = -(-self.N // t.bn)
+            tiles = -(-self.M // t.bm) * tiles_n * self.L
+            if t.pipe in (2, 3) and t.stages <= 3 and tiles >= 4 * NUM_CUS:
+                for walk in (2, 4, 8):
+                    tw = replace(t, walk=walk)
+                    if walk <= tiles_n and tiles // walk >= NUM_CUS and self.fits(tw) and tw not in out:
+                        out.append(tw)
         return out
 
     def fits(self, t: TileConfig) -> bool:
         """The tile's stages fit the LDS and hold this epilogue's reduction exchange area."""
-        return reduction_lds_bytes(t, self.ir.row_state, self.ir.col_state) <= t.lds_bytes() <= LDS_LIMIT
+        need = reduction_lds_bytes(t, self.ir.row_state, self.ir.col_state)
+        if t.walk > 1:
+            # the epilogue's exchange area is the one stage the ring leaves free between tiles; the running row
+            # states sit behind the stages
+            return (t.pipe >= 2 and not self.ir.col_state and need <= t.stage_bytes()
+                    and self.K % t.bk == 0 and self.K // t.bk >= t.stages
+                    and t.lds_bytes() + t.bm * max(1, self.ir.row_state) * 4 <= LDS_LIMIT)
+        return need <= t.lds_bytes() <= LDS_LIMIT
 
     def heuristic(self) -> TileConfig:
         """Pick the candidate with the lowest modelled time: number of
@@ -155,7 +177,7 @@ class AutoTunerBase:
         eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3}
         best, best_cost = None, None
         for t in self.candidates():
-            if t.pipe not in (0, 2) or t.stages == 1:
+            if t.pipe not in (0, 2) or t.stages == 1 or t.walk > 1:
                 continue    # untuned default: a ping-pong tile or the plain double-buffered ring
             tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
             wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 else 1
@@ -222,7 +244,7 @@ class AutoTunerBase:
 
     def profile(self, tile: TileConfig) -> float:
         from .. import jit
-        module = jit.load_module(self.ir, KernelSpec(self.a_kc, self.b_kc, self.bf16, tile))
+        module = jit.load_module(self.ir, KernelSpec.for_problem(self.K, self.a_kc, self.b_kc, self.bf16, tile))
         sets = self.argument_sets()
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = module.workspace_bytes(sets[0][0])

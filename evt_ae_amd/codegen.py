@@ -34,13 +34,21 @@ class TileConfig:
     # 3: ping-pong with one barrier per k-tile; 4 + flags: as 3 with 1 = the barrier inside group 0's MFMA phase,
     # 2 = group 0 issues its transfers between its LDS reads, 4 = group 1 as well (stages >= 3)
     pipe: int = 0
+    # > 1: a workgroup computes this many consecutive tiles of a row block, the operand ring running on from one
+    # into the next, and per-row reductions leave one partial per workgroup (ping-pong pipelines, no per-column
+    # reduction in the epilogue); pays when the tiles outnumber the CUs several times
+    walk: int = 1
 
     def tag(self) -> str:
         return (f"{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_s{self.stages}"
-                f"_{'dma' if self.dma else 'safe'}_g{self.group_m}" + (f"_p{self.pipe}" if self.pipe else ""))
+                f"_{'dma' if self.dma else 'safe'}_g{self.group_m}" + (f"_p{self.pipe}" if self.pipe else "")
+                + (f"_n{self.walk}" if self.walk > 1 else ""))
+
+    def stage_bytes(self) -> int:
+        return (self.bm + self.bn) * self.bk * 2
 
     def lds_bytes(self) -> int:
-        return self.stages * (self.bm + self.bn) * self.bk * 2
+        return self.stages * self.stage_bytes()
 
 
 @dataclass(frozen=True)
@@ -49,6 +57,16 @@ class KernelSpec:
     b_kc: bool          # B contiguous along K (column-major, i.e. stored [N, K])
     bf16: bool
     tile: TileConfig
+    # K is a multiple of the tile's bk for every launch of the module: the global -> LDS transfers then carry no
+    # per-lane test against K (measured 2-3 % on 8192 x 1024 x 4096)
+    k_exact: bool = False
+
+    @staticmethod
+    def for_problem(K: int, a_kc: bool, b_kc: bool, bf16: bool, tile: TileConfig) -> "KernelSpec":
+        return KernelSpec(a_kc, b_kc, bf16, tile, bool(tile.dma and K % tile.bk == 0))
+
+    def tag(self) -> str:
+        return self.tile.tag() + ("_kx" if self.k_exact else "")
 
 
 def reduction_lds_bytes(t: "TileConfig", row_state: int, col_state: int) -> int:
@@ -195,6 +213,8 @@ class Codegen:
         raise NotImplementedError(n.op)
 
     def slot_off(self, k: int, batch: str = "t.batch") -> str:
+        if batch == "t.batch" and getattr(self, "_tile_offsets", False):
+            return f"bo_{k}"      # computed once at the top of tile()
         return f"evt::batch_offset({batch}, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2)"
 
     # -- sections ---------------------------------------------------------------
@@ -301,6 +321,21 @@ class Codegen:
         e("constexpr int MI = Cfg::MI, NI = Cfg::NI;")
         if row_reds or col_reds:
             e("__syncthreads();  // all waves are done reading the last operand tile from LDS")
+        # each tensor's batch offset once per tile (it holds a division; left inside the row loops it is redone
+        # for every row)
+        for k in range(len(ir.slots)):
+            e(f"[[maybe_unused]] const int64_t bo_{k} = evt::batch_offset(t.batch, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2);")
+        self._tile_offsets = True
+        # one value per row (column vectors): check-free path through buffer loads, the row's offset in a scalar
+        col_loads = sorted({ir.nodes[n].slot for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "col"})
+        for k in col_loads:
+            e(f"[[maybe_unused]] __amdgpu_buffer_rsrc_t rc_{k};")
+            e(f"[[maybe_unused]] uint32_t vc_{k} = 0;")
+            e(f"[[maybe_unused]] const uint32_t cp_{k} = (uint32_t)p.t{k}_sm * (uint32_t)sizeof(*p.t{k});")
+            e("if constexpr (FAST) {")
+            e(f"  rc_{k} = evt::make_rsrc((const char*)(p.t{k} + bo_{k} + (int64_t)t.row_u * p.t{k}_sm));")
+            e(f"  vc_{k} = (uint32_t)(t.row_l * (int)p.t{k}_sm) * (uint32_t)sizeof(*p.t{k});")
+            e("}")
         # hoisted values
         for name in hoisted:
             self.emit_node(e, ir.nodes[name], hoisted=True)
@@ -495,6 +530,7 @@ class Codegen:
         e("(void)p; (void)t; (void)g; (void)acc;")
         e.dedent()
         e("}")
+        self._tile_offsets = False
 
     def emit_tile_store(self, e: _Emitter, k: int, arr: str):
         """Store the NI values `arr` of row (mi, v) to tile slot k (inside the row loops)."""
@@ -534,7 +570,10 @@ class Codegen:
                 if hoisted:   # depends on the batch only
                     e(f"const float {c} = evt::ld_f32(p.t{k}, {base});")
                 else:
-                    e(f"const float {c} = rok ? evt::ld_f32(p.t{k}, {base} + (int64_t)row * p.t{k}_sm) : 0.f;")
+                    ct = DTYPE_CTYPES[s.dtype]
+                    e(f"float {c};")
+                    e(f"if constexpr (FAST) {c} = evt::buffer_ld_f32<{ct}>(rc_{k}, vc_{k}, (uint32_t)Tile::row_step(mi, v) * cp_{k});")
+                    e(f"else {c} = rok ? evt::ld_f32(p.t{k}, {base} + (int64_t)row * p.t{k}_sm) : 0.f;")
             else:
                 e(f"const float {c} = evt::ld_f32(p.t{k}, 0);")
         elif n.op == "rres":
@@ -569,7 +608,8 @@ class Codegen:
             e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) mx = t.col_ok(ni) ? fmaxf(mx, {x}) : mx;")
             e("mx = evt::half_wave_max(mx);")
             e("float se = 0.f;")
-            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) se += t.col_ok(ni) ? evt::op_exp({x} - mx) : 0.f;")
+            e("const float mxs = mx * evt::kLog2e;")
+            e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) se += t.col_ok(ni) ? evt::op_exp_minus({x}, mxs) : 0.f;")
             e(f"rst[{o}] = mx; rst[{o + 1}] = evt::half_wave_sum(se);")
         elif r.kind == "welford":
             e("const float cnt = wcnt;")
@@ -592,6 +632,7 @@ class Codegen:
             "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
             "tile": asdict(t),
             "a_k_contiguous": self.spec.a_kc,
+            "k_multiple_of": self.spec.tile.bk if self.spec.k_exact else 1,   # launches with another K are refused
             "b_k_contiguous": self.spec.b_kc,
             "element": "bf16" if self.spec.bf16 else "f16",
             "batched": self.ir.batched,
@@ -633,12 +674,16 @@ class Codegen:
         e("};")
         b = lambda x: "true" if x else "false"  # noqa: E731
         tile_io = any((sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux") for sl in ir.slots)
+        if t.walk > 1 and (t.pipe < 2 or not t.dma or ir.col_state or not sp.k_exact):
+            raise NotImplementedError("a walk over tiles needs a ping-pong pipeline, K a multiple of bk and an epilogue "
+                                      "without per-column reduction")
         e(f"using Cfg = evt::GemmCfg<{t.bm}, {t.bn}, {t.bk}, {t.wm}, {t.wn}, {b(sp.a_kc)}, {b(sp.b_kc)}, "
-          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}, {t.pipe}, {b(tile_io)}>;")
+          f"{b(t.dma)}, {t.stages}, {b(sp.bf16)}, {t.group_m}, {t.pipe}, {b(tile_io)}, {b(t.walk > 1)}, {b(sp.k_exact)}>;")
         e(f"constexpr int kNumTensors = {len(ir.slots)};")
         e(f"constexpr int kNumScalars = {len(ir.scalars)};")
         red_lds = reduction_lds_bytes(t, ir.row_state, ir.col_state)
-        e(f"static_assert(Cfg::LDS_BYTES >= {red_lds}, \"reduction exchange area exceeds the operand LDS\");")
+        e(f"static_assert((Cfg::WALK ? Cfg::STAGE_BYTES : Cfg::LDS_BYTES) >= {red_lds}, "
+          "\"reduction exchange area exceeds the operand LDS\");")
         e("")
         e("int fill(const EvtArgs* a, evt::GemmArgs& g, Epi::Params& p) {")
         e.indent()
@@ -655,6 +700,10 @@ class Codegen:
         e("g.bdivB = a->batch_div_B > 1 ? (int)a->batch_div_B : 1; g.bs2B = a->batch_div_B > 1 ? a->batch_stride2_B : 0;")
         e("g.tiles_m = (a->M + Cfg::BM - 1) / Cfg::BM;")
         e("g.tiles_n = (a->N + Cfg::BN - 1) / Cfg::BN;")
+        e("// tiles per workgroup along a row block (Cfg::WALK); the ring needs a full set of k-tiles to carry over")
+        e("if (Cfg::K_EXACT && a->K % Cfg::BK) return EVT_ERR_ALIGNMENT;   // this module has no code for a partial k-tile")
+        e(f"g.walk = (Cfg::WALK && a->K / Cfg::BK >= Cfg::STAGES) ? {t.walk} : 1;")
+        e("g.parts_n = (g.tiles_n + g.walk - 1) / g.walk;")
         e("g.workspace = nullptr;")
         e("g.row_fold_mod = 0; g.row_fold_step = 1; g.row_fold_count = 1;")
         folds = {(r.fold) for r in ir.reduces.values() if r.axis == "row"}
@@ -670,7 +719,8 @@ class Codegen:
                 e("  if (x.l_mod != 0 || x.l_div <= 1 || a->L % x.l_div) return EVT_ERR_BAD_ARGS;")
                 e("  g.row_fold_count = (int)x.l_div; }")
         e("// few partials: the last workgroup to arrive combines them; many: a finalize kernel does")
-        e("g.row_inkernel = (g.tiles_n * g.row_fold_count <= evt::kMaxInKernelPartials && !two_kernel_reduce) ? 1 : 0;")
+        e("g.row_inkernel = (g.parts_n * g.row_fold_count <= evt::kMaxInKernelRowPartials && !two_kernel_reduce && "
+          "(int64_t)g.parts_n * a->M * Epi::ROW_STATE * 4 < 0x7fffffffLL) ? 1 : 0;   // the last arriver reads with 32-bit offsets")
         e("g.col_fold_step = 1; g.col_fold_count = 1;")
         col_folds = {r.fold for r in ir.reduces.values() if r.axis == "col"} - {""}
         if col_folds:
@@ -685,7 +735,7 @@ class Codegen:
         e("// Split-K: when the output tiles cannot fill the chip and K is long, several workgroups share a tile")
         e("// (EvtArgs.split_k: 0 = decide here, 1 = off, n = n splits)")
         e("g.splits = 1; g.k_chunk = (a->K + Cfg::BK - 1) / Cfg::BK * Cfg::BK;")
-        if t.stages > 1:
+        if t.stages > 1 and t.walk == 1:
             e("{")
             e("  const int want = a->split_k;")
             e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
@@ -739,10 +789,12 @@ class Codegen:
         e("for (int i = 0; i < kNumScalars; ++i) p.s[i] = a->scalars[i];")
         tile_slots = [k for k, sl in enumerate(ir.slots)
                       if (sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux")]
+        col_slots = [k for k, sl in enumerate(ir.slots) if sl.role == "load" and sl.kind == "col"]
         cond = " && ".join(
             [f"(p.t{k}_vec & 1) && (!(Cfg::ADJACENT && sizeof(*p.t{k}) == 2 && (Cfg::NI == 2 || Cfg::NI == 4 || Cfg::NI == 8)) || (p.t{k}_vec & 2))"
              f" && p.t{k}_sm >= 0 && p.t{k}_sm < (1 << 20)"
-             for k in tile_slots]) or "true"
+             for k in tile_slots] +
+            [f"p.t{k}_sm >= 0 && p.t{k}_sm < (1 << 20)" for k in col_slots]) or "true"
         e(f"p.fast = ({cond}) ? 1 : 0;")
         e("return EVT_OK;")
         e.dedent()
@@ -767,7 +819,7 @@ class Codegen:
         e("}")
         e("static int enqueue(evt::GemmArgs& g, const Epi::Params& p, void* ws, void* stream) {")
         e("  g.workspace = (char*)ws;")
-        e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.tiles_n * g.L * g.splits);")
+        e("  const unsigned grid = (unsigned)((int64_t)g.tiles_m * g.parts_n * g.L * g.splits);")
         e("  hipLaunchKernelGGL((evt::evt_gemm_kernel<Cfg, Epi>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  const int err = (int)hipGetLastError();")
         e("  if (err != 0) return err;")

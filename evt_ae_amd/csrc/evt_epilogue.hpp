@@ -31,6 +31,9 @@ namespace evt {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 EVT_DEV float op_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+// exp(x - m) with m_log2e = m * log2(e) computed once per row: one multiply-add per element in front of the
+// exponential instead of a subtraction and a multiplication
+EVT_DEV float op_exp_minus(float x, float m_log2e) { return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, -m_log2e)); }
 EVT_DEV float op_log(float x) { return __builtin_amdgcn_logf(x) * kLn2; }
 EVT_DEV float op_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 // sigmoid(x) = 1 / (1 + 2^(-x log2 e)); saturates to 0 / 1 for |x| large
@@ -107,12 +110,23 @@ struct TileCtx {
   int tid, lane, wm, wn;
   char* smem;
   char* workspace;
+  // Per-row reductions: this workgroup's partial is number part_n of parts_n along the row.  Without a walk
+  // that is the tile; in a walk (GemmCfg::WALK) the tiles of a workgroup fold into a running state per row,
+  // kept in LDS at walk_state, and the partial leaves with the last tile.
+  int part_n, parts_n;
+  bool walk_first, walk_last;
+  float* walk_state;
 
   EVT_DEV void init(const GemmArgs& g, int batch_, int tm, int tn, char* smem_) {
     M = g.M; N = g.N; L = g.L;
     batch = batch_; tile_m = tm; tile_n = tn; tiles_m = g.tiles_m; tiles_n = g.tiles_n;
+    part_n = tn; parts_n = g.tiles_n; walk_first = walk_last = true; walk_state = nullptr;
     m0 = tm * Cfg::BM; n0 = tn * Cfg::BN;
-    tid = threadIdx.x; lane = tid & 63;
+    tid = threadIdx.x;
+    // walking kernels run main loop and epilogue in turn: keep this lane's indices from being computed once
+    // ahead of the tile loop and carried through every main loop (see Mainloop::run)
+    if constexpr (Cfg::WALK) asm volatile("" : "+v"(tid));
+    lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     wm = wave / Cfg::WN; wn = wave % Cfg::WN;
     row_u = m0 + wm * Cfg::TM; row_l = 4 * (lane >> 5);
@@ -122,6 +136,9 @@ struct TileCtx {
     row0 = row_u + row_l;
     col0 = col_u + col_l;
     smem = smem_; workspace = g.workspace;
+  }
+  EVT_DEV void set_walk(int part, int parts, bool first, bool last, float* state) {
+    part_n = part; parts_n = parts; walk_first = first; walk_last = last; walk_state = state;
   }
   EVT_DEV int row(int mi, int v) const { return row0 + mi * 32 + 8 * (v >> 2) + (v & 3); }
   // row of register (mi, v) relative to row0: a compile-time constant once the loops are unrolled
@@ -238,6 +255,20 @@ EVT_DEV T buffer_load_elem(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t so
   else if constexpr (sizeof(T) == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b16(rs, voff, soff, 0));
   else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b8(rs, voff, soff, 0));
 }
+// One value per row (a column vector of the epilogue) through the buffer path of the check-free epilogue:
+// `rs` starts at the wave's first row, voff is this lane's byte offset, soff the row's (wave-uniform).
+template <class T>
+EVT_DEV float buffer_ld_f32(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+  if constexpr (sizeof(T) == 8) {
+    const u32x2 raw = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs, voff, soff, 0));
+    return (float)__builtin_bit_cast(T, raw);
+  } else if constexpr (sizeof(T) == 1) {   // bool
+    return buffer_load_elem<uint8_t>(rs, voff, soff) ? 1.f : 0.f;
+  } else {
+    return (float)buffer_load_elem<T>(rs, voff, soff);
+  }
+}
+
 template <class Tile, class T>
 EVT_DEV void row_load(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, T (&out)[Tile::NI]) {
   constexpr int NI = Tile::NI;
@@ -426,13 +457,18 @@ EVT_DEV float half_wave_max(float x) {
 // ---------------------------------------------------------------------------
 // workspace layout (bytes): [arrival counters | row partials | column partials]
 //   counters        one int per (batch, row block) and per (batch, column block)
-//   row partials    [L][tiles_n][M][ROW_STATE] floats (only if tiles_n > 1)
+//   row partials    [L][parts_n][M][ROW_STATE] floats (only if parts_n > 1; parts_n = tiles_n unless workgroups walk)
 //   column partials [L][tiles_m][N][COL_STATE] floats (only if tiles_m > 1)
 // The counters must be zero before the first launch (evt_workspace_init); a
 // launch leaves them zero.  Partials are written before they are read by
 // every launch.
 // ---------------------------------------------------------------------------
+// Phase 2 inside the GEMM kernel pays for few partials.  The last workgroup of a row block pays a ticket round
+// trip, one round trip for the partials and their combination on one CU, while everybody else is done; measured
+// on 1024 x 131072 (64 partials of three floats per row, 256 rows per block): 6.7 us slower than the finalize
+// kernel, which spreads the same work over the chip.  Column partials are one or two floats and fold cheaply.
 constexpr int kMaxInKernelPartials = 64;
+constexpr int kMaxInKernelRowPartials = 16;
 
 struct WsLayout {
   int64_t counter_bytes, row_bytes, col_bytes;
@@ -442,7 +478,7 @@ struct WsLayout {
 
 // a per-row reduction goes through the workspace when several tiles span the
 // row or several batches fold into one result
-__host__ __device__ inline bool row_uses_workspace(const GemmArgs& g) { return g.tiles_n > 1 || g.row_fold_count > 1; }
+__host__ __device__ inline bool row_uses_workspace(const GemmArgs& g) { return g.parts_n > 1 || g.row_fold_count > 1; }
 
 template <int ROW_STATE, int COL_STATE>
 __host__ __device__ inline WsLayout ws_layout(const GemmArgs& g) {
@@ -451,7 +487,7 @@ __host__ __device__ inline WsLayout ws_layout(const GemmArgs& g) {
   const bool col = COL_STATE > 0 && (g.tiles_m > 1 || g.col_fold_count > 1);
   const int64_t ncnt = (row ? (int64_t)g.L * g.tiles_m : 0) + (col ? (int64_t)g.L * g.tiles_n : 0);
   w.counter_bytes = (ncnt * 4 + 255) / 256 * 256;
-  w.row_bytes = row ? ((int64_t)g.L * g.tiles_n * g.M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
+  w.row_bytes = row ? ((int64_t)g.L * g.parts_n * g.M * ROW_STATE * 4 + 255) / 256 * 256 : 0;
   w.col_bytes = col ? ((int64_t)g.L * g.tiles_m * g.N * COL_STATE * 4 + 255) / 256 * 256 : 0;
   w.split_counter_bytes = w.split_bytes = 0;
   return w;
@@ -500,6 +536,51 @@ __host__ __device__ inline int col_fold_member(const GemmArgs& g, int key, int j
 // from the coherence point, so neither needs the L2 write-back / invalidate a
 // release / acquire fence would cost.
 EVT_DEV void st_device(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// N consecutive floats at byte offset `voff` of `rs` with the same cache policy (sc1: written through to, read
+// from the point where the XCDs' L2s meet), in accesses of up to 16 bytes.  A state of three floats moved word by
+// word costs three transactions per cache line, and the reading side, which bypasses its caches, fetches every
+// line three times.
+constexpr int kAuxDevice = 16;   // sc1
+// (a __builtin_bit_cast applied directly to an element of a vector reads the vector's first element with this
+// compiler: the element goes through a scalar first)
+EVT_DEV float word_as_float(uint32_t w) { return __builtin_bit_cast(float, w); }
+template <int N>
+EVT_DEV void st_device_n(__amdgpu_buffer_rsrc_t rs, uint32_t voff, const float* v) {
+  if constexpr (N >= 4) {
+    __builtin_amdgcn_raw_buffer_store_b128(u32x4{__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1]),
+                                                 __builtin_bit_cast(uint32_t, v[2]), __builtin_bit_cast(uint32_t, v[3])},
+                                           rs, voff, 0, kAuxDevice);
+    if constexpr (N > 4) st_device_n<N - 4>(rs, voff + 16, v + 4);
+  } else if constexpr (N == 3) {
+    typedef uint32_t u32x3_t __attribute__((ext_vector_type(3)));
+    __builtin_amdgcn_raw_buffer_store_b96(u32x3_t{__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1]),
+                                                  __builtin_bit_cast(uint32_t, v[2])}, rs, voff, 0, kAuxDevice);
+  } else if constexpr (N == 2) {
+    __builtin_amdgcn_raw_buffer_store_b64(u32x2{__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[1])},
+                                          rs, voff, 0, kAuxDevice);
+  } else if constexpr (N == 1) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[0]), rs, voff, 0, kAuxDevice);
+  }
+}
+template <int N>
+EVT_DEV void ld_device_n(__amdgpu_buffer_rsrc_t rs, uint32_t voff, float* out) {
+  if constexpr (N >= 4) {
+    const u32x4 r = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kAuxDevice);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) out[c] = word_as_float(r[c]);
+    if constexpr (N > 4) ld_device_n<N - 4>(rs, voff + 16, out + 4);
+  } else if constexpr (N == 3) {
+    typedef uint32_t u32x3_t __attribute__((ext_vector_type(3)));
+    const u32x3_t r = __builtin_amdgcn_raw_buffer_load_b96(rs, voff, 0, kAuxDevice);
+#pragma unroll
+    for (int c = 0; c < 3; ++c) out[c] = word_as_float(r[c]);
+  } else if constexpr (N == 2) {
+    const u32x2 r = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs, voff, 0, kAuxDevice));
+    out[0] = word_as_float(r[0]); out[1] = word_as_float(r[1]);
+  } else if constexpr (N == 1) {
+    out[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, voff, 0, kAuxDevice));
+  }
+}
 EVT_DEV float ld_device(const float* p) {
   return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -558,13 +639,32 @@ EVT_DEV int row_reduce_publish(const typename Epi::Params& p, const Tile& t, con
       for (int c = 0; c < RS; ++c) st[c] = lds[lr * RS + c];
 #pragma unroll
       for (int w = 1; w < Cfg::WN; ++w) Epi::row_combine(st, lds + (w * Cfg::BM + lr) * RS);
+      if constexpr (Cfg::WALK) {
+        // fold this tile into the walk's running state, earlier tiles on the left
+        float* run = t.walk_state + lr * RS;
+        if (!t.walk_first) {
+          float sofar[RS];
+#pragma unroll
+          for (int c = 0; c < RS; ++c) sofar[c] = run[c];
+          Epi::row_combine(sofar, st);
+#pragma unroll
+          for (int c = 0; c < RS; ++c) st[c] = sofar[c];
+        }
+        if (!t.walk_last) {
+#pragma unroll
+          for (int c = 0; c < RS; ++c) run[c] = st[c];
+          continue;
+        }
+      }
       if (!row_uses_workspace(g)) {
         Epi::row_finalize(p, t.batch, row, st);
       } else {
-        float* dst = part + (((int64_t)t.batch * t.tiles_n + t.tile_n) * t.M + row) * RS;
-#pragma unroll
-        for (int c = 0; c < RS; ++c) st_device(dst + c, st[c]);
+        st_device_n<RS>(make_rsrc((const char*)(part + ((int64_t)t.batch * t.parts_n + t.part_n) * t.M * RS)),
+                        (uint32_t)row * (RS * 4), st);
       }
+    }
+    if constexpr (Cfg::WALK) {
+      if (!t.walk_last) return -1;
     }
     if (!row_phase2_here<Epi>(g)) return -1;
     return arrive_begin((int*)t.workspace + fold_key(g, t.batch) * t.tiles_m + t.tile_m);
@@ -576,7 +676,10 @@ template <class Cfg, class Epi, class Tile>
 EVT_DEV bool row_reduce_arrived(const Tile& t, const GemmArgs& g, int ticket) {
   if constexpr (Epi::ROW_STATE > 0) {
     if (!row_phase2_here<Epi>(g)) return false;
-    return arrive_end(ticket, t.tiles_n * g.row_fold_count, (int*)(t.smem + Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4));
+    if constexpr (Cfg::WALK) {
+      if (!t.walk_last) return false;
+    }
+    return arrive_end(ticket, t.parts_n * g.row_fold_count, (int*)(t.smem + Cfg::WN * Cfg::BM * Epi::ROW_STATE * 4));
   } else {
     return false;
   }
@@ -600,7 +703,6 @@ EVT_DEV void row_reduce_complete(const typename Epi::Params& p, const Tile& t, c
     const int key = fold_key(g, t.batch);
     int* counter = (int*)t.workspace + key * t.tiles_m + t.tile_m;
     const int share = t.tid / ROWS_PER_PASS, lr0 = t.tid % ROWS_PER_PASS;
-    const int nq = t.tiles_n * g.row_fold_count;
     for (int base = 0; base < Cfg::BM; base += ROWS_PER_PASS) {
       const int lr = base + lr0;
       const int row = t.m0 + lr;
@@ -608,14 +710,26 @@ EVT_DEV void row_reduce_complete(const typename Epi::Params& p, const Tile& t, c
       float st[RS];
       Epi::row_identity(st);
       if (live) {
-#pragma unroll 4
-        for (int q = share; q < nq; q += SHARES) {
-          const int f = q / t.tiles_n, j = q - f * t.tiles_n;
-          const float* src = part + (((int64_t)fold_member(g, key, f) * t.tiles_n + j) * t.M + row) * RS;
-          float o[RS];
+        // Share s folds partials s, s + SHARES, ... of every batch of the fold, batches in fold order.  GROUP
+        // loads are in flight together (a device-scope load takes microseconds), and the addresses advance by a
+        // constant: no division per partial.
+        constexpr int GROUP = RS <= 3 ? 32 : 16;
+        const uint32_t step = (uint32_t)t.M * RS;        // floats from one partial of a row to the next (the host
+                                                         // keeps parts_n * M * RS * 4 below 2 GiB for this path)
+        for (int f = 0; f < g.row_fold_count; ++f) {
+          const __amdgpu_buffer_rsrc_t pf = make_rsrc((const char*)(part + (int64_t)fold_member(g, key, f) * t.parts_n * t.M * RS));
+          for (int j0 = share; j0 < t.parts_n; j0 += SHARES * GROUP) {
+            float o[GROUP][RS];
 #pragma unroll
-          for (int c = 0; c < RS; ++c) o[c] = ld_device(src + c);
-          Epi::row_combine(st, o);
+            for (int u = 0; u < GROUP; ++u) {
+              const int j = j0 + u * SHARES;
+              if (j < t.parts_n) ld_device_n<RS>(pf, (uint32_t)(j * step + row * RS) * 4u, o[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < GROUP; ++u) {
+              if (j0 + u * SHARES < t.parts_n) Epi::row_combine(st, o[u]);
+            }
+          }
         }
       }
       if constexpr (SHARES > 1) {
@@ -758,7 +872,7 @@ template <class Epi, int LG>
 __global__ void __launch_bounds__(256) evt_row_finalize_kernel(typename Epi::Params p, const float* part, GemmArgs g) {
   constexpr int RS = Epi::ROW_STATE > 0 ? Epi::ROW_STATE : 1;
   constexpr int G = 1 << LG;
-  const int M = g.M, tiles_n = g.tiles_n;
+  const int M = g.M, tiles_n = g.parts_n;   // partials per row and batch
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t rowid = gid >> LG;
   const int sub = (int)(gid & (G - 1));
@@ -823,7 +937,7 @@ inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hip
   if (Epi::ROW_STATE > 0 && row_uses_workspace(g) && !g.row_inkernel) {
     const float* part = (const float*)(g.workspace + wl.counter_bytes);
     int lg = 0;
-    while ((1 << lg) < g.tiles_n * g.row_fold_count && lg < 6) ++lg;
+    while ((1 << lg) < g.parts_n * g.row_fold_count && lg < 6) ++lg;
     const int64_t threads = ((int64_t)(g.L / g.row_fold_count) * g.M) << lg;
     const unsigned grid = (unsigned)((threads + 255) / 256);
     switch (lg) {
@@ -976,9 +1090,10 @@ EVT_DEV void rows_maxsumexp(const Tile& t, const float (&x)[16 * Cfg::MI][Cfg::N
   rows_broadcast<Cfg, R>(t.smem + RedAreas<Cfg, RS, CS>::BACK, t.lane, t.wm * Cfg::WN + t.wn, mx, m);
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    float a = 0.f;
+    const float ms = m[r] * kLog2e;
+    float a = t.col_ok(0) ? op_exp_minus(x[r][0], ms) : 0.f;
 #pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni) a += t.col_ok(ni) ? op_exp(x[r][ni] - m[r]) : 0.f;
+    for (int ni = 1; ni < Cfg::NI; ++ni) a += t.col_ok(ni) ? op_exp_minus(x[r][ni], ms) : 0.f;
     part[r] = a;
   }
   rows_reduce<R, false>(part, t.lane);
@@ -1055,77 +1170,127 @@ EVT_DEV void combine_welford(float& n, float& mean, float& m2, float nb, float m
 __device__ uint64_t evt_clock_probe[4];
 #endif
 
+// Split-K exchange.  Every workgroup of the tile leaves its accumulators in the workspace in register order
+// (consecutive lanes write consecutive words); the one whose ticket is the last reads all of them back in split
+// order -- its own included, so the sum does not depend on who arrived last -- and returns true: it goes on to
+// the epilogue; the others are done.
 template <class Cfg, class Epi>
-__global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
-  __shared__ __attribute__((aligned(1024))) char smem[Cfg::LDS_BYTES];
-  int batch, tm, tn;
-  const int split = g.splits > 1 ? (int)(blockIdx.x % (unsigned)g.splits) : 0;
-  const unsigned tile_id = g.splits > 1 ? blockIdx.x / (unsigned)g.splits : blockIdx.x;
-  tile_coords<Cfg::GROUP_M>(tile_id, g.splits > 1 ? gridDim.x / (unsigned)g.splits : gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
-  f32x16 acc[Cfg::MI][Cfg::NI];
-#ifdef EVT_CLOCK_PROBE
-  const uint64_t probe_c0 = __builtin_amdgcn_s_memtime(), probe_r0 = __builtin_amdgcn_s_memrealtime();
-#endif
-  Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, split, smem, acc);
-  if (g.splits > 1) {
-    // Split-K exchange.  Every workgroup of the tile leaves its accumulators in the workspace in register
-    // order (consecutive lanes write consecutive words); the one whose ticket is the last reads all of them
-    // back in split order -- its own included, so the sum does not depend on who arrived last -- and goes on
-    // to the epilogue; the others are done.
-    const WsLayout wl = ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g);
-    char* region = g.workspace + wl.counter_bytes + wl.row_bytes + wl.col_bytes;
-    int* counter = (int*)region + tile_id;
-    constexpr int REGS = Cfg::MI * Cfg::NI * 16;
-    float* part = (float*)(region + wl.split_counter_bytes) + (int64_t)tile_id * g.splits * REGS * Cfg::THREADS;
-    float* mine = part + (int64_t)split * REGS * Cfg::THREADS + threadIdx.x;
+EVT_DEV bool split_k_exchange(const GemmArgs& g, unsigned tile_id, int split, char* smem, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  const WsLayout wl = ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g);
+  char* region = g.workspace + wl.counter_bytes + wl.row_bytes + wl.col_bytes;
+  int* counter = (int*)region + tile_id;
+  constexpr int REGS = Cfg::MI * Cfg::NI * 16;
+  float* part = (float*)(region + wl.split_counter_bytes) + (int64_t)tile_id * g.splits * REGS * Cfg::THREADS;
+  float* mine = part + (int64_t)split * REGS * Cfg::THREADS + threadIdx.x;
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) st_device(mine + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS, acc[mi][ni][v]);
+  __syncthreads();                 // nobody still reads operand tiles from the LDS the flag lives in
+  if (!arrive_last(counter, g.splits, (int*)smem)) return false;
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
+  for (int sp = 0; sp < g.splits; ++sp) {
+    const float* src = part + (int64_t)sp * REGS * Cfg::THREADS + threadIdx.x;
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
       for (int ni = 0; ni < Cfg::NI; ++ni)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) st_device(mine + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS, acc[mi][ni][v]);
-    __syncthreads();                 // nobody still reads operand tiles from the LDS the flag lives in
-    if (!arrive_last(counter, g.splits, (int*)smem)) return;
-#pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < Cfg::NI; ++ni)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
-    for (int sp = 0; sp < g.splits; ++sp) {
-      const float* src = part + (int64_t)sp * REGS * Cfg::THREADS + threadIdx.x;
-#pragma unroll
-      for (int mi = 0; mi < Cfg::MI; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < Cfg::NI; ++ni)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) acc[mi][ni][v] += ld_device(src + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS);
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch
+        for (int v = 0; v < 16; ++v) acc[mi][ni][v] += ld_device(src + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS);
   }
-  regroup_columns<Cfg>(acc);
-#ifdef EVT_CLOCK_PROBE
-  const uint64_t probe_c1 = __builtin_amdgcn_s_memtime(), probe_r1 = __builtin_amdgcn_s_memrealtime();
-#endif
-  // interior tiles of an all-unit-stride epilogue (p.fast, decided on the host) take the check-free epilogue
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch
+  return true;
+}
+
+// One tile's epilogue: interior tiles of an all-unit-stride epilogue (p.fast, decided on the host) take the
+// check-free instantiation.  `part`, `first`, `last`, `state`: TileCtx::set_walk (WALK kernels only).
+template <class Cfg, class Epi>
+EVT_DEV void run_epilogue(const GemmArgs& g, const typename Epi::Params& p, int batch, int tm, int tn, char* smem,
+                          const f32x16 (&acc)[Cfg::MI][Cfg::NI], int part, bool first, bool last, float* state) {
   if (p.fast && (tm + 1) * Cfg::BM <= g.M && (tn + 1) * Cfg::BN <= g.N) {
     TileCtx<Cfg, true> t;
     t.init(g, batch, tm, tn, smem);
+    if constexpr (Cfg::WALK) t.set_walk(part, g.parts_n, first, last, state);
     Epi::template tile<Cfg, TileCtx<Cfg, true>, true>(p, t, g, acc);
   } else {
     TileCtx<Cfg, false> t;
     t.init(g, batch, tm, tn, smem);
+    if constexpr (Cfg::WALK) t.set_walk(part, g.parts_n, first, last, state);
     Epi::template tile<Cfg, TileCtx<Cfg, false>, false>(p, t, g, acc);
   }
+}
+
+template <class Cfg, class Epi>
+__global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
+  // a walking workgroup keeps one running state per row behind the operand stages
+  constexpr int WALK_BYTES = Cfg::WALK ? Cfg::BM * (Epi::ROW_STATE > 0 ? Epi::ROW_STATE : 1) * 4 : 0;
+  __shared__ __attribute__((aligned(1024))) char smem[Cfg::LDS_BYTES + WALK_BYTES];
+  int batch, tm, tn;
+  f32x16 acc[Cfg::MI][Cfg::NI];
 #ifdef EVT_CLOCK_PROBE
-  __builtin_amdgcn_s_waitcnt(0);   // the epilogue's stores have been issued and acknowledged
-  const uint64_t probe_c2 = __builtin_amdgcn_s_memtime(), probe_r2 = __builtin_amdgcn_s_memrealtime();
+  uint64_t probe_main[2] = {0, 0}, probe_epi[2] = {0, 0};
+#endif
+  if constexpr (Cfg::WALK) {
+    // one workgroup per (row block, run of g.walk tiles): main loop and epilogue alternate, the operand ring
+    // running on from tile to tile (Mainloop::Walk)
+    int pn;
+    tile_coords<Cfg::GROUP_M>(blockIdx.x, gridDim.x, g.tiles_m, g.parts_n, batch, tm, pn);
+    const int tn_first = pn * g.walk;
+    const int tn_end = tn_first + g.walk < g.tiles_n ? tn_first + g.walk : g.tiles_n;
+    typename Mainloop<Cfg>::Walk wk;
+    for (tn = tn_first; tn < tn_end; ++tn) {
+      const bool more = tn + 1 < tn_end;
+#ifdef EVT_CLOCK_PROBE
+      const uint64_t c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+#endif
+      Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, 0, smem, acc, wk, more);
+      regroup_columns<Cfg>(acc);
+#ifdef EVT_CLOCK_PROBE
+      const uint64_t c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+#endif
+      run_epilogue<Cfg, Epi>(g, p, batch, tm, tn, Mainloop<Cfg>::epilogue_lds(wk, smem), acc, pn, tn == tn_first, !more,
+                             (float*)(smem + Cfg::LDS_BYTES));
+#ifdef EVT_CLOCK_PROBE
+      const uint64_t c2 = __builtin_amdgcn_s_memtime(), r2 = __builtin_amdgcn_s_memrealtime();
+      probe_main[0] += c1 - c0; probe_main[1] += r1 - r0; probe_epi[0] += c2 - c1; probe_epi[1] += r2 - r1;
+#endif
+    }
+  } else {
+    const int split = g.splits > 1 ? (int)(blockIdx.x % (unsigned)g.splits) : 0;
+    const unsigned tile_id = g.splits > 1 ? blockIdx.x / (unsigned)g.splits : blockIdx.x;
+    tile_coords<Cfg::GROUP_M>(tile_id, g.splits > 1 ? gridDim.x / (unsigned)g.splits : gridDim.x, g.tiles_m, g.tiles_n, batch, tm, tn);
+#ifdef EVT_CLOCK_PROBE
+    const uint64_t c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+#endif
+    Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, split, smem, acc);
+    if (g.splits > 1) {
+      if (!split_k_exchange<Cfg, Epi>(g, tile_id, split, smem, acc)) return;
+    }
+    regroup_columns<Cfg>(acc);
+#ifdef EVT_CLOCK_PROBE
+    const uint64_t c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+#endif
+    run_epilogue<Cfg, Epi>(g, p, batch, tm, tn, smem, acc, tn, true, true, nullptr);
+#ifdef EVT_CLOCK_PROBE
+    __builtin_amdgcn_s_waitcnt(0);   // the epilogue's stores have been issued and acknowledged
+    const uint64_t c2 = __builtin_amdgcn_s_memtime(), r2 = __builtin_amdgcn_s_memrealtime();
+    probe_main[0] = c1 - c0; probe_main[1] = r1 - r0; probe_epi[0] = c2 - c1; probe_epi[1] = r2 - r1;
+#endif
+  }
+#ifdef EVT_CLOCK_PROBE
   if (blockIdx.x == 0 && threadIdx.x == 0) {
-    evt_clock_probe[0] = probe_c1 - probe_c0;
-    evt_clock_probe[1] = probe_r1 - probe_r0;
-    evt_clock_probe[2] = probe_c2 - probe_c1;
-    evt_clock_probe[3] = probe_r2 - probe_r1;
+    evt_clock_probe[0] = probe_main[0];
+    evt_clock_probe[1] = probe_main[1];
+    evt_clock_probe[2] = probe_epi[0];
+    evt_clock_probe[3] = probe_epi[1];
   }
 #endif
 }

@@ -72,12 +72,20 @@ struct GemmArgs {
   // they leave their accumulators in the workspace and the last one to arrive adds them up in split order and
   // runs the epilogue.  splits == 1: one workgroup per tile, nothing goes through the workspace.
   int splits, k_chunk;
+  // GemmCfg::WALK: a workgroup computes `walk` consecutive tiles of a row block, left to right, and a per-row
+  // reduction leaves one partial per workgroup: parts_n = ceil(tiles_n / walk) of them per row.  Elsewhere
+  // walk = 1 and parts_n = tiles_n.
+  int walk, parts_n;
 };
 
 // Compile-time description of one kernel variant.
 //   TILE_IO_  the epilogue reads or writes full tensors: worth giving every lane adjacent output columns
+//   WALK_     a workgroup walks over several tiles of a row block (GemmArgs::walk), the operand ring running
+//             on from one tile into the next (ping-pong loops only)
+//   K_EXACT_  K is a multiple of BK in every launch
 template <int BM_, int BN_, int BK_, int WM_, int WN_, bool A_KC_, bool B_KC_,
-          bool DMA_, int STAGES_, bool BF16_, int GROUP_M_, int PIPE_ = 0, bool TILE_IO_ = true>
+          bool DMA_, int STAGES_, bool BF16_, int GROUP_M_, int PIPE_ = 0, bool TILE_IO_ = true, bool WALK_ = false,
+          bool K_EXACT_ = false>
 struct GemmCfg {
   // PIPE 0: ring of STAGES tiles, fragments fetched inside each k-tile.
   // PIPE 1: look-ahead ring (STAGES >= 3): tile kt+1 is made visible one
@@ -102,6 +110,10 @@ struct GemmCfg {
   //         4  group 1 does the same (STAGES >= 3).
   static constexpr int PIPE = PIPE_;
   static constexpr bool PINGPONG = PIPE_ >= 2;
+  static constexpr bool WALK = WALK_;
+  // K is a multiple of BK in every launch (the host refuses others): see Operand
+  static constexpr bool K_EXACT = K_EXACT_;
+  static_assert(!WALK_ || K_EXACT_, "the carried-over operand ring has no code for a partial k-tile");
   static constexpr int PP_FLAGS = PIPE_ >= 4 ? PIPE_ - 4 : 0;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DMA = DMA_, BF16 = BF16_;
@@ -133,6 +145,7 @@ struct GemmCfg {
   static_assert(PIPE != 1 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
   static_assert(!PINGPONG || (DMA && STAGES >= 2 && WM * WN == 8), "ping-pong needs DMA, >= 2 stages, 8 waves");
   static_assert(PIPE >= 0 && PIPE <= 11, "unknown pipeline");
+  static_assert(!WALK || PINGPONG, "walking over tiles is built into the ping-pong loops");
   static_assert(!(PP_FLAGS & 4) || STAGES >= 3, "group 1 can only issue in its read phase with three or more stages");
 };
 
@@ -172,8 +185,8 @@ EVT_DEV void kc_unslot(int slot, int& r, int& q) {
 template <int RC>
 EVT_DEV int nc_swz(int k) { return ((k & 3) << 2) & (RC - 1); }
 
-EVT_DEV __amdgpu_buffer_rsrc_t make_rsrc(const char* p) {
-  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, kRsrcRange, kRsrcFlags);
+EVT_DEV __amdgpu_buffer_rsrc_t make_rsrc(const char* p, uint32_t num_records = kRsrcRange) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, num_records, kRsrcFlags);
 }
 
 // wait until at most n vector-memory operations of this wave are outstanding
@@ -189,8 +202,10 @@ EVT_DEV void wait_vmcnt() {
 //   SRC_KC   the source matrix is contiguous along K
 //   PERM_NI  >1: LDS row (w*PERM_TN + f*32 + j) holds global row
 //            (w*PERM_TN + j*PERM_NI + f)  (column interleave, B only)
+//   K_EXACT  K is a multiple of BK (the host checks): no k-tile is partial, so the transfers need no per-lane
+//            test against K, and a k-tile past the end reads as zeros through an empty buffer range
 // ---------------------------------------------------------------------------
-template <int ROWS, int BK, bool SRC_KC, bool DMA, int THREADS, int PERM_NI, int PERM_TN>
+template <int ROWS, int BK, bool SRC_KC, bool DMA, int THREADS, int PERM_NI, int PERM_TN, bool K_EXACT = false>
 struct Operand {
   static constexpr bool LDS_KC = SRC_KC || !DMA;
   static constexpr int CH = BK / 8;
@@ -247,11 +262,13 @@ struct Operand {
   };
   EVT_DEV DmaTile dma_begin(int kt) const {
     const int64_t adv = SRC_KC ? (int64_t)kt * BK * 2 : (int64_t)kt * BK * ld * 2;
-    return DmaTile{make_rsrc(base + adv), kt * BK};
+    if constexpr (K_EXACT) return DmaTile{make_rsrc(base + adv, kt * BK < K ? kRsrcRange : 0u), kt * BK};
+    else return DmaTile{make_rsrc(base + adv), kt * BK};
   }
   // transfer number i (of NLOAD) of this thread
   EVT_DEV void dma_chunk(const DmaTile& d, char* lds, int wave, int i) const {
-    const uint32_t v = (d.k0 + kin[i] < K) ? voff[i] : kOobOffset;
+    uint32_t v = voff[i];
+    if constexpr (!K_EXACT) v = (d.k0 + kin[i] < K) ? voff[i] : kOobOffset;
     char* dst = lds + (i * THREADS + wave * 64) * 16;   // wave-uniform; lane*16 added by hardware
     __builtin_amdgcn_raw_ptr_buffer_load_lds(d.rsrc, (lds_void_ptr)dst, 16, v, 0, 0, 0);
   }
@@ -476,9 +493,9 @@ EVT_DEV void regroup_columns(f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
 // The main loop: acc[mi][ni] += A_tile * B_tile over all k-tiles.
 template <class Cfg>
 struct Mainloop {
-  using OpA = Operand<Cfg::BM, Cfg::BK, Cfg::A_KC, Cfg::DMA, Cfg::THREADS, 0, 0>;
+  using OpA = Operand<Cfg::BM, Cfg::BK, Cfg::A_KC, Cfg::DMA, Cfg::THREADS, 0, 0, Cfg::K_EXACT>;
   using OpB = Operand<Cfg::BN, Cfg::BK, Cfg::B_KC, Cfg::DMA, Cfg::THREADS,
-                      Cfg::INTERLEAVE ? Cfg::NI : 0, Cfg::TN>;
+                      Cfg::INTERLEAVE ? Cfg::NI : 0, Cfg::TN, Cfg::K_EXACT>;
   using RdA = FragReader<Cfg::BM, Cfg::BK, Cfg::A_LDS_KC, Cfg::MI>;
   using RdB = FragReader<Cfg::BN, Cfg::BK, Cfg::B_LDS_KC, Cfg::NI, Cfg::REGROUP ? Cfg::NI : 0>;
   static constexpr int LPS = OpA::NLOAD + OpB::NLOAD;   // DMA ops per thread per stage
@@ -753,61 +770,119 @@ struct Mainloop {
     const int ds = stage == 0 ? Cfg::STAGES - 1 : stage - 1;
     return smem + ds * Cfg::STAGE_BYTES;
   }
-  static EVT_DEV void pp_issue(int T, int stage, const OpA& a, const OpB& b, char* smem, int wave) {
+  static EVT_DEV void pp_issue(int nk, int stage, const OpA& a, const OpB& b, char* smem, int wave) {
     char* ds = pp_refill_stage(stage, smem);
-    a.dma(T + Cfg::STAGES - 1, ds, wave);
-    b.dma(T + Cfg::STAGES - 1, ds + Cfg::A_BYTES, wave);
+    a.dma(nk, ds, wave);
+    b.dma(nk, ds + Cfg::A_BYTES, wave);
+  }
+  // GemmCfg::WALK: what a workgroup carries from one tile of its walk to the next.  The operand ring does not
+  // drain between tiles: while another tile follows (`more`), the transfers issued past the last k-tile fetch
+  // the first STAGES-1 k-tiles of that tile (same rows of A, B moved on by BN) instead of zeros, so they are
+  // in flight or landed while the epilogue runs, and the next main loop starts as if in steady state.  The
+  // stage that held the last k-tile is not refilled before that loop's first iteration: it is the epilogue's
+  // LDS (epilogue_lds).
+  struct Walk {
+    int stage = 0;        // ring stage of k-tile 0 of the coming tile
+    bool primed = false;  // its first STAGES-1 k-tiles have been issued
+  };
+  static EVT_DEV char* epilogue_lds(const Walk& wk, char* smem) {
+    if constexpr (Cfg::WALK) return pp_refill_stage(wk.stage, smem);
+    else return smem;
   }
   // Phase barriers are bare s_barrier instructions: the only memory traffic of
   // the loop is the DMA (waited for explicitly with vmcnt) and the
   // inline-assembly LDS reads (waited for inside pp_read); a fence here would
   // make the compiler drain the DMA ring at every phase.
   static EVT_DEV void pp_barrier() { __builtin_amdgcn_s_barrier(); }
-  static EVT_DEV void run_pingpong(const OpA& a, const OpB& b, const RdA& ra, const RdB& rb, char* smem,
-                                   int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  static EVT_DEV void run_pingpong(const OpA& a, OpB& b, const RdA& ra, const RdB& rb, char* smem,
+                                   int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI],
+                                   Walk& wk, bool more, int64_t b_step, int tid) {
     constexpr int S = Cfg::STAGES;
     static_assert((S - 1) * LPS < 64, "vmcnt is a 6-bit counter");
+    int stage = 0;
+    if constexpr (Cfg::WALK) stage = wk.primed ? wk.stage : 0;
+    if (!Cfg::WALK || !wk.primed) {
 #pragma unroll
-    for (int s = 0; s < S - 1; ++s) {
-      a.dma(s, smem + s * Cfg::STAGE_BYTES, wave);
-      b.dma(s, smem + s * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+      for (int s = 0; s < S - 1; ++s) {
+        a.dma(s, smem + s * Cfg::STAGE_BYTES, wave);
+        b.dma(s, smem + s * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+      }
     }
-    wait_tiles<S - 2>();            // tile 0 has landed
+    // tile 0 has landed.  In a walk the count also covers what the epilogue in between issued after the
+    // transfers (the counter runs in issue order), so this waits for those accesses too.
+    wait_tiles<S - 2>();
     __syncthreads();
     TileFrags f;
-    int stage = 0;
     const int grp = wave >> 2;
+    // k-tile to fetch in iteration T: T + S - 1 of this tile, or, past its end with a tile to follow, of that one
+    auto fetch_index = [&](int T) {
+      int nk = T + S - 1;
+      if constexpr (Cfg::WALK) {
+        if (more && nk >= KT) nk -= KT;
+      }
+      return nk;
+    };
+    auto move_on = [&](int T) {   // from here on the transfers belong to the next tile: B moves on by BN
+      if constexpr (Cfg::WALK) {
+        if (more && T + S - 1 == KT) {
+          int t2 = tid;
+          asm volatile("" : "+v"(t2));   // computed here, once per tile, not ahead of the loop and kept in registers
+          b.init(b.base + b_step, b.ld, b.rows_left - Cfg::BN, b.K, t2);
+        }
+      }
+    };
     if (grp == 0) {
       for (int T = 0; T < KT; ++T) {
+        move_on(T);
+        const int nk = fetch_index(T);
         char* ds = pp_refill_stage(stage, smem);
-        if constexpr (!PP_G0_IN_C && !PP_G0_IN_R) pp_issue(T, stage, a, b, smem, wave);
-        pp_read<PP_G0_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, T + S - 1, ds, wave);
+        if constexpr (!PP_G0_IN_C && !PP_G0_IN_R) pp_issue(nk, stage, a, b, smem, wave);
+        pp_read<PP_G0_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, nk, ds, wave);
         if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
-        pp_mma<PP_G0_IN_C, 1, 0, PP_NM - PP_REST>(f, ra, rb, acc, a, b, T + S - 1, ds, wave);
+        pp_mma<PP_G0_IN_C, 1, 0, PP_NM - PP_REST>(f, ra, rb, acc, a, b, nk, ds, wave);
         wait_tiles<S - 2>();        // my share of tile T+1 has landed
         pp_barrier();               // ends phase 2T+1
         if constexpr (PP_REST > 0) pp_mma<false, 3, PP_NM - PP_REST, PP_NM>(f, ra, rb, acc, a, b, 0, ds, wave);
         stage = stage + 1 == S ? 0 : stage + 1;
       }
     } else {
-      if constexpr (!PP_G1_IN_R) pp_issue(0, 0, a, b, smem, wave);
+      if constexpr (!PP_G1_IN_R) pp_issue(S - 1, stage, a, b, smem, wave);
       for (int T = 0; T < KT; ++T) {
+        move_on(T);
+        const int nk = fetch_index(T);
         char* ds = pp_refill_stage(stage, smem);
-        if (T > 0) pp_mma<!PP_G1_IN_R, 2, 0, PP_NM>(f, ra, rb, acc, a, b, T + S - 1, ds, wave);   // C(T-1)
+        if (T > 0) pp_mma<!PP_G1_IN_R, 2, 0, PP_NM>(f, ra, rb, acc, a, b, nk, ds, wave);   // C(T-1)
         if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
-        pp_read<PP_G1_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, T + S - 1, ds, wave);
+        pp_read<PP_G1_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, nk, ds, wave);
         wait_tiles<S - 2>();        // my share of tile T+1 has landed
         pp_barrier();               // ends phase 2T+1
         stage = stage + 1 == S ? 0 : stage + 1;
       }
       if (KT > 0) pp_mma<false, 2, 0, PP_NM>(f, ra, rb, acc, a, b, 0, smem, wave);   // C(KT-1)
     }
-    wait_vmcnt<0>();                // the zero-fill transfers past the last tile have landed
+    if constexpr (Cfg::WALK) {
+      wk.stage = stage;
+      wk.primed = more;
+      if (!more) wait_vmcnt<0>();   // the zero-fill transfers past the last tile have landed
+    } else {
+      wait_vmcnt<0>();              // the zero-fill transfers past the last tile have landed
+    }
   }
 
   static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, int split, char* smem,
                           f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
-    const int tid = threadIdx.x;
+    Walk wk;
+    run(g, batch, m0, n0, split, smem, acc, wk, false);
+  }
+  // `wk`, `more`: see Walk (WALK kernels call this once per tile of the walk, `more` while another follows)
+  static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, int split, char* smem,
+                          f32x16 (&acc)[Cfg::MI][Cfg::NI], Walk& wk, bool more) {
+    int tid = threadIdx.x;
+    // In a walk this runs once per tile with the epilogue in between.  Everything below that depends only on
+    // the thread index (transfer offsets, fragment addresses) would be hoisted out of the tile loop and then
+    // stay live, or spilled, through the epilogue, which needs every register itself; hiding where `tid` comes
+    // from makes the compiler derive them afresh for each tile.
+    if constexpr (Cfg::WALK) asm volatile("" : "+v"(tid));
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -843,7 +918,8 @@ struct Mainloop {
     if constexpr (Cfg::PIPE == 1) {
       run_lookahead(a, b, ra, rb, smem, wave, KT, acc);
     } else if constexpr (Cfg::PINGPONG) {
-      run_pingpong(a, b, ra, rb, smem, wave, KT, acc);
+      run_pingpong(a, b, ra, rb, smem, wave, KT, acc, wk, more,
+                   Cfg::B_KC ? (int64_t)Cfg::BN * g.ldb * 2 : (int64_t)Cfg::BN * 2, tid);
     } else if constexpr (Cfg::DMA && Cfg::STAGES == 1) {
       // K fits one tile (checked by the host): load it, use it
       a.dma(0, smem, wave);

@@ -202,7 +202,7 @@ class LazyModule:
             self.name = f"evt_row_{ir.key()}_{spec.tag()}"
             cg = RowCodegen(ir, spec, self.name)
         else:
-            self.name = (f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tile.tag()}"
+            self.name = (f"evt_{'bmm' if ir.batched else 'gemm'}_{ir.key()}_{spec.tag()}"
                          + ("_probe" if clock_probe else ""))
             cg = Codegen(ir, spec, self.name, clock_probe)
         self.source = cg.source()

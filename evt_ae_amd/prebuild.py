@@ -110,6 +110,9 @@ def register_all() -> List[jit.LazyModule]:
         with force_tile(tile):
             for cfg in W.CONFIGS:
                 W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, W.PIPELINE_SHAPES[cfg]))
+    for cfg, shapes, tile in W.walk_cases():
+        with force_tile(tile):
+            W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
     from .codegen import TileConfig
     with force_tile(TileConfig(*W.NO_ALLOC_TILE)):
         for cfg, cases in W.NO_ALLOC_SHAPES.items():

@@ -215,7 +215,31 @@ def pipeline_tiles():
     from .codegen import TileConfig
     return [TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 2),
             TileConfig(256, 256, 32, 2, 4, 4, True, 4, 2), TileConfig(256, 128, 64, 4, 2, 3, True, 4, 3),
-            TileConfig(128, 256, 64, 2, 4, 3, True, 4, 3), TileConfig(256, 256, 64, 2, 4, 2, True, 4, 3)]
+            TileConfig(128, 256, 64, 2, 4, 3, True, 4, 3), TileConfig(256, 256, 64, 2, 4, 2, True, 4, 3),
+            # options of the one-barrier loop: transfers issued among the LDS reads (both groups), barrier inside
+            # group 0's MFMA phase
+            TileConfig(128, 256, 64, 2, 4, 3, True, 4, 10), TileConfig(256, 128, 64, 4, 2, 3, True, 4, 11),
+            TileConfig(256, 256, 64, 2, 4, 2, True, 4, 7)]
+
+
+# Workgroups that walk over several tiles of a row block (TileConfig.walk): (config, shapes, tile).  K is a
+# multiple of bk throughout (the walk's condition); N leaves a partial last tile and a last workgroup with fewer
+# tiles than the others; M leaves a partial row block.
+def walk_cases():
+    from .codegen import TileConfig
+    return [
+        # per-row reductions only, 10 tiles along N in runs of 4 (4 + 4 + 2) and of 8 (8 + 2)
+        (5, dict(M=300, N=2504, K=192), TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2, 4)),
+        (5, dict(M=300, N=2504, K=192), TileConfig(256, 256, 64, 4, 2, 2, True, 4, 3, 8)),
+        # tile loads and stores + Welford statistics, three stages, 5 tiles in runs of 2
+        (3, dict(M=200, N=1096, K=256), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 3, 2)),
+        # two k-tiles cannot prime three stages: the module falls back to a workgroup per tile
+        (3, dict(M=200, N=1096, K=128), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 3, 2)),
+        # stores only, k-row B tile (columns regrouped after the main loop), transfers issued among the LDS reads
+        (1, dict(M=300, N=1800, K=128), TileConfig(256, 256, 64, 2, 4, 2, True, 4, 6, 3)),
+        # batched, softmax statistics + store
+        (2, dict(L=3, S=520, D=128), TileConfig(128, 128, 64, 2, 4, 2, True, 4, 2, 2)),
+    ]
 
 
 def unfused_eager(cfg: int) -> Callable:

@@ -392,3 +392,32 @@ def test_bias_gradient_behind_a_head_merge_lowers_correctly(transposed):
     for o, r in zip(got, ref):
         assert tuple(o.shape) == tuple(r.shape)
         assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3
+
+
+def test_walk_tiles_are_offered_and_refused_where_they_should(monkeypatch):
+    """Tiles whose workgroups walk over several tiles of a row block: offered by
+    the tuner only where the tiles outnumber the CUs, K is a multiple of bk and
+    no per-column reduction sits in the epilogue; refused by the code generator
+    otherwise."""
+    from evt_ae_amd.autotuner import tune_workloads
+    from evt_ae_amd.autotuner.tuner_base import force_tile
+    from evt_ae_amd.codegen import TileConfig
+    monkeypatch.setenv("EVT_TUNER_CACHE", "/nonexistent/tuner_cache.db")
+    walks = {cfg: [t for t in tuner.candidates() if t.walk > 1] for cfg, tuner in tune_workloads._tuners()}
+    assert walks[5] and all(t.pipe >= 2 and t.stages <= 3 for t in walks[5])      # 2048 tiles of 256 x 256
+    assert any(t.walk == 8 and (t.bm, t.bn) == (256, 256) for t in walks[5])
+    assert not walks[2] and not walks[3] and not walks[4]                          # one round of tiles / column sums
+    tile = TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2, 4)
+    from dataclasses import replace
+    from evt_ae_amd import jit, prebuild
+    (node4,) = W.fused_nodes(W.fuse(W.CONFIGS[4].module(), prebuild._shapes_of(4, None)))
+    assert node4.target.ir.col_state > 0
+    with pytest.raises(NotImplementedError):           # per-column reduction in the epilogue
+        jit.LazyModule(node4.target.ir, replace(node4.target.spec, tile=tile, k_exact=True))
+    with force_tile(tile):
+        gm = W.fuse(W.CONFIGS[5].module(), W.make_inputs(5, W.SMALL_SHAPES[5]))
+    (node,) = W.fused_nodes(gm)
+    assert node.target.tile == tile and node.target.spec.k_exact
+    assert "_n4_kx" in node.target.module.name
+    with pytest.raises(NotImplementedError):           # a module that must also take a K with a partial k-tile
+        jit.LazyModule(node.target.ir, replace(node.target.spec, k_exact=False))

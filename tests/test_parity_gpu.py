@@ -67,6 +67,27 @@ def test_pipeline_variants_against_oracle(cfg, tile):
     _compare(wl, outs, evt_oracle.eval_fp32(wl.module(), inputs))
 
 
+@pytest.mark.parametrize("two_kernel", [False, True], ids=["in_kernel", "finalize_kernel"])
+@pytest.mark.parametrize("case", W.walk_cases(), ids=lambda c: f"cfg{c[0]}_{c[2].tag()}_K{c[1].get('K', c[1].get('D'))}")
+def test_walking_workgroups_against_oracle(case, two_kernel, monkeypatch):
+    """Workgroups that compute several tiles of a row block in a row: the operand
+    ring carried from tile to tile, the epilogue in the one free stage, per-row
+    reductions folded over the walk into one partial per workgroup.  Runs of
+    unequal length, partial edge tiles, and phase 2 in either place."""
+    cfg, shapes, tile = case
+    if two_kernel:
+        if not W.CONFIGS[cfg].reduction_outputs:
+            pytest.skip("no reduction in this epilogue")
+        monkeypatch.setenv("EVT_TWO_KERNEL_REDUCE", "1")
+    wl, inputs, gm, outs = _run(cfg, shapes, tile=tile)
+    _compare(wl, outs, evt_oracle.eval_fp32(wl.module(), inputs))
+    again = gm(*[t.cuda() for t in inputs])
+    again = list(again) if isinstance(again, (tuple, list)) else [again]
+    torch.cuda.synchronize()
+    for a, b in zip(outs, again):
+        assert torch.equal(a, b), "two launches of the same problem differ"
+
+
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
 def test_configs_full_size(cfg):
     """Headline sizes: against the oracle (its fp32 CPU evaluation finishes in
