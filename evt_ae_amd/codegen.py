@@ -972,7 +972,7 @@ class RowCodegen(Codegen):
             for i, name in enumerate(self.hoisted):
                 k = ir.nodes[name].slot
                 e("if (nv > 0) {")
-                e(f"  if constexpr (FAST) evt::load8v(p.t{k} + n0, hz[{i}][c]);")
+                e(f"  if (FAST && nv == 8) evt::load8v(p.t{k} + n0, hz[{i}][c]);")
                 e(f"  else evt::load8s(p.t{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, hz[{i}][c]);")
                 e("} else {")
                 e(f"  #pragma unroll\n  for (int j = 0; j < 8; ++j) hz[{i}][c][j] = 0.f;")
@@ -1006,45 +1006,59 @@ class RowCodegen(Codegen):
         e("for (int c = 0; c < Cfg::CH; ++c) {")
         e.indent()
         e("const int nv = t.valid(c);")
-        e("if (nv > 0) {")
-        e.indent()
         e("const int n0 = t.col0(c);")
-        for name in inner:
-            n = ir.nodes[name]
-            c = _cname(name)
-            e(f"float {c}[8];")
-            if n.op == "accum":
-                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = acc[c][j];")
-            elif n.op == "anchorval":
-                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = av[{n.comp}][c][j];")
-            elif n.op == "load" and ir.slots[n.slot].kind == "rand":
-                k, r = n.slot, ir.rng_scalar
-                e(f"evt::rand8((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r}]) | ((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r + 1}]) << 32), "
-                  f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u + 16u * __builtin_bit_cast(uint32_t, p.s[{r + 3}]), o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, {c});")
-            elif n.op == "load" and name in self.hoisted:
-                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
-            elif n.op == "load":
-                k = n.slot
-                e(f"if constexpr (FAST) evt::load8v(p.t{k} + o_{k} + n0, {c});")
-                e(f"else evt::load8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {c});")
-            else:
-                e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = {self.expr(n, 'j')};")
-        for s in tile_stores:
-            k = s.slot
-            src = _cname(s.input)
-            if not self.var_n[s.input]:
-                e(f"float b_{k}[8];\n#pragma unroll\nfor (int j = 0; j < 8; ++j) b_{k}[j] = {src};")
-                src = f"b_{k}"
-            e(f"if constexpr (FAST) evt::store8v(p.t{k} + o_{k} + n0, {src});")
-            e(f"else evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
-        for r in col_reds:
-            x = f"{_cname(r.input)}[j]" if self.var_n[r.input] else _cname(r.input)
-            o = r.state_offset
-            e("#pragma unroll")
-            if r.kind == "sum":
-                e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] += j < nv ? {x} : 0.f;")
-            else:
-                e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] = j < nv ? fmaxf(cst[{o}][c][j], {x}) : cst[{o}][c][j];")
+
+        def chunk_body(vector: bool):
+            """The epilogue on this lane's 8 columns of chunk c: whole groups through 16-byte accesses (check-free
+            instantiation only), the group that straddles the row end element by element."""
+            for name in inner:
+                n = ir.nodes[name]
+                c = _cname(name)
+                e(f"float {c}[8];")
+                if n.op == "accum":
+                    e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = acc[c][j];")
+                elif n.op == "anchorval":
+                    e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = av[{n.comp}][c][j];")
+                elif n.op == "load" and ir.slots[n.slot].kind == "rand":
+                    k, r = n.slot, ir.rng_scalar
+                    e(f"evt::rand8((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r}]) | ((uint64_t)__builtin_bit_cast(uint32_t, p.s[{r + 1}]) << 32), "
+                      f"__builtin_bit_cast(uint32_t, p.s[{r + 2}]), {k}u + 16u * __builtin_bit_cast(uint32_t, p.s[{r + 3}]), o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, {c});")
+                elif n.op == "load" and name in self.hoisted:
+                    e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
+                elif n.op == "load":
+                    k = n.slot
+                    if vector:
+                        e(f"evt::load8v(p.t{k} + o_{k} + n0, {c});")
+                    else:
+                        e(f"evt::load8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {c});")
+                else:
+                    e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = {self.expr(n, 'j')};")
+            for s in tile_stores:
+                k = s.slot
+                src = _cname(s.input)
+                if not self.var_n[s.input]:
+                    e(f"float b_{k}[8];\n#pragma unroll\nfor (int j = 0; j < 8; ++j) b_{k}[j] = {src};")
+                    src = f"b_{k}"
+                if vector:
+                    e(f"evt::store8v(p.t{k} + o_{k} + n0, {src});")
+                else:
+                    e(f"evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
+            for r in col_reds:
+                x = f"{_cname(r.input)}[j]" if self.var_n[r.input] else _cname(r.input)
+                o = r.state_offset
+                e("#pragma unroll")
+                if r.kind == "sum":
+                    e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] += j < nv ? {x} : 0.f;")
+                else:
+                    e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] = j < nv ? fmaxf(cst[{o}][c][j], {x}) : cst[{o}][c][j];")
+
+        e("if (FAST && nv == 8) {")
+        e.indent()
+        chunk_body(True)
+        e.dedent()
+        e("} else if (nv > 0) {")
+        e.indent()
+        chunk_body(False)
         e.dedent()
         e("}")
         e.dedent()
@@ -1132,7 +1146,7 @@ class RowCodegen(Codegen):
         e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0; g.colws = nullptr;")
         if ir.col_state:
             e("if (a->L != 1) return EVT_ERR_BAD_ARGS;      // the per-column reductions run over every row")
-        e(f"g.fast = (g.vecA && {'g.vecB && ' if two else ''}(a->N & 7) == 0) ? 1 : 0;")
+        e(f"g.fast = (g.vecA && {'g.vecB && ' if two else ''}a->N >= 8) ? 1 : 0;")
         e(f"g.eps = {'a->scalars[%d]' % ir.anchor_scalar if ir.anchor_scalar is not None else '0.f'};")
         if stats:
             # the forward statistics are two fp32 load slots with one value per row, contiguous over all rows

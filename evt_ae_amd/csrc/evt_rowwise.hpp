@@ -41,7 +41,8 @@ struct RowArgs {
   float eps;                 // layer norm
   int vecA, vecB;            // rows of A / B may be read with 16-byte loads
   float* colws;              // per-column reductions of the epilogue: [workgroups][COL_STATE][N] partials
-  int fast;                  // N % 8 == 0 and every anchor operand is dword aligned: whole 8-column groups only
+  int fast;                  // N >= 8 and every anchor operand is dword aligned: whole 8-column groups move as 16
+                             // bytes without checks, the group that straddles the row end (N % 8 != 0) on its own
 };
 
 // ELT: 0 = f16, 1 = bf16, 2 = f32 element type of the anchor operands
@@ -278,18 +279,31 @@ EVT_DEV void row_fetch_one(const char* base, int64_t ld, int64_t bs, int vec, co
   using T = typename RowElt<Cfg::ELT>::type;
   const T* row = reinterpret_cast<const T*>(base) + (int64_t)t.l * bs + (int64_t)t.m * ld;
   if constexpr (FAST) {
-    // every lane loads 16-byte groups; a lane whose group lies past the row end reads the row's first group
-    // instead (always there) and the value is replaced afterwards: no branch, no partial group
+    // Every lane loads 16-byte groups; a lane whose group is not wholly inside the row reads the row's first
+    // group instead (always there: N >= 8) and the value is replaced afterwards: no branch in the body.  When
+    // N is no multiple of 8, one lane per row holds a group that straddles the row end; it fetches its few
+    // elements one by one in a tail of its own, so all whole groups keep the straight-line body.
     constexpr int Q = sizeof(T) * 8 / 16;
 #pragma unroll
     for (int c = 0; c < Cfg::CH; ++c) {
-      const bool in = t.col0(c) < t.N;
+      const bool full = t.valid(c) == 8;
       union { q16 q[Q]; T e[8]; } u;
-      const q16* src = reinterpret_cast<const q16*>(row + (in ? t.col0(c) : 0));
+      const q16* src = reinterpret_cast<const q16*>(row + (full ? t.col0(c) : 0));
 #pragma unroll
       for (int i = 0; i < Q; ++i) u.q[i] = src[i];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[c][j] = in ? u.e[j] : (T)fill;
+      for (int j = 0; j < 8; ++j) x[c][j] = full ? u.e[j] : (T)fill;
+    }
+    if (t.N & 7) {      // wave-uniform
+#pragma unroll
+      for (int c = 0; c < Cfg::CH; ++c) {
+        const int v = t.valid(c);
+        if (v > 0 && v < 8) {
+#pragma unroll
+          for (int j = 0; j < 7; ++j)
+            if (j < v) x[c][j] = row[t.col0(c) + j];
+        }
+      }
     }
     return;
   }
