@@ -960,7 +960,7 @@ class RowCodegen(Codegen):
         inner = [n for n in need if self.var_n[n]]
         nh = len(self.hoisted)
         e(f"static constexpr int NH = {nh};   // row vectors kept in registers across the rows of a wave")
-        e("template <class Cfg, bool FAST, class Ctx>")
+        e("template <class Cfg, int FAST, class Ctx>")
         e(f"static EVT_DEV void hoist(const Params& p, const Ctx& t, float (&hz)[{max(nh, 1)}][Cfg::CH][8]) {{")
         e.indent()
         if nh:
@@ -972,7 +972,7 @@ class RowCodegen(Codegen):
             for i, name in enumerate(self.hoisted):
                 k = ir.nodes[name].slot
                 e("if (nv > 0) {")
-                e(f"  if (FAST && nv == 8) evt::load8v(p.t{k} + n0, hz[{i}][c]);")
+                e(f"  if (FAST == 2 || (FAST == 1 && nv == 8)) evt::load8v(p.t{k} + n0, hz[{i}][c]);")
                 e(f"  else evt::load8s(p.t{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, hz[{i}][c]);")
                 e("} else {")
                 e(f"  #pragma unroll\n  for (int j = 0; j < 8; ++j) hz[{i}][c][j] = 0.f;")
@@ -982,13 +982,21 @@ class RowCodegen(Codegen):
         e("(void)p; (void)t; (void)hz;")
         e.dedent()
         e("}")
-        e("template <class Cfg, bool FAST, class Ctx>")
+        e("template <class Cfg, int FAST, class Ctx>")
         e(f"static EVT_DEV void row(const Params& p, const Ctx& t, const float (&acc)[Cfg::CH][8], const float (&rv)[2], "
           f"const float (&av)[{max(self.anchor_values, 1)}][Cfg::CH][8], "
-          f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8], float (&cst)[{max(ir.col_state, 1)}][Cfg::CH][8]) {{")
+          f"const float (&hz)[{max(nh, 1)}][Cfg::CH][8], float (&cst)[{max(ir.col_state, 1)}][Cfg::CH][8], "
+          f"float (&rsv)[{max(len(row_stores), 1)}]) {{")
         e.indent()
         for k, s in enumerate(ir.slots):
-            e(f"const int64_t o_{k} = evt::batch_offset(t.l, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2) + (int64_t)t.m * p.t{k}_sm;")
+            # a single batch (the common 2-D case) needs none of batch_offset's divisions
+            e(f"const int64_t o_{k} = (t.L == 1 ? (int64_t)0 : evt::batch_offset(t.l, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2)) + (int64_t)t.m * p.t{k}_sm;")
+        # one row per wave: its tensors' rows as buffer resources (chunk_body(buffer=True))
+        buffered = sorted({ir.nodes[n].slot for n in inner if ir.nodes[n].op == "load" and n not in self.hoisted
+                           and ir.slots[ir.nodes[n].slot].kind != "rand"} | {s_.slot for s_ in tile_stores})
+        for k in buffered:
+            e(f"[[maybe_unused]] __amdgpu_buffer_rsrc_t rs_{k};")
+            e(f"if constexpr (FAST == 2 && Cfg::RPW == 1) rs_{k} = evt::make_rsrc(evt::wave_uniform(p.t{k} + o_{k}));")
         for name in outer:
             n = ir.nodes[name]
             c = _cname(name)
@@ -1008,7 +1016,7 @@ class RowCodegen(Codegen):
         e("const int nv = t.valid(c);")
         e("const int n0 = t.col0(c);")
 
-        def chunk_body(vector: bool):
+        def chunk_body(vector: bool, buffer: bool = False):
             """The epilogue on this lane's 8 columns of chunk c: whole groups through 16-byte accesses (check-free
             instantiation only), the group that straddles the row end element by element."""
             for name in inner:
@@ -1027,7 +1035,10 @@ class RowCodegen(Codegen):
                     e(f"#pragma unroll\nfor (int j = 0; j < 8; ++j) {c}[j] = hz[{self.hoisted.index(name)}][c][j];")
                 elif n.op == "load":
                     k = n.slot
-                    if vector:
+                    if buffer:
+                        e(f"evt::load8v_b<std::remove_cv_t<std::remove_pointer_t<decltype(p.t{k})>>>(rs_{k}, "
+                          f"nv > 0 ? (uint32_t)n0 * (uint32_t)sizeof(*p.t{k}) : evt::kOobOffset, {c});")
+                    elif vector:
                         e(f"evt::load8v(p.t{k} + o_{k} + n0, {c});")
                     else:
                         e(f"evt::load8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {c});")
@@ -1039,7 +1050,10 @@ class RowCodegen(Codegen):
                 if not self.var_n[s.input]:
                     e(f"float b_{k}[8];\n#pragma unroll\nfor (int j = 0; j < 8; ++j) b_{k}[j] = {src};")
                     src = f"b_{k}"
-                if vector:
+                if buffer:
+                    e(f"evt::store8v_b<std::remove_pointer_t<decltype(p.t{k})>>(rs_{k}, "
+                      f"nv > 0 ? (uint32_t)n0 * (uint32_t)sizeof(*p.t{k}) : evt::kOobOffset, {src});")
+                elif vector:
                     e(f"evt::store8v(p.t{k} + o_{k} + n0, {src});")
                 else:
                     e(f"evt::store8s(p.t{k} + o_{k} + (int64_t)n0 * p.t{k}_sn, p.t{k}_sn, p.t{k}_vec != 0, nv, {src});")
@@ -1052,7 +1066,22 @@ class RowCodegen(Codegen):
                 else:
                     e(f"for (int j = 0; j < 8; ++j) cst[{o}][c][j] = j < nv ? fmaxf(cst[{o}][c][j], {x}) : cst[{o}][c][j];")
 
-        e("if (FAST && nv == 8) {")
+        # FAST 2: every group is whole; FAST 1: whole groups and the one that straddles the row end; 0: generic
+        e("if constexpr (FAST == 2 && Cfg::RPW == 1) {")
+        e.indent()
+        chunk_body(True, buffer=True)      # every lane, no branch: lanes without columns are dropped by the range check
+        e.dedent()
+        e("} else if constexpr (FAST == 2) {")
+        e.indent()
+        e("if (nv > 0) {")
+        e.indent()
+        chunk_body(True)
+        e.dedent()
+        e("}")
+        e.dedent()
+        e("} else {")
+        e.indent()
+        e("if (FAST == 1 && nv == 8) {")
         e.indent()
         chunk_body(True)
         e.dedent()
@@ -1063,16 +1092,29 @@ class RowCodegen(Codegen):
         e("}")
         e.dedent()
         e("}")
-        if row_stores:
-            e("if (t.sub == 0) {")
-            e.indent()
-            for s in row_stores:
-                if self.var_n[s.input]:
-                    raise NotImplementedError("per-row output of a per-element value")
-                e(f"evt::st_f32(p.t{s.slot}, o_{s.slot}, {_cname(s.input)});")
-            e.dedent()
-            e("}")
-        e("(void)p; (void)t; (void)acc; (void)rv; (void)av; (void)hz; (void)cst;")
+        e.dedent()
+        e("}")
+        # one value per row (mean, rstd, ...): handed back to the kernel, which collects the values of the rows a
+        # wave visits and stores them together (row_store_one below)
+        for i, s in enumerate(row_stores):
+            if self.var_n[s.input]:
+                raise NotImplementedError("per-row output of a per-element value")
+            e(f"rsv[{i}] = {_cname(s.input)};")
+        e("(void)p; (void)t; (void)acc; (void)rv; (void)av; (void)hz; (void)cst; (void)rsv;")
+        e.dedent()
+        e("}")
+        e(f"static constexpr int NRS = {len(row_stores)};   // per-row outputs")
+        esize = {"f16": 2, "bf16": 2, "f32": 4, "i32": 4, "i64": 8, "bool": 1, "u8": 1, "i8": 1}
+        nst = sum(max(1, esize[ir.slots[s_.slot].dtype] // 2) for s_ in tile_stores)
+        e("// store instructions row() issues per chunk of a row when every lane stores without a branch (16 bytes each)")
+        e(f"static constexpr int CHUNK_STORES = {nst};")
+        e("// per-row output number i of row (l, m); L: number of batches")
+        e("static EVT_DEV void row_store_one(const Params& p, int L, int l, int m, int i, float v) {")
+        e.indent()
+        for i, s in enumerate(row_stores):
+            k = s.slot
+            e(f"if (i == {i}) evt::st_f32(p.t{k}, (L == 1 ? (int64_t)0 : evt::batch_offset(l, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2)) + (int64_t)m * p.t{k}_sm, v);")
+        e("(void)p; (void)L; (void)l; (void)m; (void)i; (void)v;")
         e.dedent()
         e("}")
 
@@ -1146,7 +1188,7 @@ class RowCodegen(Codegen):
         e("g.mean = nullptr; g.rstd = nullptr; g.gamma = nullptr; g.vecG = 0; g.colws = nullptr;")
         if ir.col_state:
             e("if (a->L != 1) return EVT_ERR_BAD_ARGS;      // the per-column reductions run over every row")
-        e(f"g.fast = (g.vecA && {'g.vecB && ' if two else ''}a->N >= 8) ? 1 : 0;")
+        e(f"g.fast = (g.vecA && {'g.vecB && ' if two else ''}a->N >= 8) ? ((a->N & 7) == 0 ? 2 : 1) : 0;")
         e(f"g.eps = {'a->scalars[%d]' % ir.anchor_scalar if ir.anchor_scalar is not None else '0.f'};")
         if stats:
             # the forward statistics are two fp32 load slots with one value per row, contiguous over all rows
@@ -1178,7 +1220,7 @@ class RowCodegen(Codegen):
         vec_slots = [k for k, sl in enumerate(ir.slots) if k not in ir.anchor_slots and
                      ((sl.role == "load" and sl.kind in ("aux", "row")) or (sl.role == "store" and sl.domain == "tile"))]
         cond = " && ".join(f"p.t{k}_vec" for k in vec_slots) or "1"
-        e(f"p.fast = (g.fast && {cond}) ? 1 : 0;   // every per-element tensor of the epilogue is unit-stride and dword aligned too")
+        e(f"p.fast = ({cond}) ? g.fast : 0;   // every per-element tensor of the epilogue is unit-stride and dword aligned too")
         e("return EVT_OK;")
         e.dedent()
         e("}")
@@ -1190,7 +1232,11 @@ class RowCodegen(Codegen):
         e("// workgroups per CU before waves start walking over several rows (0: one pass, a workgroup per Cfg::ROWS rows);")
         e("// walking pays when row vectors are kept in registers across the rows of a wave, and bounds the number of")
         e("// partials of a per-column reduction")
-        default_cap = 4 if ir.col_state else (16 if self.hoisted else 0)
+        has_row_outputs = any(s_.domain == "row" for s_ in ir.stores)
+        # per-row outputs leave in batches only when a wave visits several consecutive rows (measured on a layer norm
+        # over 131072 x 1024: 128 us with a workgroup per four rows, 107 / 102.5 / 107 us with 16 / 32 / 48
+        # workgroups per CU)
+        default_cap = 4 if ir.col_state else (32 if has_row_outputs else (16 if self.hoisted else 0))
         if 1 < sp.wpr < 16:
             # a row per workgroup: 8 waves per CU walk over the rows, each fetching its next row ahead (measured
             # on 4096 x 30528: 100 us against 108 us with a workgroup per row)
@@ -1241,8 +1287,9 @@ class RowCodegen(Codegen):
         e("}")
         e("static int enqueue(evt::RowArgs& g, const Epi::Params& p, unsigned grid, void* ws, void* stream) {")
         e("  g.colws = (float*)ws;")
-        e("  if (p.fast) hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, true>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
-        e("  else hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, false>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  if (p.fast == 2) hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, 2>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  else if (p.fast == 1) hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, 1>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
+        e("  else hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, 0>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  int err = (int)hipGetLastError();")
         e("  if (err != 0 || Epi::COL_STATE == 0) return err;")
         e("  hipLaunchKernelGGL((evt::evt_row_col_finalize_kernel<Epi>), dim3((g.N + 63) / 64), dim3(1024), 0, (hipStream_t)stream, g, p, (int)grid);")

@@ -41,8 +41,9 @@ struct RowArgs {
   float eps;                 // layer norm
   int vecA, vecB;            // rows of A / B may be read with 16-byte loads
   float* colws;              // per-column reductions of the epilogue: [workgroups][COL_STATE][N] partials
-  int fast;                  // N >= 8 and every anchor operand is dword aligned: whole 8-column groups move as 16
-                             // bytes without checks, the group that straddles the row end (N % 8 != 0) on its own
+  int fast;                  // every anchor operand is dword aligned and 2: N % 8 == 0, whole 8-column groups only;
+                             // 1: N >= 8, whole groups move as 16 bytes without checks, the group that straddles the
+                             // row end on its own; 0: neither
 };
 
 // ELT: 0 = f16, 1 = bf16, 2 = f32 element type of the anchor operands
@@ -243,6 +244,49 @@ EVT_DEV void store8v(T* p, const float (&val)[8]) {
   }
 }
 
+// The same through buffer instructions, for kernels whose lanes all work on one row (RowCfg::RPW == 1): `rs`
+// starts at the row, a lane without columns passes kOobOffset and the hardware drops its access (loads give 0).
+// No lane is masked off and no branch surrounds the access, so the compiler knows how many memory operations
+// an iteration issues and can wait for the row fetched ahead without also waiting for the stores behind it.
+// a pointer that has the same value in every lane, moved to scalar registers
+EVT_DEV const char* wave_uniform(const void* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+template <class T>
+EVT_DEV void load8v_b(__amdgpu_buffer_rsrc_t rs, uint32_t voff, float (&out)[8]) {
+  constexpr int Q = (sizeof(T) * 8 + 15) / 16;
+  union { q16 q[Q]; q8 h; T e[8]; } u;
+  if constexpr (sizeof(T) * 8 >= 16) {
+#pragma unroll
+    for (int i = 0; i < Q; ++i) u.q[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + 16 * i, 0, 0);
+  } else {
+    u.h = __builtin_bit_cast(q8, __builtin_amdgcn_raw_buffer_load_b64(rs, voff, 0, 0));
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if constexpr (std::is_same<T, bool>::value) out[j] = u.e[j] ? 1.f : 0.f;
+    else out[j] = (float)u.e[j];
+  }
+}
+template <class T>
+EVT_DEV void store8v_b(__amdgpu_buffer_rsrc_t rs, uint32_t voff, const float (&val)[8]) {
+  constexpr int Q = (sizeof(T) * 8 + 15) / 16;
+  union { q16 q[Q]; q8 h; T e[8]; } u;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if constexpr (std::is_same<T, bool>::value) u.e[j] = val[j] != 0.f;
+    else u.e[j] = (T)val[j];
+  }
+  if constexpr (sizeof(T) * 8 >= 16) {
+#pragma unroll
+    for (int i = 0; i < Q; ++i) __builtin_amdgcn_raw_buffer_store_b128(u.q[i], rs, voff + 16 * i, 0, 0);
+  } else {
+    __builtin_amdgcn_raw_buffer_store_b64(u.h, rs, voff, 0, 0);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // the four anchors: fill acc[CH][8] (and rv[0..1] = per-row values) for row t
 // ---------------------------------------------------------------------------
@@ -273,28 +317,32 @@ EVT_DEV void load8_raw(const T* p, bool vec, int valid, T fill, T (&out)[8]) {
   }
 }
 
-template <class Cfg, bool FAST>
+template <class Cfg, int FAST>
 EVT_DEV void row_fetch_one(const char* base, int64_t ld, int64_t bs, int vec, const RowCtx<Cfg>& t, float fill,
                            typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8]) {
   using T = typename RowElt<Cfg::ELT>::type;
-  const T* row = reinterpret_cast<const T*>(base) + (int64_t)t.l * bs + (int64_t)t.m * ld;
-  if constexpr (FAST) {
-    // Every lane loads 16-byte groups; a lane whose group is not wholly inside the row reads the row's first
-    // group instead (always there: N >= 8) and the value is replaced afterwards: no branch in the body.  When
-    // N is no multiple of 8, one lane per row holds a group that straddles the row end; it fetches its few
-    // elements one by one in a tail of its own, so all whole groups keep the straight-line body.
+  const T* row = reinterpret_cast<const T*>(base) + (t.L == 1 ? (int64_t)0 : (int64_t)t.l * bs) + (int64_t)t.m * ld;
+  // FAST 2: N is a multiple of 8 and the rows are dword aligned; FAST 1: the rows are dword aligned and N >= 8.
+  if constexpr (FAST != 0) {
+    // Every lane loads 16-byte groups; a lane whose group is not (wholly) inside the row reads the row's first
+    // group instead (always there) and the value is replaced afterwards: no branch in the body.  FAST 1: one
+    // lane per row holds a group that straddles the row end; it fetches its few elements one by one in a tail
+    // of its own, so all whole groups keep the straight-line body.
     constexpr int Q = sizeof(T) * 8 / 16;
 #pragma unroll
     for (int c = 0; c < Cfg::CH; ++c) {
-      const bool full = t.valid(c) == 8;
+      const bool full = FAST == 2 ? t.col0(c) < t.N : t.valid(c) == 8;
       union { q16 q[Q]; T e[8]; } u;
       const q16* src = reinterpret_cast<const q16*>(row + (full ? t.col0(c) : 0));
 #pragma unroll
       for (int i = 0; i < Q; ++i) u.q[i] = src[i];
+      // FAST 2: the registers are taken as they come; groups past the row end are replaced by `fill` when the
+      // row is consumed (row_widen), so that nothing here waits for the loads and a row fetched ahead stays in
+      // flight under the arithmetic of the row before it
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[c][j] = full ? u.e[j] : (T)fill;
+      for (int j = 0; j < 8; ++j) x[c][j] = (FAST == 2 || full) ? u.e[j] : (T)fill;
     }
-    if (t.N & 7) {      // wave-uniform
+    if constexpr (FAST == 1) {
 #pragma unroll
       for (int c = 0; c < Cfg::CH; ++c) {
         const int v = t.valid(c);
@@ -319,22 +367,26 @@ EVT_DEV void row_fetch_one(const char* base, int64_t ld, int64_t bs, int vec, co
   }
 }
 
-template <class Cfg, bool FAST>
+template <class Cfg, int FAST>
 EVT_DEV void row_fetch(const RowArgs& g, const RowCtx<Cfg>& t, RowRaw<Cfg>& raw) {
   row_fetch_one<Cfg, FAST>(g.A, g.lda, g.bsA, g.vecA, t, Cfg::OP == ROW_SOFTMAX ? -INFINITY : 0.f, raw.a);
   if constexpr (RowRaw<Cfg>::TWO) row_fetch_one<Cfg, FAST>(g.B, g.ldb, g.bsB, g.vecB, t, 0.f, raw.b);
   if constexpr (Cfg::OP == ROW_LAYERNORM_BWD) { raw.mean = g.mean[t.r]; raw.rstd = g.rstd[t.r]; }
 }
 
-template <class Cfg>
-EVT_DEV void row_widen(const typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8], float (&y)[Cfg::CH][8]) {
+// FAST 2: lanes whose group lies past the row end hold some other group's values (row_fetch_one): `fill` there
+template <class Cfg, int FAST>
+EVT_DEV void row_widen(const RowCtx<Cfg>& t, float fill, const typename RowElt<Cfg::ELT>::type (&x)[Cfg::CH][8],
+                       float (&y)[Cfg::CH][8]) {
 #pragma unroll
-  for (int c = 0; c < Cfg::CH; ++c)
+  for (int c = 0; c < Cfg::CH; ++c) {
+    const bool in = FAST != 2 || t.col0(c) < t.N;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) y[c][j] = (float)x[c][j];
+    for (int j = 0; j < 8; ++j) y[c][j] = in ? (float)x[c][j] : fill;
+  }
 }
 
-template <class Cfg>
+template <class Cfg, int FAST>
 EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>& raw, const float (&gz)[Cfg::CH][8],
                       float (&acc)[Cfg::CH][8], float (&rv)[2], float (&av)[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8],
                       RowReduce<Cfg>& red) {
@@ -342,7 +394,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
   const float rn = 1.f / (float)g.N;
   if constexpr (Cfg::OP == ROW_SOFTMAX) {
     // aten._softmax over the last axis: exp(x - max) / sum, all in fp32
-    row_widen<Cfg>(raw.a, acc);
+    row_widen<Cfg, FAST>(t, -INFINITY, raw.a, acc);
     float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -368,8 +420,8 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
   } else if constexpr (Cfg::OP == ROW_SOFTMAX_BWD) {
     // aten._softmax_backward_data: (g - sum(g * y)) * y
     float y[CH][8];
-    row_widen<Cfg>(raw.a, acc);
-    row_widen<Cfg>(raw.b, y);
+    row_widen<Cfg, FAST>(t, 0.f, raw.a, acc);
+    row_widen<Cfg, FAST>(t, 0.f, raw.b, y);
     float s = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -384,7 +436,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
   } else if constexpr (Cfg::OP == ROW_LAYERNORM) {
     // aten.native_layer_norm without weight and bias: (x - mean) * rstd, mean, rstd;
     // two passes over the registers (mean first, then centred squares)
-    row_widen<Cfg>(raw.a, acc);
+    row_widen<Cfg, FAST>(t, 0.f, raw.a, acc);
     float s = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -413,7 +465,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
     //   xh = (x - mean) rstd ;  dx = rstd (g - mean_n(g) - xh mean_n(g xh))
     //   (g already multiplied by the weight when there is one)
     float xh[CH][8];
-    row_widen<Cfg>(raw.a, acc);
+    row_widen<Cfg, FAST>(t, 0.f, raw.a, acc);
     if constexpr (Cfg::AV >= 1) {      // the weight / bias gradients are column sums of g * xhat and of g
 #pragma unroll
       for (int c = 0; c < CH; ++c)
@@ -426,7 +478,7 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[c][j] *= gz[c][j];
     }
-    row_widen<Cfg>(raw.b, xh);
+    row_widen<Cfg, FAST>(t, 0.f, raw.b, xh);
     const float mean = raw.mean, rstd = raw.rstd;
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -456,29 +508,65 @@ EVT_DEV void row_main(const RowArgs& g, const RowCtx<Cfg>& t, const RowRaw<Cfg>&
   (void)av;
 }
 
-// Each wave walks rows first, first + stride, ... (stride = all waves of the
-// grid x rows per wave) and fetches the next row before it reduces the present
-// one, so a wave always has a row's worth of loads in flight; the grid is sized
-// to fill the chip once instead of one workgroup per handful of rows.
-template <class Cfg, class Epi, bool FAST>
+// Rows are dealt in runs: walker w (a wave, or the workgroup when it shares a
+// row) visits rows [w * run, (w + 1) * run), RPW at a time, and fetches the
+// next visit's rows before it reduces the present ones, so it always has a
+// row's worth of loads in flight; the grid is sized to fill the chip once
+// instead of one workgroup per handful of rows.  A run of consecutive rows lets
+// the per-row outputs of the epilogue (a layer norm's mean and rstd) leave
+// together: lane j keeps the values of the j-th row since the last flush, and
+// up to 64 rows are written by one store instruction per output.  One 4-byte
+// store per row and output costs a fifth of the kernel's time on 131072 x 1024.
+template <class Cfg, class Epi, int FAST>
 __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typename Epi::Params p) {
   constexpr int CS = Epi::COL_STATE;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t rows = (int64_t)g.L * g.M;
-  const int64_t stride = (int64_t)gridDim.x * Cfg::ROWS;
+  constexpr int STEP = Cfg::WPR > 1 ? 1 : Cfg::RPW;        // rows per visit
+  const int64_t walkers = Cfg::WPR > 1 ? (int64_t)gridDim.x : (int64_t)gridDim.x * Cfg::WAVES;
+  const int64_t me = Cfg::WPR > 1 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * Cfg::WAVES + wave;
+  // With per-row outputs in the epilogue a walker takes a run of consecutive rows (RUNS), so that their outputs
+  // can leave together; otherwise the walkers' rows interleave (visit k of walker w is row block w + k * walkers),
+  // which keeps the whole chip inside one window of the tensor at any time and measures a few percent faster.
+  constexpr bool RUNS = Epi::NRS > 0;
+  const int64_t run = RUNS ? (rows + walkers * STEP - 1) / (walkers * STEP) * STEP : rows;
+  const int64_t first = RUNS ? me * run : me * STEP;
+  const int64_t end = (RUNS && first + run < rows) ? first + run : rows;
+  const int64_t stride = RUNS ? (int64_t)STEP : walkers * STEP;      // from one visit to the next
   RowCtx<Cfg> t;
   t.M = g.M; t.N = g.N; t.L = g.L;
   t.sub = Cfg::WPR > 1 ? (int)threadIdx.x : lane % Cfg::LPR;
   __shared__ float xch[2 * 16];
   RowReduce<Cfg> red{xch, 0};
   static_assert(CS == 0 || Cfg::WPR == 1, "per-column reductions need a row per wave");
+  // (batch, row in the batch) of the walker's present row: kept up to date by addition, since the rows of a run
+  // follow each other (a 64-bit division per visit costs more instructions than the rest of a short row's work).
+  // Batches shorter than 64 rows take the division.
+  const bool stepwise = RUNS && g.M >= 64;                                  // uniform
+  int cur_l = 0, cur_m = 0;                                                 // of row `base`
+  if (first < rows) { cur_l = (int)(first / g.M); cur_m = (int)(first % g.M); }
   auto locate = [&](int64_t base) {
-    const int64_t r = base + (Cfg::WPR > 1 ? 0 : lane / Cfg::LPR);
-    t.ok = r < rows;
+    const int sub_row = Cfg::WPR > 1 ? 0 : lane / Cfg::LPR;
+    const int64_t r = base + sub_row;
+    t.ok = r < end;                 // rows from `end` on belong to the next walker (or do not exist)
     t.r = t.ok ? r : rows - 1;      // lanes past the end recompute the last row and store nothing
-    t.l = (int)(t.r / g.M);
-    t.m = (int)(t.r % g.M);
+    if (stepwise) {
+      int m = cur_m + sub_row, l = cur_l;
+      if (m >= g.M) { m -= g.M; l += 1; }
+      t.l = t.ok ? l : g.L - 1;
+      t.m = t.ok ? m : g.M - 1;
+    } else if (g.L == 1) {          // uniform: a single batch needs no division
+      t.l = 0;
+      t.m = (int)t.r;
+    } else {
+      t.l = (int)(t.r / g.M);
+      t.m = (int)(t.r % g.M);
+    }
+  };
+  auto advance = [&]() {            // `base` moves on by one visit
+    cur_m += STEP;
+    if (cur_m >= g.M) { cur_m -= g.M; cur_l += 1; }
   };
   // this lane's share of the epilogue's per-column reductions, carried over all rows the wave visits
   float cst[CS > 0 ? CS : 1][Cfg::CH][8];
@@ -495,11 +583,15 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
   }
   // wave-uniform; the same for every wave of the workgroup when they share a row (so all of them reach the barriers
   // of the reductions the same number of times)
-  int64_t base = Cfg::WPR > 1 ? (int64_t)blockIdx.x : ((int64_t)blockIdx.x * Cfg::WAVES + wave) * Cfg::RPW;
-  if (base < rows) {
-    RowRaw<Cfg> cur;
+  int64_t base = first;
+  // per-row outputs on their way out: lane j holds those of row flush_first + j
+  constexpr int NRS = Epi::NRS;
+  float hold[NRS > 0 ? NRS : 1];
+  int64_t flush_first = first;
+  int flush_l = cur_l, flush_m = cur_m;      // (batch, row) of flush_first
+  int held = 0;
+  if (base < end) {
     locate(base);
-    row_fetch<Cfg, FAST>(g, t, cur);
     float hz[Epi::NH > 0 ? Epi::NH : 1][Cfg::CH][8];
     Epi::template hoist<Cfg, FAST>(p, t, hz);
     float gz[Cfg::CH][8];          // layer norm backward: this lane's columns of the weight, read once
@@ -518,30 +610,73 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
         }
       }
     }
-    while (true) {
-      const RowCtx<Cfg> here = t;
-      const int64_t next = base + stride;
-      const bool more = next < rows;                                         // wave-uniform
-      RowRaw<Cfg> ahead;
-      if constexpr (Cfg::LOOKAHEAD) {
-        if (more) {
-          locate(next);
-          row_fetch<Cfg, FAST>(g, t, ahead);
-        }
-      }
+    // everything that happens to one fetched row; `more`: the walker has further rows
+    auto consume = [&](const RowCtx<Cfg>& here, const RowRaw<Cfg>& raw, bool more) {
       float acc[Cfg::CH][8];
       float rv[2];
       float av[Cfg::AV > 0 ? Cfg::AV : 1][Cfg::CH][8];
-      row_main<Cfg>(g, here, cur, gz, acc, rv, av, red);
-      if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, av, hz, cst);
-      if (!more) break;
-      if constexpr (Cfg::LOOKAHEAD) {
-        cur = ahead;
-      } else {
-        locate(next);
-        row_fetch<Cfg, FAST>(g, t, cur);
+      row_main<Cfg, FAST>(g, here, raw, gz, acc, rv, av, red);
+      float rsv[NRS > 0 ? NRS : 1];
+      if (here.ok) Epi::template row<Cfg, FAST>(p, here, acc, rv, av, hz, cst, rsv);
+      if constexpr (NRS > 0) {
+        // the rows of this visit take slots held .. held + STEP - 1 (STEP divides 64, so a visit never wraps)
+#pragma unroll
+        for (int i = 0; i < NRS; ++i) {
+          float v = rsv[i];
+          if constexpr (STEP > 1) v = __shfl(v, ((lane - held) & (STEP - 1)) * Cfg::LPR, 64);   // row group -> slot lane
+          if (lane >= held && lane < held + STEP) hold[i] = v;
+        }
+        held += STEP;
+        if (held == 64 || !more) {
+          const int64_t r = flush_first + lane;
+          if (lane < held && r < end && (Cfg::WPR == 1 || wave == 0)) {
+            int l, m;
+            if (stepwise) {
+              l = flush_l; m = flush_m + lane;
+              if (m >= g.M) { m -= g.M; l += 1; }
+            } else {
+              l = (int)(r / g.M); m = (int)(r % g.M);
+            }
+#pragma unroll
+            for (int i = 0; i < NRS; ++i) Epi::row_store_one(p, g.L, l, m, i, hold[i]);
+          }
+          flush_first += held;
+          flush_m += held;
+          if (stepwise && flush_m >= g.M) { flush_m -= g.M; flush_l += 1; }
+          held = 0;
+        }
       }
-      base = next;
+    };
+    {
+      RowRaw<Cfg> cur;
+      row_fetch<Cfg, FAST>(g, t, cur);
+      // The first row is waited for here, once.  Left to the compiler, the wait sits at the top of the loop body
+      // (where the first row's registers may still be on their way), behind the fetch of the next row, and
+      // because the counter runs in issue order it would then wait for that fetch in every iteration.
+      if constexpr (Cfg::LOOKAHEAD) __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+      while (true) {
+        const RowCtx<Cfg> here = t;
+        const int64_t next = base + stride;
+        const bool more = next < end;                                          // wave-uniform
+        RowRaw<Cfg> ahead;
+        if constexpr (Cfg::LOOKAHEAD) {
+          if (more) {
+            advance();
+            locate(next);
+            row_fetch<Cfg, FAST>(g, t, ahead);
+          }
+        }
+        consume(here, cur, more);
+        if (!more) break;
+        if constexpr (Cfg::LOOKAHEAD) {
+          cur = ahead;
+        } else {
+          advance();
+          locate(next);
+          row_fetch<Cfg, FAST>(g, t, cur);
+        }
+        base = next;
+      }
     }
   }
   if constexpr (CS > 0) {
