@@ -725,12 +725,12 @@ class Codegen:
         col_folds = {r.fold for r in ir.reduces.values() if r.axis == "col"} - {""}
         if col_folds:
             # batches that agree modulo l_mod of the reduction's output tensor fold into one per-column result;
-            # their partials are combined by the last workgroup to arrive (no separate finalize kernel for this)
+            # few partials are combined by the last workgroup to arrive, many by the finalize kernel
             k = next(s_.slot for s_ in ir.stores if s_.domain == "col")
             e(f"{{ const EvtTensorArg& x = a->tensors[{k}];")
             e("  if (x.l_mod <= 0 || x.l_div != 1 || a->L % x.l_mod) return EVT_ERR_BAD_ARGS;")
             e("  g.col_fold_step = (int)x.l_mod; g.col_fold_count = a->L / (int)x.l_mod;")
-            e("  if ((int64_t)g.tiles_m * g.col_fold_count > evt::kMaxInKernelPartials || two_kernel_reduce) return EVT_ERR_RANGE; }")
+            e("}")
         e("g.col_inkernel = (g.tiles_m * g.col_fold_count <= evt::kMaxInKernelPartials && !two_kernel_reduce) ? 1 : 0;")
         e("// Split-K: when the output tiles cannot fill the chip and K is long, several workgroups share a tile")
         e("// (EvtArgs.split_k: 0 = decide here, 1 = off, n = n splits)")

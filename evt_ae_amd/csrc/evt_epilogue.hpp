@@ -900,32 +900,38 @@ __global__ void __launch_bounds__(256) evt_row_finalize_kernel(typename Epi::Par
 }
 
 // Phase 2 of per-column reductions: a block of 256 threads covers 256 / G
-// columns; G threads per column each fold every G-th tile partial (in tile
-// order), LDS combines the G results in order.  Threads of equal share index
-// read adjacent columns, i.e. adjacent addresses.
+// columns; G threads per column each fold every G-th partial (batches of a
+// fold in fold order, tiles in tile order), LDS combines the G results in
+// order.  Threads of equal share index read adjacent columns, i.e. adjacent
+// addresses.  One result per (fold key, column): without a fold the key is
+// the batch.
 template <class Epi>
-__global__ void __launch_bounds__(256) evt_col_finalize_kernel(typename Epi::Params p, const float* part,
-                                                               int N, int L, int tiles_m, int G) {
+__global__ void __launch_bounds__(256) evt_col_finalize_kernel(typename Epi::Params p, const float* part, GemmArgs g, int G) {
   constexpr int CS = Epi::COL_STATE > 0 ? Epi::COL_STATE : 1;
   __shared__ float lds[256 * CS];
+  const int N = g.N, tiles_m = g.tiles_m;
+  const int keys = g.L / g.col_fold_count;
   const int per = 256 / G;
   const int sub = threadIdx.x / per, c = threadIdx.x % per;
   const int64_t colid = (int64_t)blockIdx.x * per + c;
-  const bool live = colid < (int64_t)L * N;
-  const int batch = live ? (int)(colid / N) : 0, col = live ? (int)(colid % N) : 0;
+  const bool live = colid < (int64_t)keys * N;
+  const int key = live ? (int)(colid / N) : 0, col = live ? (int)(colid % N) : 0;
   float st[CS];
   Epi::col_identity(st);
   if (live) {
-    const float* src = part + ((int64_t)batch * tiles_m * N + col) * CS;
+    const int nq = tiles_m * g.col_fold_count;
 #pragma unroll 4
-    for (int j = sub; j < tiles_m; j += G) Epi::col_combine(st, src + (int64_t)j * N * CS);
+    for (int q = sub; q < nq; q += G) {
+      const int f = q / tiles_m, j = q - f * tiles_m;
+      Epi::col_combine(st, part + (((int64_t)col_fold_member(g, key, f) * tiles_m + j) * N + col) * CS);
+    }
   }
 #pragma unroll
   for (int k = 0; k < CS; ++k) lds[threadIdx.x * CS + k] = st[k];
   __syncthreads();
   if (live && sub == 0) {
     for (int s2 = 1; s2 < G; ++s2) Epi::col_combine(st, lds + (s2 * per + c) * CS);
-    Epi::col_finalize(p, batch, col, st);
+    Epi::col_finalize(p, col_fold_member(g, key, 0), col, st);
   }
 }
 
@@ -949,14 +955,14 @@ inline int launch_finalize(const typename Epi::Params& p, const GemmArgs& g, hip
       default: hipLaunchKernelGGL((evt_row_finalize_kernel<Epi, 6>), dim3(grid), dim3(256), 0, stream, p, part, g); break;
     }
   }
-  if (Epi::COL_STATE > 0 && g.tiles_m > 1 && !g.col_inkernel) {
+  if (Epi::COL_STATE > 0 && col_uses_workspace(g) && !g.col_inkernel) {
     const float* part = (const float*)(g.workspace + wl.counter_bytes + wl.row_bytes);
     int G = 1;
-    while (G < 16 && G * 4 <= g.tiles_m) G *= 2;      // >= 4 partials per thread
+    while (G < 16 && G * 4 <= g.tiles_m * g.col_fold_count) G *= 2;      // >= 4 partials per thread
     const int per = 256 / G;
-    const int64_t cols = (int64_t)g.L * g.N;
+    const int64_t cols = (int64_t)(g.L / g.col_fold_count) * g.N;
     hipLaunchKernelGGL((evt_col_finalize_kernel<Epi>), dim3((unsigned)((cols + per - 1) / per)), dim3(256), 0, stream,
-                       p, part, g.N, g.L, g.tiles_m, G);
+                       p, part, g, G);
   }
   return (int)hipGetLastError();
 }

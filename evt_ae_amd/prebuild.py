@@ -72,6 +72,8 @@ def register_all() -> List[jit.LazyModule]:
     for transposed in (False, True):
         mod, ins = W.head_merge_bias_grad(transposed=transposed)
         W.fuse(mod, _meta(ins))
+        mod, ins = W.head_merge_bias_grad(transposed=transposed, **W.HEAD_MERGE_MANY_PARTIALS)
+        W.fuse(mod, _meta(ins))
     for anchor in W.RANDOM_EPILOGUE_ANCHORS:
         for seed in W.RANDOM_EPILOGUE_SEEDS[:12 if anchor == "mm" else 6]:
             mod, ins = W.random_epilogue(seed, anchor)

@@ -905,6 +905,11 @@ class HeadMergeBiasGrad(torch.nn.Module):
         return w, aten.view(aten.sum(w, [0], True), [H * D])
 
 
+# more batches per result than the last workgroup of a column block combines itself (64 partials): 24 batches x
+# 3 .. 10 row tiles per result, finished by the finalize kernel
+HEAD_MERGE_MANY_PARTIALS = dict(B=24, H=2, S=640, D=64, K=32)
+
+
 def head_merge_bias_grad(B: int = 4, H: int = 6, S: int = 320, D: int = 64, K: int = 96, transposed: bool = False,
                          seed: int = 0):
     g = torch.Generator(device="cpu").manual_seed(0xB1A5 + seed)

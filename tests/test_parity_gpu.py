@@ -744,18 +744,27 @@ def test_bench_argument_sets_are_independent():
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("phase2", ["in_kernel", "finalize_kernel", "many_partials"])
 @pytest.mark.parametrize("transposed", [False, True], ids=["per_column", "per_row"])
-def test_bias_gradient_behind_a_head_merge(transposed):
+def test_bias_gradient_behind_a_head_merge(transposed, phase2, monkeypatch):
     """The backward pattern of an attention projection: batched product over
     B * H heads, result merged into [B * S, H * D] by the store, bias gradient
     = sum over all rows, i.e. per column (or, for the transposed product, per
     row) and over the batches that agree modulo H.  Several row tiles and
-    several batches per result; repeated launches are bit-identical."""
-    mod, inputs = W.head_merge_bias_grad(transposed=transposed)
+    several batches per result, combined by the last workgroup to arrive, by the
+    finalize kernel on request, and by the finalize kernel because there are
+    more partials per result (24 batches x the row tiles) than a workgroup
+    combines; repeated launches are bit-identical."""
+    if phase2 == "finalize_kernel":
+        monkeypatch.setenv("EVT_TWO_KERNEL_REDUCE", "1")
+    many = phase2 == "many_partials"
+    mod, inputs = W.head_merge_bias_grad(transposed=transposed, **(W.HEAD_MERGE_MANY_PARTIALS if many else {}))
     gm = W.fuse(mod, inputs)
     (node,) = fused_nodes(gm)
     (red,) = node.target.ir.reduces.values()
-    assert red.fold == "mod" and red.axis == ("row" if transposed else "col") and red.fold_count == 4
+    assert red.fold == "mod" and red.axis == ("row" if transposed else "col") and red.fold_count == (24 if many else 4)
+    if many and not transposed:
+        assert -(-node.target.problem[0] // node.target.tile.bm) * red.fold_count > 64
     dev = [t.cuda() for t in inputs]
     outs = [o.clone() for o in gm(*dev)]
     again = gm(*dev)
