@@ -16,6 +16,7 @@ import operator
 import itertools
 import os
 from contextlib import nullcontext
+from dataclasses import replace
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -473,21 +474,30 @@ class FusedGEMM(FusedOpBase):
     def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
         super().__init__(node, epilogue_visitor)
         lhs_node, rhs_node = node.args[0], node.args[1]
+        lhs_shape, dtype = node_shape_dtype(lhs_node)
+        rhs_shape, _ = node_shape_dtype(rhs_node)
+        M, K = lhs_shape[-2:]
+        N = rhs_shape[-1]
+        # A column-major output is computed as C^T = B^T A^T (reference: the `transposed` problems of
+        # evt_fuser.py:573-596): the operands change places, and what was row-major is read as column-major.
+        self.transposed = bool(getattr(epilogue_visitor, "transposed", False))
+        if self.transposed:
+            lhs_node, rhs_node = rhs_node, lhs_node
+            M, N = N, M
         self.lhs_layout = self.get_src_layout(lhs_node)
         self.rhs_layout = self.get_src_layout(rhs_node)
         self.A = self.get_src(lhs_node)
         self.B = self.get_src(rhs_node)
         self.args = [self.A, self.B]
-
-        lhs_shape, dtype = node_shape_dtype(lhs_node)
-        rhs_shape, _ = node_shape_dtype(rhs_node)
-        M, K = lhs_shape[-2:]
-        N = rhs_shape[-1]
         self.problem = (M, N, K, 1)
         if dtype not in (torch.float16, torch.bfloat16):
             raise NotImplementedError(f"GEMM operands of dtype {dtype}")
-        self.a_kc = self.lhs_layout == "RowMajor"
-        self.b_kc = self.rhs_layout == "ColumnMajor"
+        if self.transposed:     # the new A is the old B seen as [N, K], the new B the old A seen as [K, M]
+            self.a_kc = self.lhs_layout == "ColumnMajor"
+            self.b_kc = self.rhs_layout == "RowMajor"
+        else:
+            self.a_kc = self.lhs_layout == "RowMajor"
+            self.b_kc = self.rhs_layout == "ColumnMajor"
         self.lda = K if self.a_kc else M
         self.ldb = K if self.b_kc else N
         dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb, 0, 0)
@@ -516,7 +526,8 @@ class FusedGEMM(FusedOpBase):
         return A, self.lda, 0, B, self.ldb, 0
 
     def anchor_eager(self, A, B):
-        return torch.mm(A if self.a_kc else A.t(), B.t() if self.b_kc else B)
+        C = torch.mm(A if self.a_kc else A.t(), B.t() if self.b_kc else B)
+        return C.t() if self.transposed else C
 
     def get_src_layout(self, node: Node) -> str:
         if packet(node.target) == aten.permute and node.name in self.partition_names:
@@ -546,7 +557,6 @@ class FusedBMM(FusedOpBase):
         rhs_shape, _ = node_shape_dtype(rhs_node)
         L, M, K = lhs_shape
         N = rhs_shape[-1]
-        self.problem = (M, N, K, L)
         if dtype not in (torch.float16, torch.bfloat16):
             raise NotImplementedError(f"BMM operands of dtype {dtype}")
 
@@ -557,6 +567,15 @@ class FusedBMM(FusedOpBase):
         self.chain_B, self.B = operand_chain(rhs_node, inside)
         sa = operand_strides(self.chain_A, lhs_shape)
         sb = operand_strides(self.chain_B, rhs_shape)
+        # A column-major output is computed as C^T = B^T A^T (reference: evt_fuser.py:573-596): the operands change
+        # places, each seen transposed (its m and n strides exchanged).
+        self.transposed = bool(getattr(epilogue_visitor, "transposed", False))
+        if self.transposed:
+            flip = lambda st: None if st is None else replace(st, stride_m=st.stride_n, stride_n=st.stride_m)   # noqa: E731
+            self.chain_A, self.chain_B, self.A, self.B = self.chain_B, self.chain_A, self.B, self.A
+            sa, sb = flip(sb), flip(sa)
+            M, N = N, M
+        self.problem = (M, N, K, L)
         self.args = [self.A, self.B]
         self.copy_A = self.copy_B = False
         self.bdiva, self.bs2a, self.bdivb, self.bs2b = 1, 0, 1, 0
@@ -609,10 +628,14 @@ class FusedBMM(FusedOpBase):
         return x
 
     def operands(self, A, B):
+        # a copied operand is laid out as the kernel's [L, M, K] / [L, K, N]; in a transposed problem the eager
+        # chain yields it the other way round
         if self.copy_A:
-            A = self._replay(self.chain_A, A).contiguous()
+            A = self._replay(self.chain_A, A)
+            A = (A.transpose(1, 2) if self.transposed else A).contiguous()
         if self.copy_B:
-            B = self._replay(self.chain_B, B).contiguous()
+            B = self._replay(self.chain_B, B)
+            B = (B.transpose(1, 2) if self.transposed else B).contiguous()
         return A, self.lda, self.bsa, B, self.ldb, self.bsb
 
     def build_arguments(self, visitor_args, *args, block=None):
@@ -626,6 +649,8 @@ class FusedBMM(FusedOpBase):
         return a, keep
 
     def anchor_eager(self, A, B):
+        if self.transposed:     # A, B are the original right and left operands
+            return torch.bmm(self._replay(self.chain_B, B), self._replay(self.chain_A, A))
         return torch.bmm(self._replay(self.chain_A, A), self._replay(self.chain_B, B))
 
 
@@ -743,6 +768,8 @@ class EVTFuser:
                          aten.native_layer_norm_backward]
     row_targets = {aten._softmax: FusedSoftmax, aten._softmax_backward_data: FusedSoftmaxBackward,
                    aten.native_layer_norm: FusedLayerNorm, aten.native_layer_norm_backward: FusedLayerNormBackward}
+    # compute C^T = B^T A^T when the outputs are column-major (tests switch it off to reach the strided stores)
+    allow_transpose = True
 
     def __init__(self, element_compute=torch.float32, **kwargs):
         self.element_compute = element_compute
@@ -912,11 +939,17 @@ class EVTFuser:
         for out in outputs:
             self._insert_store(out, store_key)
         self.ir.finalize()
+        # a column-major output: compute the transposed product instead (operands exchanged by the fused op), so
+        # that the stores run along the kernel's n
+        self.transposed = False
+        if self.allow_transpose and tgt not in self.row_targets and self.ir.wants_transpose():
+            self.ir.transpose()
+            self.ir.finalize()
+            self.transposed = True
         # slot indices may have been compacted by finalize(): rebuild the map
         self._rebuild_slot_sources()
         self.return_names = [o.name for o in outputs]
         self.reduction_names = [s.name for s in self.ir.slots if s.role == "store" and s.domain != "tile"]
-        self.transposed = False
 
         return self.get_fused_node(anchor)
 

@@ -23,7 +23,7 @@ from __future__ import annotations
 
 import hashlib
 import json
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, replace
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -468,6 +468,42 @@ class EpilogueIR:
         live = set(self.live_nodes())
         used = {self.nodes[n].reduce for n in live if self.nodes[n].op == "rres"}
         return [r for r in self.reduces.values() if r.name in used]
+
+    # -- transposed problems ---------------------------------------------------
+    def wants_transpose(self) -> bool:
+        """True when every full-tensor access of the epilogue is strided along n and
+        the stores are unit-stride along m: the output is column-major, and
+        computing C^T = B^T A^T instead gives the kernel unit-stride (vector,
+        check-free) accesses.  The counterpart of the reference's `transposed`
+        problems (python/gtl/compiler/passes/evt_fuser.py:573-596)."""
+        if self.M <= 1 or self.N <= 1:
+            return False
+        tile = [s for s in self.slots if s.domain == "tile" and s.kind == "aux"]
+        stores = [s for s in tile if s.role == "store"]
+        if not stores:
+            return False
+        if any(n.op == "colidx" for n in self.nodes.values()):
+            return False            # there is no row-index value to take its place
+        for r in self.reduces.values():
+            if r.axis == "row" and (r.kind not in ("sum", "max") or r.fold == "div"):
+                return False        # per-column reductions are sums and maxima, folded modulo only
+        return all(s.strides.stride_n != 1 for s in tile) and all(s.strides.stride_m == 1 for s in stores)
+
+    def transpose(self) -> None:
+        """Exchange the roles of m and n everywhere: the IR then describes the
+        epilogue of the transposed product (call finalize() again afterwards)."""
+        swap = {"row": "col", "col": "row"}
+        self.M, self.N = self.N, self.M
+        for s in self.slots:
+            s.strides = replace(s.strides, stride_m=s.strides.stride_n, stride_n=s.strides.stride_m)
+            s.domain = swap.get(s.domain, s.domain)
+            s.kind = swap.get(s.kind, s.kind)
+        for n in self.nodes.values():
+            n.domain = swap.get(n.domain, n.domain)
+        for r in self.reduces.values():
+            r.axis = swap[r.axis]
+        for st in self.stores:
+            st.domain = swap.get(st.domain, st.domain)
 
     def finalize(self) -> None:
         """Dead-code elimination, state packing, validation."""

@@ -69,11 +69,20 @@ def register_all() -> List[jit.LazyModule]:
     for n in W.AFFINE_LN_LENGTHS:
         mod, ins = W.affine_layer_norm(n)
         W.fuse(mod, _meta(ins), passes=[pass_decomposition, pass_fusion])
-    for transposed in (False, True):
-        mod, ins = W.head_merge_bias_grad(transposed=transposed)
-        W.fuse(mod, _meta(ins))
-        mod, ins = W.head_merge_bias_grad(transposed=transposed, **W.HEAD_MERGE_MANY_PARTIALS)
-        W.fuse(mod, _meta(ins))
+    from .evt_fuser import EVTFuser
+    for swap in (True, False):          # column-major outputs: operands exchanged, and the strided stores without
+        EVTFuser.allow_transpose = swap
+        try:
+            for transposed in (False, True):
+                mod, ins = W.head_merge_bias_grad(transposed=transposed)
+                W.fuse(mod, _meta(ins))
+                mod, ins = W.head_merge_bias_grad(transposed=transposed, **W.HEAD_MERGE_MANY_PARTIALS)
+                W.fuse(mod, _meta(ins))
+            for batched in (False, True):
+                mod, ins = W.column_major_store(batched)
+                W.fuse(mod, _meta(ins))
+        finally:
+            EVTFuser.allow_transpose = True
     for anchor in W.RANDOM_EPILOGUE_ANCHORS:
         for seed in W.RANDOM_EPILOGUE_SEEDS[:12 if anchor == "mm" else 6]:
             mod, ins = W.random_epilogue(seed, anchor)

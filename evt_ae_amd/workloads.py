@@ -919,6 +919,33 @@ def head_merge_bias_grad(B: int = 4, H: int = 6, S: int = 320, D: int = 64, K: i
     return HeadMergeBiasGrad(B, H, S, D, transposed), [a, b]
 
 
+class ColumnMajorStore(torch.nn.Module):
+    """A product whose result leaves the kernel transposed: gelu(a @ b + bias +
+    r^T) stored as [N, M] (permute + copy, folded into the store), r read
+    through the same permute, with a reduction of the stored values on top --
+    the bias-gradient sum over all rows for the GEMM, a maximum along every
+    row for the batched product.  The column-major outputs of the reference's
+    `transposed` problems (evt_fuser.py:573-596)."""
+    def __init__(self, batched: bool) -> None:
+        super().__init__()
+        self.batched = batched
+
+    def forward(self, a, b, bias, r):
+        perm = [0, 2, 1] if self.batched else [1, 0]
+        out = aten.bmm(a, b) if self.batched else aten.mm(a, b)
+        y = aten.gelu(aten.add(aten.add(out, bias), aten.permute(r, perm)))
+        yt = aten.clone(aten.permute(y, perm), memory_format=torch.contiguous_format)
+        red = aten.amax(y, [2]) if self.batched else aten.sum(y, [0])
+        return yt, red
+
+
+def column_major_store(batched: bool, seed: int = 0):
+    g = torch.Generator(device="cpu").manual_seed(0xC01A + seed)
+    h = lambda *sh: (torch.randn(*sh, generator=g) * 0.3).half()   # noqa: E731
+    lead, (M, N, K) = ((3,), (200, 136, 64)) if batched else ((), (320, 192, 96))
+    return ColumnMajorStore(batched), [h(*lead, M, K), h(*lead, K, N), h(N), h(*lead, N, M)]
+
+
 class RandomEpilogue(torch.nn.Module):
     """A seeded random epilogue tree behind a GEMM: 5 .. 9 element-wise steps
     over the accumulator, a same-shape tensor, a row vector, a column vector

@@ -92,10 +92,13 @@ def test_batch_folded_row_reductions_lower_correctly():
     inputs = W.pattern_inputs("bmm2")
     gm = _check(W.BMMPartition2, inputs)
     (n,) = fused_nodes(gm)
+    # the product is stored with the row index fastest, so the problem is computed transposed
+    # (evt_fuser.py:573-596): the sum over the sequence axis is then one per column
+    assert n.target.transposed
     (red,) = n.target.ir.reduces.values()
-    assert (red.axis, red.fold, red.fold_step, red.fold_count) == ("row", "mod", 16, 2)
-    (st,) = [s.strides for s in n.target.ir.slots if s.domain == "row"]
-    assert (st.l_mod, st.l_div, st.stride_l, st.stride_m, st.stride_n) == (16, 1, 64, 1, 0)
+    assert (red.axis, red.fold, red.fold_step, red.fold_count) == ("col", "mod", 16, 2)
+    (st,) = [s.strides for s in n.target.ir.slots if s.domain == "col"]
+    assert (st.l_mod, st.l_div, st.stride_l, st.stride_m, st.stride_n) == (16, 1, 64, 0, 1)
 
     gm = _check(W.FoldConsecutiveBatches, W.fold_consecutive_inputs())
     (n,) = fused_nodes(gm)
@@ -375,23 +378,59 @@ def test_rows_too_long_for_the_row_kernel_stay_eager():
     assert [target_name(n.target) for n in gm.graph.nodes if n.op == "call_function"] == ["_softmax", "mul"]
 
 
-@pytest.mark.parametrize("transposed", [False, True])
-def test_bias_gradient_behind_a_head_merge_lowers_correctly(transposed):
+@pytest.mark.parametrize("transposed, swap", [(False, True), (True, True), (True, False)])
+def test_bias_gradient_behind_a_head_merge_lowers_correctly(transposed, swap, monkeypatch):
     """A batched product over B * H heads, merged into [B * S, H * D] by a permuted
     store, with the bias gradient (sum over every row) on top: per column and
-    over the batches that agree modulo H, or, for the transposed product, along
-    the rows with the same fold.  One kernel, values from the IR interpreter."""
+    over the batches that agree modulo H.  The transposed product ([D, S] per
+    head) is computed with its operands exchanged and is then the same problem;
+    with the exchange switched off the same sum runs along the rows with the
+    same fold.  One kernel, values from the IR interpreter."""
+    monkeypatch.setattr(EVTFuser, "allow_transpose", swap)
     mod, inputs = W.head_merge_bias_grad(B=2, H=3, S=40, D=16, K=24, transposed=transposed)
     gm = W.fuse(mod, inputs)
     (n,) = fused_nodes(gm)
     assert not [x for x in gm.graph.nodes if x.op == "call_function" and target_name(x.target) in ("sum", "clone", "bmm")]
+    assert n.target.transposed == (transposed and swap)
+    assert n.target.problem == ((16, 40, 24, 6) if transposed and not swap else (40, 16, 24, 6))
     (red,) = n.target.ir.reduces.values()
-    assert (red.axis, red.fold, red.fold_step, red.fold_count) == ("row" if transposed else "col", "mod", 3, 2)
+    assert (red.axis, red.fold, red.fold_step, red.fold_count) == ("row" if transposed and not swap else "col", "mod", 3, 2)
     got = run_emulated(gm, inputs)
     ref = evt_oracle.eval_fp32(mod, inputs)
     for o, r in zip(got, ref):
         assert tuple(o.shape) == tuple(r.shape)
         assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3
+
+
+@pytest.mark.parametrize("batched", [False, True], ids=["mm", "bmm"])
+def test_column_major_outputs_are_computed_transposed(batched, monkeypatch):
+    """A result stored as [N, M] (permute + copy behind the epilogue) makes the
+    fused op exchange its operands and compute C^T = B^T A^T, as the reference's
+    `transposed` problems do (evt_fuser.py:573-596): the full-tensor load and
+    store then run along the kernel's n, the row vector becomes a per-row value,
+    the sum over all rows a sum along each row (the batched product's row maximum
+    a per-column maximum).  With the exchange switched off the same graph lowers
+    to strided accesses; both agree with eager fp32."""
+    mod, inputs = W.column_major_store(batched)
+    M, N, K = inputs[0].shape[-2], inputs[1].shape[-1], inputs[0].shape[-1]
+    for swap in (True, False):
+        monkeypatch.setattr(EVTFuser, "allow_transpose", swap)
+        gm = W.fuse(mod, inputs)
+        (n,) = fused_nodes(gm)
+        op = n.target
+        assert op.transposed == swap
+        assert op.problem[:3] == ((N, M, K) if swap else (M, N, K))
+        assert (op.a_kc, op.b_kc) == ((False, True) if swap else (True, False))    # the same memory, read the other way
+        full = [s.strides for s in op.ir.slots if s.domain == "tile" and s.kind == "aux"]
+        assert len(full) == 2 and all((st.stride_n == 1) == swap for st in full)
+        (red,) = op.ir.reduces.values()
+        assert red.axis == (("col" if batched else "row") if swap else ("row" if batched else "col"))
+        got = run_emulated(gm, inputs)
+        ref = evt_oracle.eval_fp32(mod, inputs)
+        assert len(got) == len(ref) == 2
+        for o, r in zip(got, ref):
+            assert tuple(o.shape) == tuple(r.shape)
+            assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3
 
 
 def test_walk_tiles_are_offered_and_refused_where_they_should(monkeypatch):

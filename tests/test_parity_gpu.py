@@ -13,6 +13,7 @@ import torch
 
 from evt_ae_amd import workloads as W
 from evt_ae_amd.autotuner.tuner_base import force_tile
+from evt_ae_amd.evt_fuser import EVTFuser
 from oracle import evt_oracle
 from evt_ae_amd.passes import target_name
 from tests.util import fused_nodes, rand_slot
@@ -744,17 +745,50 @@ def test_bench_argument_sets_are_independent():
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("swap", [True, False], ids=["operands_exchanged", "strided_store"])
+@pytest.mark.parametrize("batched", [False, True], ids=["mm", "bmm"])
+def test_column_major_outputs(batched, swap, monkeypatch):
+    """gelu(a @ b + bias + r^T) stored as [N, M], with the sum over all rows (GEMM)
+    or the maximum along every row (batched product) of the stored values: computed
+    as C^T = B^T A^T with the operands exchanged (evt_fuser.py:573-596 in the
+    reference), so that load and store are unit-stride along the kernel's n, and,
+    with the exchange switched off, through strided accesses.  Both against eager
+    fp32, and against each other."""
+    mod, inputs = W.column_major_store(batched)
+    monkeypatch.setattr(EVTFuser, "allow_transpose", swap)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    assert node.target.transposed == swap
+    dev = [t.cuda() for t in inputs]
+    outs = [o.clone() for o in gm(*dev)]
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    assert len(outs) == len(refs) == 2
+    for o, r in zip(outs, refs):
+        assert tuple(o.shape) == tuple(r.shape)
+        assert evt_oracle.max_rel_err(o, r) <= FP16_TOL
+    if swap:
+        monkeypatch.setattr(EVTFuser, "allow_transpose", False)
+        other = W.fuse(mod, inputs)(*dev)
+        torch.cuda.synchronize()
+        assert evt_oracle.max_rel_err(outs[0], other[0].float().cpu()) <= FP16_TOL
+        assert evt_oracle.max_rel_err(outs[1], other[1].float().cpu()) <= FP16_TOL
+
+
 @pytest.mark.parametrize("phase2", ["in_kernel", "finalize_kernel", "many_partials"])
-@pytest.mark.parametrize("transposed", [False, True], ids=["per_column", "per_row"])
-def test_bias_gradient_behind_a_head_merge(transposed, phase2, monkeypatch):
+@pytest.mark.parametrize("transposed, swap", [(False, True), (True, False), (True, True)],
+                         ids=["per_column", "per_row", "operands_exchanged"])
+def test_bias_gradient_behind_a_head_merge(transposed, swap, phase2, monkeypatch):
     """The backward pattern of an attention projection: batched product over
     B * H heads, result merged into [B * S, H * D] by the store, bias gradient
     = sum over all rows, i.e. per column (or, for the transposed product, per
-    row) and over the batches that agree modulo H.  Several row tiles and
-    several batches per result, combined by the last workgroup to arrive, by the
-    finalize kernel on request, and by the finalize kernel because there are
+    row; with the operands exchanged the transposed product is the per-column
+    problem again) and over the batches that agree modulo H.  Several row tiles
+    and several batches per result, combined by the last workgroup to arrive, by
+    the finalize kernel on request, and by the finalize kernel because there are
     more partials per result (24 batches x the row tiles) than a workgroup
     combines; repeated launches are bit-identical."""
+    monkeypatch.setattr(EVTFuser, "allow_transpose", swap)
     if phase2 == "finalize_kernel":
         monkeypatch.setenv("EVT_TWO_KERNEL_REDUCE", "1")
     many = phase2 == "many_partials"
@@ -762,8 +796,10 @@ def test_bias_gradient_behind_a_head_merge(transposed, phase2, monkeypatch):
     gm = W.fuse(mod, inputs)
     (node,) = fused_nodes(gm)
     (red,) = node.target.ir.reduces.values()
-    assert red.fold == "mod" and red.axis == ("row" if transposed else "col") and red.fold_count == (24 if many else 4)
-    if many and not transposed:
+    per_row = transposed and not swap
+    assert node.target.transposed == (transposed and swap)
+    assert red.fold == "mod" and red.axis == ("row" if per_row else "col") and red.fold_count == (24 if many else 4)
+    if many and not per_row:
         assert -(-node.target.problem[0] // node.target.tile.bm) * red.fold_count > 64
     dev = [t.cuda() for t in inputs]
     outs = [o.clone() for o in gm(*dev)]

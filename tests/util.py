@@ -23,6 +23,8 @@ def emulate_fused(op: FusedOpBase, *args):
         acc = Al @ Bl
     else:
         acc = op.anchor_eager(A, B)        # replays the operands' layout chains
+        if op.transposed:                  # the IR describes the epilogue of the transposed product
+            acc = acc.transpose(1, 2)
     loads = {}
     for k, slot in enumerate(op.ir.slots):
         kind, ref = op.slot_sources[k]
