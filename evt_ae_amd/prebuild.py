@@ -87,6 +87,9 @@ def register_all() -> List[jit.LazyModule]:
         for seed in W.RANDOM_EPILOGUE_SEEDS[:12 if anchor == "mm" else 6]:
             mod, ins = W.random_epilogue(seed, anchor)
             W.fuse(mod, _meta(ins))
+            if anchor in ("mm", "bmm") and seed < 6:
+                mod, ins = W.random_epilogue(seed, anchor, column_major=True)
+                W.fuse(mod, _meta(ins))
     for anchor, n, dt in W.ROW_LONG_CASES:
         mod, ins = W.row_edge_case(anchor, n, dt)
         W.fuse(mod, _meta(ins))

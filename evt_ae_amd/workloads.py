@@ -956,11 +956,14 @@ class RandomEpilogue(torch.nn.Module):
     UNARY = ("relu", "tanh", "sigmoid", "neg", "abs", "gelu", "exp_small", "sqrt_abs", "rsqrt_abs1")
     BINARY = ("add", "sub", "mul", "maximum", "minimum", "div_abs1", "where_gt")
 
-    def __init__(self, seed: int, anchor: str = "mm", n: int = 0):
+    def __init__(self, seed: int, anchor: str = "mm", n: int = 0, column_major: bool = False):
         super().__init__()
         import random
         rng = random.Random(0xE71 + seed + 1000 * ("mm", "bmm", "softmax", "layernorm").index(anchor))
         self.anchor, self.n = anchor, n
+        # the same-shape tensor is stored [N, M] and read through a permute, and the full-size results leave
+        # through permute + copy: every full-tensor access of the epilogue is column-major (products only)
+        self.column_major = column_major
         self.steps = []
         n_vals = 4                       # accum, aux, row, col
         # the first operand of every step comes from the accumulator's side (value 0 or an earlier step), so the
@@ -992,6 +995,9 @@ class RandomEpilogue(torch.nn.Module):
             acc = aten._softmax(A, -1, False)
         else:
             acc = operator.getitem(aten.native_layer_norm(A, [self.n], None, None, 1e-5), 0)
+        perm = [0, 2, 1] if self.anchor == "bmm" else [1, 0]
+        if self.column_major:
+            aux = aten.permute(aux, perm)
         vals = [acc, aux, row, col]
         for op, a, b in self.steps:
             x = vals[a]
@@ -1020,6 +1026,8 @@ class RandomEpilogue(torch.nn.Module):
         outs = [last]
         if self.extra is not None:
             outs.append(aten.add(vals[self.extra], aux))           # full size whatever the value's own shape
+        if self.column_major:
+            outs = [aten.clone(aten.permute(o, perm), memory_format=torch.contiguous_format) for o in outs]
         if self.reduce is not None:
             outs.append(aten.sum(aten.abs(last), [self.reduce + (1 if self.anchor == "bmm" else 0)], True))
         return tuple(outs)
@@ -1031,18 +1039,21 @@ RANDOM_EPILOGUE_SEEDS = tuple(range(12))
 RANDOM_EPILOGUE_ANCHORS = ("mm", "bmm", "softmax", "layernorm")
 
 
-def random_epilogue(seed: int, anchor: str = "mm", M: int = 320, N: int = 192, K: int = 96, L: int = 3):
+def random_epilogue(seed: int, anchor: str = "mm", M: int = 320, N: int = 192, K: int = 96, L: int = 3,
+                    column_major: bool = False):
     """(module, CPU inputs) of the seeded random epilogue behind `anchor`; M, N, K are no multiples of the
-    large tiles.  The row-wise anchors take A alone ([M, N]); B is an unused input there."""
+    large tiles.  The row-wise anchors take A alone ([M, N]); B is an unused input there.  `column_major`
+    (products only): see RandomEpilogue."""
     g = torch.Generator(device="cpu").manual_seed(0xE71 + seed)
     h = lambda *sh: (torch.randn(*sh, generator=g) * 0.5).half()   # noqa: E731
+    full = (N, M) if column_major else (M, N)
     if anchor == "mm":
-        ins = [h(M, K), h(K, N), h(M, N), h(N), h(M, 1)]
+        ins = [h(M, K), h(K, N), h(*full), h(N), h(M, 1)]
     elif anchor == "bmm":
-        ins = [h(L, M, K), h(L, K, N), h(L, M, N), h(N), h(M, 1)]
+        ins = [h(L, M, K), h(L, K, N), h(L, *full), h(N), h(M, 1)]
     else:
         ins = [h(M, N) * 4, h(1), h(M, N), h(N), h(M, 1)]
-    return RandomEpilogue(seed, anchor, N), ins
+    return RandomEpilogue(seed, anchor, N, column_major), ins
 
 
 class AffineLayerNorm(torch.nn.Module):

@@ -433,6 +433,24 @@ def test_column_major_outputs_are_computed_transposed(batched, monkeypatch):
             assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3
 
 
+@pytest.mark.parametrize("anchor", ["mm", "bmm"])
+def test_random_trees_with_column_major_tensors_lower_transposed(anchor):
+    """Seeded random epilogue trees whose full-size tensors are all stored [N, M]:
+    one fused kernel computing the transposed product, values from the IR
+    interpreter against eager fp32."""
+    for seed in W.RANDOM_EPILOGUE_SEEDS[:6]:
+        mod, inputs = W.random_epilogue(seed, anchor, column_major=True)
+        gm = W.fuse(mod, inputs)
+        (n,) = fused_nodes(gm)
+        assert n.target.transposed
+        got = run_emulated(gm, inputs)
+        ref = evt_oracle.eval_fp32(mod, inputs)
+        assert len(got) == len(ref)
+        for o, r in zip(got, ref):
+            assert tuple(o.shape) == tuple(r.shape)
+            assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3, (anchor, seed)
+
+
 def test_walk_tiles_are_offered_and_refused_where_they_should(monkeypatch):
     """Tiles whose workgroups walk over several tiles of a row block: offered by
     the tuner only where the tiles outnumber the CUs, K is a multiple of bk and

@@ -533,6 +533,34 @@ def test_random_epilogue_trees(anchor, seed):
             f"{anchor} seed {seed} output {k}: max rel err {err:.3e}"
 
 
+@pytest.mark.parametrize("seed", W.RANDOM_EPILOGUE_SEEDS[:6])
+@pytest.mark.parametrize("anchor", ["mm", "bmm"])
+def test_random_epilogue_trees_with_column_major_tensors(anchor, seed):
+    """The same random trees with every full-size tensor of the epilogue stored
+    [N, M]: the same-shape operand read through a permute, the results leaving
+    through permute + copy.  The fused op computes the transposed product (row
+    vector and column vector change roles, a sum along the rows becomes one over
+    them); one kernel, every output against the fp32 oracle."""
+    mod, inputs = W.random_epilogue(seed, anchor, column_major=True)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    assert node.target.transposed
+    left = [n for n in gm.graph.nodes if n.op == "call_function" and target_name(n.target) not in ("getitem", "view")
+            and n is not node]
+    assert not left, left
+    outs = gm(*[t.cuda() for t in inputs])
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    torch.cuda.synchronize()
+    refs = evt_oracle.eval_fp32(mod, inputs)
+    assert len(outs) == len(refs)
+    for k, (o, r) in enumerate(zip(outs, refs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        reduced = r.numel() < inputs[2].numel()
+        err = evt_oracle.max_rel_err(o, r)
+        assert err <= (REDUCTION_TOL if reduced and o.dtype == torch.float32 else FP16_TOL), \
+            f"{anchor} seed {seed} output {k}: max rel err {err:.3e}"
+
+
 @pytest.mark.parametrize("n", W.AFFINE_LN_LENGTHS)
 def test_layer_norm_with_weight_and_bias_on_long_rows(n):
     """native_layer_norm with weight and bias (moved into the epilogue by
