@@ -61,7 +61,8 @@ def _encoder_tuners(dims=None):
 SHORT_LIST = [(256, 256, 64, 4, 2, 2, 2), (256, 256, 64, 2, 4, 2, 3), (256, 256, 64, 2, 4, 2, 6), (256, 256, 64, 4, 2, 2, 0),
               (256, 128, 64, 4, 2, 3, 3), (256, 128, 64, 4, 2, 3, 10), (256, 128, 64, 4, 2, 3, 2),
               (128, 256, 64, 2, 4, 3, 3), (128, 256, 64, 2, 4, 3, 10), (128, 256, 64, 2, 4, 3, 2), (128, 128, 64, 2, 4, 4, 2),
-              (128, 128, 64, 4, 2, 2, 2), (128, 128, 64, 2, 4, 2, 3), (128, 128, 64, 2, 2, 2, 0), (64, 64, 64, 2, 2, 2, 0)]
+              (128, 128, 64, 4, 2, 2, 2), (128, 128, 64, 2, 4, 2, 3), (128, 128, 64, 2, 2, 2, 0), (64, 64, 64, 2, 2, 2, 0),
+              (128, 128, 64, 2, 2, 3, 12), (128, 128, 64, 2, 2, 4, 12)]
 
 
 def main():

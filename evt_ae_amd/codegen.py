@@ -32,7 +32,9 @@ class TileConfig:
     # 0: plain ring; 1: look-ahead ring with pinned instruction order (stages >= 3);
     # 2: ping-pong, the two waves of a SIMD alternate MFMA and LDS-read phases (8 waves, stages >= 2);
     # 3: ping-pong with one barrier per k-tile; 4 + flags: as 3 with 1 = the barrier inside group 0's MFMA phase,
-    # 2 = group 0 issues its transfers between its LDS reads, 4 = group 1 as well (stages >= 3)
+    # 2 = group 0 issues its transfers between its LDS reads, 4 = group 1 as well (stages >= 3);
+    # 12: one wave per SIMD (4 waves, stages >= 2): each wave interleaves the MFMAs of a k sub-step with the LDS
+    # reads of the next; 64 x 64 wave tiles on a 128 x 128 tile instead of the 64 x 32 of eight waves
     pipe: int = 0
     # > 1: a workgroup computes this many consecutive tiles of a row block, the operand ring running on from one
     # into the next, and per-row reductions leave one partial per workgroup (ping-pong pipelines, no per-column
@@ -674,6 +676,9 @@ class Codegen:
         e("};")
         b = lambda x: "true" if x else "false"  # noqa: E731
         tile_io = any((sl.role == "store" and sl.domain == "tile") or (sl.role == "load" and sl.kind == "aux") for sl in ir.slots)
+        if t.pipe == 12 and (t.wm * t.wn != 4 or not t.dma or t.stages < 2 or t.walk > 1):
+            raise NotImplementedError("the one-wave-per-SIMD loop needs four waves, the 16-byte transfers, two or more "
+                                      "stages and one tile per workgroup")
         if t.walk > 1 and (t.pipe < 2 or not t.dma or ir.col_state or not sp.k_exact):
             raise NotImplementedError("a walk over tiles needs a ping-pong pipeline, K a multiple of bk and an epilogue "
                                       "without per-column reduction")

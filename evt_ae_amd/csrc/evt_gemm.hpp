@@ -108,8 +108,13 @@ struct GemmCfg {
   //            of its read phase instead of between its MFMAs (with two stages:
   //            instead of in one burst in front of the reads);
   //         4  group 1 does the same (STAGES >= 3).
+  // PIPE 12: one wave per SIMD (4 waves, STAGES >= 2): each wave alternates MFMAs on the fragments of one k
+  //         sub-step with the LDS reads of the next, its transfers spread between them; one barrier per
+  //         k-tile.  A 128 x 256 tile then has 64 x 128 wave tiles, a quarter less LDS read traffic per MFMA
+  //         than the 64 x 64 wave tiles of eight waves.
   static constexpr int PIPE = PIPE_;
-  static constexpr bool PINGPONG = PIPE_ >= 2;
+  static constexpr bool SOLO = PIPE_ == 12;
+  static constexpr bool PINGPONG = PIPE_ >= 2 && !SOLO;
   static constexpr bool WALK = WALK_;
   // K is a multiple of BK in every launch (the host refuses others): see Operand
   static constexpr bool K_EXACT = K_EXACT_;
@@ -144,7 +149,8 @@ struct GemmCfg {
   static_assert(STAGES >= 1 && STAGES <= 8, "1..8 stages");
   static_assert(PIPE != 1 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
   static_assert(!PINGPONG || (DMA && STAGES >= 2 && WM * WN == 8), "ping-pong needs DMA, >= 2 stages, 8 waves");
-  static_assert(PIPE >= 0 && PIPE <= 11, "unknown pipeline");
+  static_assert(PIPE >= 0 && PIPE <= 12, "unknown pipeline");
+  static_assert(!SOLO || (DMA && STAGES >= 2 && WM * WN == 4 && (BK / 16) % 2 == 0), "one wave per SIMD: DMA, >= 2 stages, 4 waves");
   static_assert(!WALK || PINGPONG, "walking over tiles is built into the ping-pong loops");
   static_assert(!(PP_FLAGS & 4) || STAGES >= 3, "group 1 can only issue in its read phase with three or more stages");
 };
@@ -395,6 +401,40 @@ struct FragReader {
   EVT_DEV void issue(uint32_t lds, Tile& t) const {
 #pragma unroll
     for (int i = 0; i < NREADS; ++i) issue_one(lds, t, i);
+  }
+  // The fragments of one k sub-step (one wave per SIMD pipeline): issue_sub() for every i < SUB_READS, then
+  // lds_wait_all(), pin_sub(), frag_sub().
+  struct Sub {
+    u32x4 q[LDS_KC ? NFRAG : 1];
+    u32x2 h[LDS_KC ? 1 : 2 * NFRAG];
+  };
+  static constexpr int SUB_READS = LDS_KC ? NFRAG : 2 * NFRAG;
+  EVT_DEV void issue_sub(uint32_t lds, Sub& t, int ks, int i) const {
+    if constexpr (LDS_KC) {
+      t.q[i] = lds_read_b128(lds + off[ks] + i * (32 * CH * 16));
+    } else {
+      const int f = i >> 1;
+      t.h[i] = lds_read_tr16_b64(lds + off[f] + ks * (16 * RC * 16) + (i & 1) * (4 * RC * 16));
+    }
+  }
+  EVT_DEV void pin_sub(Sub& t) const {
+    if constexpr (LDS_KC) {
+#pragma unroll
+      for (int i = 0; i < NFRAG; ++i) lds_pin(t.q[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2 * NFRAG; ++i) lds_pin(t.h[i]);
+    }
+  }
+  EVT_DEV u32x4 frag_sub(const Sub& t, int f) const {
+    if constexpr (LDS_KC) {
+      return t.q[f];
+    } else {
+      const u32x2 lo = t.h[2 * f], hi = t.h[2 * f + 1];
+      u32x4 r;
+      r.x = lo.x; r.y = lo.y; r.z = hi.x; r.w = hi.y;
+      return r;
+    }
   }
   EVT_DEV void pin(Tile& t) const {
     if constexpr (LDS_KC) {
@@ -869,6 +909,102 @@ struct Mainloop {
     }
   }
 
+  // ---- one wave per SIMD (PIPE 12) ------------------------------------------
+  // Four waves, each alone on its SIMD, so nothing else fills the matrix pipe while a wave reads: every wave
+  // works through the k sub-steps (16 wide) of a k-tile with two fragment sets, issuing after each MFMA of
+  // sub-step s its share of the LDS reads of sub-step s+1 (of the next k-tile behind the last one) and of the
+  // transfers of k-tile T+STAGES-1 into the stage tile T-1 occupied.  The order is pinned instruction by
+  // instruction; the reads are waited for once per sub-step, a whole sub-step of MFMAs after they were issued.
+  // One barrier per k-tile, in front of the first reads of the next: tile T+1 has landed for every wave, and
+  // every wave has the last fragments of tile T in registers, so its stage may be refilled from then on.
+  struct SubFrags {
+    typename RdA::Sub a;
+    typename RdB::Sub b;
+  };
+  static constexpr int SO_NR = RdA::SUB_READS + RdB::SUB_READS;   // LDS reads per sub-step
+  static constexpr int SO_NM = Cfg::MI * Cfg::NI;                 // MFMAs per sub-step
+  static EVT_DEV void so_read_all(SubFrags& f, const char* lds, const RdA& ra, const RdB& rb, int ks) {
+    const uint32_t la = lds_addr(lds), lb = lds_addr(lds + Cfg::A_BYTES);
+#pragma unroll
+    for (int i = 0; i < RdA::SUB_READS; ++i) ra.issue_sub(la, f.a, ks, i);
+#pragma unroll
+    for (int i = 0; i < RdB::SUB_READS; ++i) rb.issue_sub(lb, f.b, ks, i);
+  }
+  static EVT_DEV void run_solo(const OpA& a, const OpB& b, const RdA& ra, const RdB& rb, char* smem,
+                               int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+    constexpr int S = Cfg::STAGES, KS = Cfg::KS;
+    static_assert((S - 1) * LPS < 64, "vmcnt is a 6-bit counter");
+    // transfers past the last k-tile read as zeros (or are switched off lane by lane) and land in stages nobody
+    // reads any more: the vmcnt bookkeeping stays uniform
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+      a.dma(s, smem + s * Cfg::STAGE_BYTES, wave);
+      b.dma(s, smem + s * Cfg::STAGE_BYTES + Cfg::A_BYTES, wave);
+    }
+    wait_tiles<S - 2>();   // my share of tile 0 has landed
+    pp_barrier();
+    SubFrags f[2];
+    so_read_all(f[0], smem, ra, rb, 0);
+    int stage = 0;
+    for (int T = 0; T < KT; ++T) {
+      const int nstage = stage + 1 == S ? 0 : stage + 1;
+      const char* cur = smem + stage * Cfg::STAGE_BYTES;
+      const char* nxt = smem + nstage * Cfg::STAGE_BYTES;
+      char* ds = pp_refill_stage(stage, smem);
+      const typename OpA::DmaTile da = a.dma_begin(T + S - 1);
+      const typename OpB::DmaTile db = b.dma_begin(T + S - 1);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        SubFrags& now = f[ks & 1];
+        SubFrags& next = f[(ks + 1) & 1];
+        lds_wait_all();            // the fragments of this sub-step, issued a sub-step ago
+        ra.pin_sub(now.a);
+        rb.pin_sub(now.b);
+        const bool last = ks == KS - 1;
+        const uint32_t la = lds_addr(last ? nxt : cur), lb = la + Cfg::A_BYTES;
+        const int nks = last ? 0 : ks + 1;
+        // Slots: the reads of the next sub-step go out behind the first MFMAs (SO_RD of them), so that they are
+        // back long before the sub-step ends; the transfers behind the others.  In the last sub-step of a k-tile
+        // the barrier stands behind the first SO_BAR MFMAs -- the matrix pipe has work while it resolves -- and
+        // the reads, which are of the next k-tile, follow it.
+        constexpr int SO_RD = SO_NM >= 4 ? SO_NM / 2 : SO_NM, SO_BAR = SO_NM >= 4 ? 2 : 1;
+        constexpr int PER = (LPS + KS - 2) / (KS - 1);           // transfers per sub-step
+#pragma unroll
+        for (int m = 0; m < SO_NM; ++m) {
+          const int mi = m / Cfg::NI, ni = m % Cfg::NI;
+          acc[mi][ni] = mfma32<Cfg::BF16>(ra.frag_sub(now.a, mi), rb.frag_sub(now.b, ni), acc[mi][ni]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (last && m == SO_BAR - 1) {
+            wait_tiles<S - 2>();     // my share of tile T+1 has landed
+            pp_barrier();            // everybody's has; everybody holds the last fragments of tile T
+          }
+          const int r0 = last ? SO_BAR - 1 : 0;                  // first slot with reads
+#pragma unroll
+          for (int i = 0; i < SO_NR; ++i) {
+            if (r0 + (i * SO_RD) / SO_NR == m) {
+              if (i < RdA::SUB_READS) ra.issue_sub(la, next.a, nks, i);
+              else rb.issue_sub(lb, next.b, nks, i - RdA::SUB_READS);
+            }
+          }
+          if (!last) {             // the transfers go out during the first KS-1 sub-steps, behind the barrier of tile T-1
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+              const int c = ks * PER + j;
+              if (c < LPS && SO_RD % SO_NM + (j * (SO_NM - SO_RD % SO_NM)) / PER == m) {
+                if (c < OpA::NLOAD) a.dma_chunk(da, ds, wave, c);
+                else b.dma_chunk(db, ds + Cfg::A_BYTES, wave, c - OpA::NLOAD);
+              }
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      stage = nstage;
+    }
+    lds_wait_all();                // the reads issued behind the last tile (nobody uses them)
+    wait_vmcnt<0>();               // the transfers past the last tile have landed
+  }
+
   static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, int split, char* smem,
                           f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
     Walk wk;
@@ -917,6 +1053,8 @@ struct Mainloop {
 
     if constexpr (Cfg::PIPE == 1) {
       run_lookahead(a, b, ra, rb, smem, wave, KT, acc);
+    } else if constexpr (Cfg::SOLO) {
+      run_solo(a, b, ra, rb, smem, wave, KT, acc);
     } else if constexpr (Cfg::PINGPONG) {
       run_pingpong(a, b, ra, rb, smem, wave, KT, acc, wk, more,
                    Cfg::B_KC ? (int64_t)Cfg::BN * g.ldb * 2 : (int64_t)Cfg::BN * 2, tid);

@@ -211,7 +211,8 @@ NO_ALLOC_TOO_BIG = (5, dict(M=1024, N=131072, K=64), (256, 256, 64, 4, 2, 2, Tru
 
 def pipeline_tiles():
     """Ping-pong main-loop variants (pipe 2: two barriers per k-tile, pipe 3:
-    one) on every stage count / k-depth / wave grid they are instantiated with."""
+    one) and the one-wave-per-SIMD loop (pipe 12) on every stage count / k-depth /
+    wave grid they are instantiated with."""
     from .codegen import TileConfig
     return [TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 2),
             TileConfig(256, 256, 32, 2, 4, 4, True, 4, 2), TileConfig(256, 128, 64, 4, 2, 3, True, 4, 3),
@@ -219,7 +220,10 @@ def pipeline_tiles():
             # options of the one-barrier loop: transfers issued among the LDS reads (both groups), barrier inside
             # group 0's MFMA phase
             TileConfig(128, 256, 64, 2, 4, 3, True, 4, 10), TileConfig(256, 128, 64, 4, 2, 3, True, 4, 11),
-            TileConfig(256, 256, 64, 2, 4, 2, True, 4, 7)]
+            TileConfig(256, 256, 64, 2, 4, 2, True, 4, 7),
+            # one wave per SIMD: three and four stages, square and oblong wave tiles, two stages
+            TileConfig(128, 128, 64, 2, 2, 3, True, 4, 12), TileConfig(128, 128, 64, 2, 2, 4, True, 4, 12),
+            TileConfig(256, 128, 64, 2, 2, 3, True, 4, 12), TileConfig(128, 256, 64, 2, 2, 2, True, 4, 12)]
 
 
 # Workgroups that walk over several tiles of a row block (TileConfig.walk): (config, shapes, tile).  K is a

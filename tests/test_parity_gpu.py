@@ -62,8 +62,9 @@ def test_configs_against_oracle(cfg, shapes):
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
 @pytest.mark.parametrize("tile", W.pipeline_tiles(), ids=lambda t: t.tag())
 def test_pipeline_variants_against_oracle(cfg, tile):
-    """Every ping-pong main-loop variant on shapes with several tiles in M, N and
-    K, partial edge tiles and a K tail (one k-tile only for the batched config)."""
+    """Every ping-pong main-loop variant and the one-wave-per-SIMD loop on shapes
+    with several tiles in M, N and K, partial edge tiles and a K tail (one k-tile
+    only for the batched config)."""
     wl, inputs, gm, outs = _run(cfg, W.PIPELINE_SHAPES[cfg], tile=tile)
     _compare(wl, outs, evt_oracle.eval_fp32(wl.module(), inputs))
 
