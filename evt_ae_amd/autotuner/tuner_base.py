@@ -181,14 +181,17 @@ class AutoTunerBase:
         eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3}
         best, best_cost = None, None
         for t in self.candidates():
-            if t.pipe not in (0, 2) or t.stages == 1 or t.walk > 1:
-                continue    # untuned default: a ping-pong tile or the plain double-buffered ring
             tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
+            # untuned default: a ping-pong tile or the plain double-buffered ring, or, for one round of 128 x 128
+            # tiles with a CU each, the one-wave-per-SIMD loop (measured 8-19 % faster there than eight waves)
+            solo = t.pipe == 12 and (t.bm, t.bn, t.stages) == (128, 128, 3) and tiles <= NUM_CUS and self.K >= 4 * t.bk
+            if (t.pipe not in (0, 2) and not solo) or t.stages == 1 or t.walk > 1:
+                continue
             wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 else 1
             if tiles <= NUM_CUS:
                 wg_per_cu = 1       # one workgroup per CU at most: nothing shares a CU's throughput
             rounds = -(-tiles // (NUM_CUS * wg_per_cu))
-            cost = rounds * wg_per_cu * t.bm * t.bn / (eff.get((t.bm, t.bn), 0.5) * (1.15 if t.pipe == 2 else 1.0))
+            cost = rounds * wg_per_cu * t.bm * t.bn / (eff.get((t.bm, t.bn), 0.5) * (1.3 if solo else 1.15 if t.pipe == 2 else 1.0))
             # few tiles, a long K and a small output: the kernel splits K over several workgroups per tile (the
             # rule of the generated host code); the exchange of partial tiles eats about half of the gain, and
             # more than four splits are not rewarded here
