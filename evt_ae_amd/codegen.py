@@ -1297,7 +1297,7 @@ class RowCodegen(Codegen):
         e("  else hipLaunchKernelGGL((evt::evt_row_kernel<Cfg, Epi, 0>), dim3(grid), dim3(Cfg::THREADS), 0, (hipStream_t)stream, g, p);")
         e("  int err = (int)hipGetLastError();")
         e("  if (err != 0 || Epi::COL_STATE == 0) return err;")
-        e("  hipLaunchKernelGGL((evt::evt_row_col_finalize_kernel<Epi>), dim3((g.N + 63) / 64), dim3(1024), 0, (hipStream_t)stream, g, p, (int)grid);")
+        e("  hipLaunchKernelGGL((evt::evt_row_col_finalize_kernel<Epi>), dim3((g.N + evt::kColFinalizeCols - 1) / evt::kColFinalizeCols), dim3(1024), 0, (hipStream_t)stream, g, p, (int)grid);")
         e("  return (int)hipGetLastError();")
         e("}")
         return e.text()
