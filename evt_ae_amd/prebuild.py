@@ -118,8 +118,12 @@ def register_all() -> List[jit.LazyModule]:
     from .passes import pass_decomposition, pass_fusion
     W.fuse(W.Dropout1Undecomposed(), _meta(W.pattern_inputs("dropout1")), passes=[pass_decomposition, pass_fusion])
     from .autotuner.tuner_base import force_tile
+    from .codegen import TileConfig
     for cfg, shapes in W.SPLIT_K_SHAPES.items():
         W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
+        for tile in W.SPLIT_K_TILES:
+            with force_tile(TileConfig(*tile)):
+                W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
     for tile in W.pipeline_tiles():
         with force_tile(tile):
             for cfg in W.CONFIGS:

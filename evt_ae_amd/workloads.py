@@ -177,6 +177,10 @@ SPLIT_K_SHAPES = {
     5: dict(M=72, N=1032, K=2056),
 }
 
+# tiles the split-K shapes are also run with (besides the tuner's own choice): a ping-pong loop and the
+# one-wave-per-SIMD loop, (bm, bn, bk, wm, wn, stages, dma, group_m, pipe)
+SPLIT_K_TILES = ((128, 256, 64, 2, 4, 3, True, 4, 10), (128, 128, 64, 2, 2, 3, True, 4, 12))
+
 PIPELINE_SHAPES = {
     1: dict(M=300, N=264, K=200),
     2: dict(L=2, S=200, D=72),

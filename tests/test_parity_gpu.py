@@ -13,6 +13,7 @@ import torch
 
 from evt_ae_amd import workloads as W
 from evt_ae_amd.autotuner.tuner_base import force_tile
+from evt_ae_amd.codegen import TileConfig
 from evt_ae_amd.evt_fuser import EVTFuser
 from oracle import evt_oracle
 from evt_ae_amd.passes import target_name
@@ -623,20 +624,27 @@ def test_aot_encoder_layer_training_step(fused_qkv):
         assert err <= max(2e-2, 2.0 * err_eager), f"{name}: norm-wise error {err:.3e} (eager fp16: {err_eager:.3e})"
 
 
+@pytest.mark.parametrize("tile", [None, *W.SPLIT_K_TILES], ids=lambda t: "tuner" if t is None else TileConfig(*t).tag())
 @pytest.mark.parametrize("cfg", list(W.SPLIT_K_SHAPES))
-def test_split_k(cfg, monkeypatch):
+def test_split_k(cfg, tile, monkeypatch):
     """Few output tiles and a long K: several workgroups share a tile, leave their
     accumulators in the workspace and the last to arrive adds them in split order
     and runs the epilogue (with its own per-row / per-column reductions).  Checked
     against the oracle with the automatic split, with a forced odd split and with
     splitting off; repeated launches are bit-identical (the order of the sum is
-    fixed), and the automatic choice really splits."""
+    fixed), and the automatic choice really splits.  With the tuner's tile, a
+    ping-pong tile and a one-wave-per-SIMD tile."""
     shapes = W.SPLIT_K_SHAPES[cfg]
     wl = W.CONFIGS[cfg]
     inputs = W.make_inputs(cfg, shapes)
     refs = evt_oracle.eval_fp32(wl.module(), inputs)
     dev = [t.cuda() for t in inputs]
-    gm = W.fuse(wl.module(), inputs)
+    if tile is None:
+        gm = W.fuse(wl.module(), inputs)
+    else:
+        with force_tile(TileConfig(*tile)):
+            gm = W.fuse(wl.module(), inputs)
+        assert fused_nodes(gm)[0].target.tile == TileConfig(*tile)
     (node,) = fused_nodes(gm)
     op = node.target
     results = {}
