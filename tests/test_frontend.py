@@ -451,6 +451,32 @@ def test_random_trees_with_column_major_tensors_lower_transposed(anchor):
             assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3, (anchor, seed)
 
 
+def test_column_major_output_beside_a_column_index_stays_untransposed():
+    """A column index in the epilogue (here a gather along the row) has no
+    counterpart in the transposed problem, where columns are rows: the
+    column-major store is then kept as a strided store, and the values still
+    agree with eager fp32."""
+    aten = torch.ops.aten
+
+    class StoreAndGather(torch.nn.Module):
+        def forward(self, a, b, labels):
+            out = aten.mm(a, b)
+            t = aten.clone(aten.permute(aten.mul(out, 0.5), [1, 0]), memory_format=torch.contiguous_format)
+            return t, aten.gather(out, 1, aten.unsqueeze(labels, 1))
+
+    g = torch.Generator().manual_seed(3)
+    inputs = [(torch.randn(72, 40, generator=g) * 0.5).half(), (torch.randn(40, 56, generator=g) * 0.5).half(),
+              torch.randint(0, 56, (72,), generator=g)]
+    gm = W.fuse(StoreAndGather(), inputs)
+    (n,) = fused_nodes(gm)
+    assert not n.target.transposed and n.target.problem[:2] == (72, 56)
+    (st,) = [s.strides for s in n.target.ir.slots if s.role == "store" and s.domain == "tile"]
+    assert (st.stride_m, st.stride_n) == (1, 72)
+    for o, r in zip(run_emulated(gm, inputs), evt_oracle.eval_fp32(StoreAndGather(), inputs)):
+        assert tuple(o.shape) == tuple(r.shape)
+        assert evt_oracle.max_rel_err(o.float(), r) <= 5e-3
+
+
 def test_walk_tiles_are_offered_and_refused_where_they_should(monkeypatch):
     """Tiles whose workgroups walk over several tiles of a row block: offered by
     the tuner only where the tiles outnumber the CUs, K is a multiple of bk and
