@@ -161,6 +161,26 @@ def test_tuner_cache_round_trip(tmp_path, monkeypatch):
     assert tuner.get_best_config() == t
 
 
+def test_untuned_problems_get_a_modelled_tile(monkeypatch):
+    """Without a cache row the tuner models its choice: 256 x 256 ping-pong tiles
+    when they fill the chip, the one-wave-per-SIMD loop for one round of 128 x 128
+    tiles over a K of at least four k-tiles, and every choice is a tile the
+    epilogue fits."""
+    from evt_ae_amd.autotuner.gemm_tuner import MMTuner
+    monkeypatch.setenv("EVT_TUNER_CACHE", "/nonexistent/tuner_cache.db")
+    inputs = W.make_inputs(1, W.GOLDEN_SHAPES[1])
+    (n,) = fused_nodes(W.fuse(W.CONFIGS[1].module(), [t.to("meta") for t in inputs]))
+    picks = {}
+    for problem in ((8192, 8192, 1024, 1), (4096, 1024, 2048, 1), (2048, 2048, 2048, 1), (4096, 1024, 128, 1)):
+        tuner = MMTuner(problem, True, True, False, True, n.target.ir)
+        picks[problem] = t = tuner.heuristic()
+        assert tuner.fits(t) and t in tuner.candidates()
+    big, solo_a, solo_b, short_k = picks.values()
+    assert (big.bm, big.bn, big.pipe) == (256, 256, 2)
+    assert (solo_a.bm, solo_a.bn, solo_a.wm * solo_a.wn, solo_a.pipe) == (128, 128, 4, 12) and solo_a == solo_b
+    assert short_k.pipe != 12       # two k-tiles do not fill a three-stage ring
+
+
 def test_shipped_tuner_cache_is_read():
     """Every row of the shipped tile cache parses into a TileConfig of this
     version and is what tracing the headline workloads selects."""
