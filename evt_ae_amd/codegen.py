@@ -750,9 +750,11 @@ class Codegen:
             e("  int s = 1;")
             e("  if (want > 1) s = want < kt ? want : kt;")
             e("  // automatic: only small outputs -- every split writes and the last arriver reads a whole fp32 tile, which")
-            e("  // costs more than the idle CUs once the output runs to megabytes")
+            e("  // costs more than the idle CUs once the output runs to megabytes; at most 4 Mi elements over all splits")
+            e("  // (1024 x 1024 x 4096 measured 22 us with 4 splits, 40 us with 8, 30 us unsplit)")
             e("  else if (want == 0 && tiles * 2 <= cus && kt >= 8 && (int64_t)a->M * a->N * a->L <= (1 << 20)) "
-              "{ s = (int)(cus / tiles); if (s > 8) s = 8; if (s > kt / 4) s = kt / 4; }")
+              "{ s = (int)(cus / tiles); if (s > 8) s = 8; if (s > kt / 4) s = kt / 4;"
+              " const int64_t cap = (4 << 20) / ((int64_t)a->M * a->N * a->L); if (s > cap) s = cap < 1 ? 1 : (int)cap; }")
             e("  if (s >= 2) {")
             e("    const int chunk = (kt + s - 1) / s;")
             e("    g.splits = (kt + chunk - 1) / chunk;      // every split has work")
