@@ -79,8 +79,9 @@ def register_all() -> List[jit.LazyModule]:
                 mod, ins = W.head_merge_bias_grad(transposed=transposed, **W.HEAD_MERGE_MANY_PARTIALS)
                 W.fuse(mod, _meta(ins))
             for batched in (False, True):
-                mod, ins = W.column_major_store(batched)
-                W.fuse(mod, _meta(ins))
+                for dtype in (torch.float16, torch.bfloat16):
+                    mod, ins = W.column_major_store(batched, dtype=dtype)
+                    W.fuse(mod, _meta(ins))
         finally:
             EVTFuser.allow_transpose = True
     for anchor in W.RANDOM_EPILOGUE_ANCHORS:

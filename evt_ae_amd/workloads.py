@@ -947,9 +947,9 @@ class ColumnMajorStore(torch.nn.Module):
         return yt, red
 
 
-def column_major_store(batched: bool, seed: int = 0):
+def column_major_store(batched: bool, seed: int = 0, dtype=torch.float16):
     g = torch.Generator(device="cpu").manual_seed(0xC01A + seed)
-    h = lambda *sh: (torch.randn(*sh, generator=g) * 0.3).half()   # noqa: E731
+    h = lambda *sh: (torch.randn(*sh, generator=g) * 0.3).to(dtype)   # noqa: E731
     lead, (M, N, K) = ((3,), (200, 136, 64)) if batched else ((), (320, 192, 96))
     return ColumnMajorStore(batched), [h(*lead, M, K), h(*lead, K, N), h(N), h(*lead, N, M)]
 

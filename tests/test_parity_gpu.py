@@ -782,20 +782,22 @@ def test_bench_argument_sets_are_independent():
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
 @pytest.mark.parametrize("swap", [True, False], ids=["operands_exchanged", "strided_store"])
 @pytest.mark.parametrize("batched", [False, True], ids=["mm", "bmm"])
-def test_column_major_outputs(batched, swap, monkeypatch):
+def test_column_major_outputs(batched, swap, dtype, monkeypatch):
     """gelu(a @ b + bias + r^T) stored as [N, M], with the sum over all rows (GEMM)
     or the maximum along every row (batched product) of the stored values: computed
     as C^T = B^T A^T with the operands exchanged (evt_fuser.py:573-596 in the
     reference), so that load and store are unit-stride along the kernel's n, and,
     with the exchange switched off, through strided accesses.  Both against eager
     fp32, and against each other."""
-    mod, inputs = W.column_major_store(batched)
+    mod, inputs = W.column_major_store(batched, dtype=dtype)
+    tol = FP16_TOL      # 2e-2: wide enough for bf16's 8 mantissa bits as well
     monkeypatch.setattr(EVTFuser, "allow_transpose", swap)
     gm = W.fuse(mod, inputs)
     (node,) = fused_nodes(gm)
-    assert node.target.transposed == swap
+    assert node.target.transposed == swap and node.target.spec.bf16 == (dtype == torch.bfloat16)
     dev = [t.cuda() for t in inputs]
     outs = [o.clone() for o in gm(*dev)]
     torch.cuda.synchronize()
@@ -803,13 +805,13 @@ def test_column_major_outputs(batched, swap, monkeypatch):
     assert len(outs) == len(refs) == 2
     for o, r in zip(outs, refs):
         assert tuple(o.shape) == tuple(r.shape)
-        assert evt_oracle.max_rel_err(o, r) <= FP16_TOL
+        assert evt_oracle.max_rel_err(o, r) <= tol
     if swap:
         monkeypatch.setattr(EVTFuser, "allow_transpose", False)
         other = W.fuse(mod, inputs)(*dev)
         torch.cuda.synchronize()
-        assert evt_oracle.max_rel_err(outs[0], other[0].float().cpu()) <= FP16_TOL
-        assert evt_oracle.max_rel_err(outs[1], other[1].float().cpu()) <= FP16_TOL
+        assert evt_oracle.max_rel_err(outs[0], other[0].float().cpu()) <= tol
+        assert evt_oracle.max_rel_err(outs[1], other[1].float().cpu()) <= tol
 
 
 @pytest.mark.parametrize("phase2", ["in_kernel", "finalize_kernel", "many_partials"])
