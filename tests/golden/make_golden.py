@@ -1,5 +1,5 @@
 """Writes tests/golden/configs_small.npz: seeded inputs of the five headline
-subgraphs at the fixture shapes (workloads.GOLDEN_SHAPES) and the outputs of PyTorch's fp32 eager
+subgraphs at the fixture shapes (patterns.GOLDEN_SHAPES) and the outputs of PyTorch's fp32 eager
 evaluation of each subgraph on CPU (the specified oracle for this path; the
 reference itself ships no numeric vectors and cannot run here because its
 CUTLASS dependency is an empty submodule).
@@ -14,7 +14,7 @@ import numpy as np
 ROOT = Path(__file__).resolve().parents[2]
 sys.path.insert(0, str(ROOT))
 
-from evt_ae_amd import workloads as W   # noqa: E402
+from tests import patterns as W   # noqa: E402
 from oracle import evt_oracle           # noqa: E402
 
 

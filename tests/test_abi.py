@@ -9,7 +9,8 @@ from pathlib import Path
 import pytest
 import torch
 
-from evt_ae_amd import jit, workloads as W
+from evt_ae_amd import jit
+from tests import patterns as W
 from tests.util import fused_nodes
 
 ROOT = Path(__file__).resolve().parent.parent

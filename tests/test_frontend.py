@@ -7,7 +7,7 @@ import operator
 import pytest
 import torch
 
-from evt_ae_amd import workloads as W
+from tests import patterns as W
 from evt_ae_amd.evt_fuser import EVTFuser, FusedBMM, FusedGEMM, target_name
 from oracle import evt_oracle
 from tests.util import fused_nodes, rand_slot, run_emulated

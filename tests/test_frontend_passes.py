@@ -12,7 +12,7 @@ import pytest
 import torch
 from torch.fx import symbolic_trace
 
-from evt_ae_amd import workloads as W
+from tests import patterns as W
 from evt_ae_amd.aot_helper import aot_capture, joint_optimization
 from evt_ae_amd.evt_fuser import legalize_graph, target_name
 from evt_ae_amd.passes import (GTLFrontend, pass_clean_up, pass_cse, pass_decomposition, pass_loss_elimination)

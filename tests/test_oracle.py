@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from evt_ae_amd import workloads as W
+from tests import patterns as W
 from oracle import evt_oracle as O
 
 aten = torch.ops.aten

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from evt_ae_amd import workloads as W
+from tests import patterns as W
 from evt_ae_amd.autotuner.tuner_base import force_tile
 from evt_ae_amd.codegen import TileConfig
 from evt_ae_amd.evt_fuser import EVTFuser

@@ -15,7 +15,7 @@ import pytest
 import torch
 from torch.fx.passes.tools_common import legalize_graph
 
-from evt_ae_amd import workloads as W
+from tests import patterns as W
 from evt_ae_amd.evt_fuser import EVTFuser, packet, target_name
 from evt_ae_amd.partitioner import AnchorPartitionILP, PartitionCache, _volume_bits
 from evt_ae_amd.passes import Partitioning, _fusible, internal_volume_bits

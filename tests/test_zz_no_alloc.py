@@ -9,7 +9,8 @@ import ctypes
 import pytest
 import torch
 
-from evt_ae_amd import jit, workloads as W
+from evt_ae_amd import jit
+from tests import patterns as W
 from evt_ae_amd.autotuner.tuner_base import force_tile
 from evt_ae_amd.codegen import STATIC_SCRATCH_BYTES, TileConfig
 from evt_ae_amd.workloads import fused_nodes
