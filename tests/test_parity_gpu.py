@@ -782,6 +782,36 @@ def test_bench_argument_sets_are_independent():
             assert torch.equal(a, b)
 
 
+def test_tuning_at_trace_time(tmp_path, monkeypatch):
+    """EVT_AUTOTUNE=1 with an empty cache: tracing times the candidate tiles on
+    the device (here two of them, both built ahead of time), stores the faster
+    with its time under the problem's key, and the next trace reads that row;
+    the tuned op still agrees with the oracle."""
+    import sqlite3
+    from evt_ae_amd.autotuner.gemm_tuner import MMTuner
+    cache = tmp_path / "tuner_cache.db"
+    monkeypatch.setenv("EVT_TUNER_CACHE", str(cache))
+    monkeypatch.setenv("EVT_AUTOTUNE", "1")
+    tiles = [t for t in W.pipeline_tiles() if (t.bm, t.bn, t.stages, t.pipe) in ((256, 256, 2, 2), (128, 128, 3, 12))]
+    assert len(tiles) == 2
+    monkeypatch.setattr(MMTuner, "candidates", lambda self: list(tiles))
+    monkeypatch.setattr(MMTuner, "warmup_iterations", 3)
+    monkeypatch.setattr(MMTuner, "profile_iterations", 10)
+    wl, inputs, gm, outs = _run(3, W.PIPELINE_SHAPES[3])
+    op = fused_nodes(gm)[0].target
+    assert op.tile in tiles
+    con = sqlite3.connect(str(cache))
+    rows = con.execute("SELECT key, us FROM best_config_mm").fetchall()
+    con.close()
+    assert len(rows) == 1 and rows[0][0].startswith("264_520_328_f16_f16_") and 0 < rows[0][1] < 1e4
+    _compare(wl, outs, evt_oracle.eval_fp32(wl.module(), inputs))
+    # the row is what an untuned trace now selects, without timing anything
+    monkeypatch.setenv("EVT_AUTOTUNE", "0")
+    monkeypatch.setattr(MMTuner, "profile", lambda self, tile: pytest.fail("timed a tile although a row exists"))
+    again = fused_nodes(W.fuse(wl.module(), inputs))[0].target
+    assert again.tile == op.tile
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
 @pytest.mark.parametrize("swap", [True, False], ids=["operands_exchanged", "strided_store"])
 @pytest.mark.parametrize("batched", [False, True], ids=["mm", "bmm"])
