@@ -85,30 +85,46 @@ def reduction_lds_bytes(t: "TileConfig", row_state: int, col_state: int) -> int:
     return max(need, t.wm * t.wn * 64 * row_state * 4)
 
 
-ABI_VERSION = 4            # EVT_ABI_VERSION of include/evt_amd.h
+ABI_VERSION = 5            # EVT_ABI_VERSION of include/evt_amd.h
 STATIC_SCRATCH_BYTES = 1 << 20
 
 
-def emit_static_scratch(e: "_Emitter") -> None:
+def emit_static_scratch(e: "_Emitter", needed: bool) -> None:
     """File-scope device array that takes the workspace's place in `evt_launch_static`, and the per-device
-    look-up of its address (each GPU that loads the module holds its own copy)."""
+    look-up of its address (each GPU that loads the module holds its own copy).  A module whose kernels never use
+    a workspace (`needed` false) carries no array."""
     e("// ---- evt_launch_static: the entry point that allocates nothing ------------------------------------------")
     e("namespace {")
+    if not needed:
+        e("constexpr int64_t kScratchBytes = 0;   // this module's kernels use no workspace: no array")
+        e("[[maybe_unused]] int scratch_for_stream(void* stream, void** out) { (void)stream; *out = nullptr; return EVT_OK; }")
+        e("}  // namespace")
+        return
     e(f"constexpr int64_t kScratchBytes = {STATIC_SCRATCH_BYTES};")
     e("static __device__ __align__(256) unsigned char scratch[kScratchBytes];")
     e("constexpr int kMaxDevices = 64;")
     e("void* scratch_address[kMaxDevices];   // device address of `scratch` on each GPU, looked up on first use")
     e("std::mutex scratch_mutex;")
-    e("// `scratch` names a host-side stand-in; kernels, fills and copies take the address this returns")
-    e("int scratch_on_current_device(void** out) {")
-    e("  int dev = -1;")
-    e("  const hipError_t e0 = hipGetDevice(&dev);")
+    e("// `scratch` names a host-side stand-in; kernels, fills and copies take the address this returns: the array's")
+    e("// address on the GPU that `stream` belongs to (the current one for the null stream).  The first call per GPU")
+    e("// looks the address up with that GPU current, which may load the code object: it has to happen outside a")
+    e("// stream capture.")
+    e("int scratch_for_stream(void* stream, void** out) {")
+    e("  int cur = -1, dev = -1;")
+    e("  const hipError_t e0 = hipGetDevice(&cur);")
     e("  if (e0 != hipSuccess) return (int)e0;")
+    e("  dev = cur;")
+    e("  if (stream) {")
+    e("    const hipError_t es = hipStreamGetDevice((hipStream_t)stream, &dev);")
+    e("    if (es != hipSuccess) return (int)es;")
+    e("  }")
     e("  if (dev < 0 || dev >= kMaxDevices) return EVT_ERR_RANGE;")
     e("  std::lock_guard<std::mutex> lock(scratch_mutex);")
     e("  if (!scratch_address[dev]) {")
     e("    void* ptr = nullptr;")
+    e("    if (dev != cur) { const hipError_t e2 = hipSetDevice(dev); if (e2 != hipSuccess) return (int)e2; }")
     e("    const hipError_t e1 = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));")
+    e("    if (dev != cur) (void)hipSetDevice(cur);")
     e("    if (e1 != hipSuccess) return (int)e1;")
     e("    if (!ptr) return EVT_ERR_WORKSPACE;")
     e("    scratch_address[dev] = ptr;")
@@ -631,7 +647,8 @@ class Codegen:
         return {
             "abi": ABI_VERSION,
             "name": self.name,
-            "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
+            # what evt_launch_static can hold in place of a workspace (0: these kernels never use one)
+            "static_scratch_bytes": STATIC_SCRATCH_BYTES if self.uses_workspace() else 0,
             "tile": asdict(t),
             "a_k_contiguous": self.spec.a_kc,
             "k_multiple_of": self.spec.tile.bk if self.spec.k_exact else 1,   # launches with another K are refused
@@ -646,6 +663,12 @@ class Codegen:
             # scalars[rng_scalars .. +3] = 32-bit patterns of (seed low, seed high, offset, stream id) for rand_like
             "rng_scalars": self.ir.rng_scalar,
         }
+
+    def uses_workspace(self) -> bool:
+        """Can a launch of this module need a workspace: cross-tile reductions, or split-K (rings of two or more
+        stages outside a walk)?"""
+        t = self.spec.tile
+        return bool(self.ir.row_state or self.ir.col_state or (t.stages > 1 and t.walk == 1))
 
     def source(self) -> str:
         ir, sp, t = self.ir, self.spec, self.spec.tile
@@ -695,7 +718,7 @@ class Codegen:
         e("if (!a || !a->A || !a->B) return EVT_ERR_BAD_ARGS;")
         e("if (a->num_tensors != kNumTensors || a->num_scalars != kNumScalars) return EVT_ERR_BAD_ARGS;")
         e("if (a->M <= 0 || a->N <= 0 || a->K <= 0 || a->L <= 0) return EVT_ERR_BAD_ARGS;")
-        e("if (a->split_k < 0 || (a->flags & ~EVT_FLAG_TWO_KERNEL_REDUCE)) return EVT_ERR_BAD_ARGS;")
+        e("if (a->split_k < 0 || (a->flags & ~(EVT_FLAG_TWO_KERNEL_REDUCE | EVT_FLAG_ROW_WG_PER_CU_MASK))) return EVT_ERR_BAD_ARGS;")
         e("const bool two_kernel_reduce = (a->flags & EVT_FLAG_TWO_KERNEL_REDUCE) != 0;")
         e("g.M = a->M; g.N = a->N; g.K = a->K; g.L = a->L;")
         e("g.A = (const char*)a->A; g.lda = a->lda; g.bsA = a->batch_stride_A;")
@@ -763,6 +786,8 @@ class Codegen:
             e("}")
         e("if ((int64_t)g.tiles_m * g.tiles_n * a->L * g.splits > 0x7fffffffLL) return EVT_ERR_RANGE;")
         e("if (a->N > (1 << 24)) return EVT_ERR_RANGE;   // column indices are carried as fp32")
+        e("// a row's partial state is addressed with a 32-bit buffer offset inside its (batch, part) block")
+        e("if (Epi::ROW_STATE > 0 && (int64_t)a->M * Epi::ROW_STATE * 4 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
         if t.stages == 1:
             e("if (a->K > Cfg::BK) return EVT_ERR_RANGE;   // single-stage variant: K must fit one tile")
         if t.dma:
@@ -840,22 +865,29 @@ class Codegen:
         e("  if (need > 0 && (!ws || ws_bytes < need || ((uintptr_t)ws & 15))) return EVT_ERR_WORKSPACE;   // 16-byte aligned")
         e("  return enqueue(g, p, ws, stream);")
         e("}")
-        emit_static_scratch(e)
+        emit_static_scratch(e, self.uses_workspace())
         e('extern "C" int evt_launch_static(const EvtArgs* a, void* stream) {')
         e("  evt::GemmArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  const int64_t need = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g).total();")
+        e("  const evt::WsLayout wl = evt::ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g);")
+        e("  const int64_t need = wl.total();")
         e("  if (need > kScratchBytes) return EVT_ERR_SCRATCH;   // this problem's partial results do not fit the static array")
         e("  void* ws = nullptr;")
         e("  if (need > 0) {")
-        e("    const int rs = scratch_on_current_device(&ws);")
+        e("    const int rs = scratch_for_stream(stream, &ws);")
         e("    if (rs != EVT_OK) return rs;")
-        e("    // the array keeps the last call's contents, and another problem size lays its counters out elsewhere:")
-        e("    // everything this launch uses starts at zero (a fill kernel, not a memset node)")
-        e("    hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (uint32_t*)ws, (need + 3) / 4);")
-        e("    const int ef = (int)hipGetLastError();")
-        e("    if (ef != 0) return ef;")
+        e("    // The array keeps the last call's contents, and another problem size lays its counters out elsewhere:")
+        e("    // the arrival counters of this launch start at zero (fill kernels, not memset nodes).  Partial results")
+        e("    // and split-K tiles are written by every launch before it reads them and need no clearing.")
+        e("    const int64_t regions[2][2] = {{0, wl.counter_bytes}, {wl.counter_bytes + wl.row_bytes + wl.col_bytes, wl.split_counter_bytes}};")
+        e("    for (const auto& r : regions) {")
+        e("      if (r[1] <= 0) continue;")
+        e("      const unsigned blocks = (unsigned)((r[1] / 4 + 255) / 256 < 64 ? (r[1] / 4 + 255) / 256 : 64);")
+        e("      hipLaunchKernelGGL(evt::evt_fill_zero_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint32_t*)((char*)ws + r[0]), r[1] / 4);")
+        e("      const int ef = (int)hipGetLastError();")
+        e("      if (ef != 0) return ef;")
+        e("    }")
         e("  }")
         e("  return enqueue(g, p, ws, stream);")
         e("}")
@@ -1130,7 +1162,8 @@ class RowCodegen(Codegen):
         return {
             "abi": ABI_VERSION,
             "name": self.name,
-            "static_scratch_bytes": STATIC_SCRATCH_BYTES,   # what evt_launch_static can hold in place of a workspace
+            # what evt_launch_static can hold in place of a workspace (0: this kernel never uses one)
+            "static_scratch_bytes": STATIC_SCRATCH_BYTES if self.ir.col_state else 0,
             "anchor": sp.op,
             "row": {"chunks": sp.ch, "lanes_per_row": sp.lpr * sp.wpr, "waves_per_row": sp.wpr, "max_n": sp.max_n},
             "element": sp.elt,
@@ -1248,11 +1281,13 @@ class RowCodegen(Codegen):
             # a row per workgroup: 8 waves per CU walk over the rows, each fetching its next row ahead (measured
             # on 4096 x 30528: 100 us against 108 us with a workgroup per row)
             default_cap = 8 // sp.wpr
-        e("static unsigned grid_for(const evt::RowArgs& g) {")
-        e(f"  static const int per_cu = [] {{ const char* s = getenv(\"EVT_ROW_WG_PER_CU\"); int v = s ? atoi(s) : {default_cap}; "
-          f"return {'v > 0 ? v : 4' if ir.col_state else 'v'}; }}();")
+        e("static unsigned grid_for(const evt::RowArgs& g, int flags) {")
+        e("  // EvtArgs.flags carries the caller's choice (EVT_FLAG_ROW_WG_PER_CU); the module reads no environment")
+        e(f"  int per_cu = (flags & EVT_FLAG_ROW_WG_PER_CU_MASK) ? ((flags & EVT_FLAG_ROW_WG_PER_CU_MASK) >> 8) - 1 : {default_cap};")
         e("  static const int cus = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, "
           "hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256; return n; }();")
+        if ir.col_state:
+            e("  if (per_cu <= 0) per_cu = 4;   // a per-column reduction needs a bounded number of partials")
         e("  const int64_t want = ((int64_t)g.L * g.M + Cfg::ROWS - 1) / Cfg::ROWS;")
         e("  return (unsigned)((per_cu <= 0 || want < (int64_t)cus * per_cu) ? want : (int64_t)cus * per_cu);")
         e("}")
@@ -1261,7 +1296,7 @@ class RowCodegen(Codegen):
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
         e("  // partials of the per-column reductions, one per (workgroup, state word, column); nothing else is staged")
-        e("  return (int64_t)grid_for(g) * Epi::COL_STATE * g.N * 4;")
+        e("  return (int64_t)grid_for(g, a->flags) * Epi::COL_STATE * g.N * 4;")
         e("}")
         e('extern "C" int evt_workspace_init(void* ws, int64_t bytes, void* stream) {')
         e("  (void)ws; (void)bytes; (void)stream;      // no counters: every partial is written before it is read")
@@ -1272,22 +1307,22 @@ class RowCodegen(Codegen):
         e("  evt::RowArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  const unsigned grid = grid_for(g);")
+        e("  const unsigned grid = grid_for(g, a->flags);")
         e("  const int64_t need = (int64_t)grid * Epi::COL_STATE * g.N * 4;")
         e("  if (need > 0 && (!ws || ws_bytes < need)) return EVT_ERR_WORKSPACE;")
         e("  return enqueue(g, p, grid, ws, stream);")
         e("}")
-        emit_static_scratch(e)
+        emit_static_scratch(e, bool(ir.col_state))
         e('extern "C" int evt_launch_static(const EvtArgs* a, void* stream) {')
         e("  evt::RowArgs g; Epi::Params p;")
         e("  const int rc = fill(a, g, p);")
         e("  if (rc != EVT_OK) return rc;")
-        e("  const unsigned grid = grid_for(g);")
+        e("  const unsigned grid = grid_for(g, a->flags);")
         e("  const int64_t need = (int64_t)grid * Epi::COL_STATE * g.N * 4;")
         e("  if (need > kScratchBytes) return EVT_ERR_SCRATCH;")
         e("  void* ws = nullptr;")
         e("  if (need > 0) {   // partials only, each written before it is read: nothing to clear")
-        e("    const int rs = scratch_on_current_device(&ws);")
+        e("    const int rs = scratch_for_stream(stream, &ws);")
         e("    if (rs != EVT_OK) return rs;")
         e("  }")
         e("  return enqueue(g, p, grid, ws, stream);")

@@ -13,7 +13,7 @@ from __future__ import annotations
 
 import ctypes
 import operator
-import itertools
+import zlib
 import os
 from contextlib import nullcontext
 from dataclasses import replace
@@ -123,16 +123,27 @@ def _contig_strides(shape: Sequence[int]) -> Tuple[int, ...]:
 # ---------------------------------------------------------------------------
 
 
-_RAND_STREAM_IDS = itertools.count(1)
+def rand_stream_id(anchor_name: str) -> int:
+    """Stream id of a fused op's rand_like tensors: a 28-bit hash of its anchor
+    node's name.  Names are unique inside a graph, so two fused ops of one model
+    draw unrelated numbers, and they do not change from trace to trace, so the
+    same model traced again with the same seed draws the same masks (a count of
+    the ops created in the process would depend on every earlier trace, dry runs
+    included)."""
+    return (zlib.crc32(anchor_name.encode()) & 0x0FFFFFFF) or 1
 
 
 def launch_switches() -> Tuple[int, int]:
     """(EvtArgs.split_k, EvtArgs.flags) from the host's environment, read at
     every call: EVT_SPLIT_K=1|n turns split-K off / asks for n splits,
     EVT_TWO_KERNEL_REDUCE=1 finishes cross-tile reductions in the finalize
-    kernel.  The kernel modules themselves read no environment."""
+    kernel, EVT_ROW_WG_PER_CU=n sets the workgroups per CU of the row-wise
+    kernels.  The kernel modules themselves read no environment."""
     split = os.environ.get("EVT_SPLIT_K")
     flags = jit.EVT_FLAG_TWO_KERNEL_REDUCE if os.environ.get("EVT_TWO_KERNEL_REDUCE") == "1" else 0
+    per_cu = os.environ.get("EVT_ROW_WG_PER_CU")
+    if per_cu:
+        flags |= jit.evt_flag_row_wg_per_cu(max(0, min(254, int(per_cu))))
     return (max(0, int(split)) if split else 0), flags
 
 
@@ -161,11 +172,11 @@ class FusedOpBase:
         self._workspace = {}
         # rand_like stream: 64-bit seed (torch's global seed at the time of the call unless `rand_seed` is set), a
         # 32-bit offset that advances by one per launch, so successive calls draw different numbers, and a stream
-        # id of the op's own (process-wide count, in trace order) that goes into the generator's counter next to
-        # the slot index: two fused ops with rand_like tensors of equal shape draw unrelated numbers, as eager
-        # PyTorch does.  The offset is a launch argument: a captured HIP graph replays the mask it was captured with.
+        # id of the op's own (rand_stream_id: from the anchor node's name) that goes into the generator's counter
+        # next to the slot index: two fused ops with rand_like tensors of equal shape draw unrelated numbers, as
+        # eager PyTorch does.  The offset is a launch argument: a captured HIP graph replays the mask it was captured with.
         self._rand_seed: Optional[int] = None
-        self.rand_stream = next(_RAND_STREAM_IDS) & 0x0FFFFFFF
+        self.rand_stream = rand_stream_id(node.name)
         self.rand_offset = 0
         self.last_rand_state: Optional[Tuple[int, int]] = None   # (seed, offset) the most recent launch used
 
@@ -636,6 +647,14 @@ class FusedBMM(FusedOpBase):
         if self.copy_B:
             B = self._replay(self.chain_B, B)
             B = (B.transpose(1, 2) if self.transposed else B).contiguous()
+        if self.tile.dma:
+            # as in FusedGEMM.operands: a source tensor that starts at an odd storage offset is copied into a fresh
+            # (aligned) allocation; the strides inside it and the base offset of a `select` (both multiples of 8
+            # elements, or the element-wise module was chosen) carry over
+            if A.data_ptr() & 15:
+                A = A.clone()
+            if B.data_ptr() & 15:
+                B = B.clone()
         return A, self.lda, self.bsa, B, self.ldb, self.bsb
 
     def build_arguments(self, visitor_args, *args, block=None):
@@ -698,6 +717,7 @@ class FusedRowOp(FusedOpBase):
         a = block if block is not None else self.argument_block()
         a.M, a.N, a.K, a.L = M, N, 1, L
         a.A, a.lda, a.batch_stride_A = ops[0].data_ptr(), N, M * N
+        a.split_k, a.flags = launch_switches()
         if len(ops) > 1:
             a.B, a.ldb, a.batch_stride_B = ops[1].data_ptr(), N, M * N
         keep = list(ops)

@@ -62,6 +62,12 @@ class EvtArgs(ctypes.Structure):
 
 
 EVT_FLAG_TWO_KERNEL_REDUCE = 1
+EVT_FLAG_ROW_WG_PER_CU_MASK = 0xFF00
+
+
+def evt_flag_row_wg_per_cu(n: int) -> int:
+    """EVT_FLAG_ROW_WG_PER_CU(n) of include/evt_amd.h."""
+    return ((n + 1) & 0xFF) << 8
 
 ERROR_NAMES = {-1: "EVT_ERR_BAD_ARGS", -2: "EVT_ERR_ALIGNMENT", -3: "EVT_ERR_WORKSPACE", -4: "EVT_ERR_RANGE",
                -5: "EVT_ERR_SCRATCH"}

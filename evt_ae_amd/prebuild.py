@@ -1,6 +1,6 @@
 """Ahead-of-time build of every kernel module the smoke check and the benchmark
-use, so that nothing has to be compiled on the GPU box (tests/prebuild_tests.py
-does the same for the modules of the tests).
+use, so that nothing has to be compiled on the GPU box (`--with-tests` adds the
+modules of the repository's tests, which tests/prebuild_tests.py lists).
 
 Each workload is traced on meta tensors (no data, no GPU) exactly as it will be
 at run time, which registers its kernel module; the modules are then compiled
@@ -59,9 +59,40 @@ def register_all() -> List[jit.LazyModule]:
     return jit.registered_modules()
 
 
-def build_all(jobs: int = 8, force: bool = False, verbose: bool = True, register=None) -> List[jit.LazyModule]:
-    """`register`: further tracing to do before the build (a callable; it registers modules as a side effect)."""
+def _register_tests():
+    """The test catalogue's tracing step, when the repository's tests/ tree is there (a checkout); an installed
+    package has none, and only the benchmark's modules are built then."""
+    try:
+        from tests import prebuild_tests
+    except ImportError:
+        return None
+    return prebuild_tests.register_tests
+
+
+def prune_stale(mods, verbose: bool = True) -> int:
+    """Remove the files of modules that nothing registered any more: after a change of the kernel headers or the
+    ABI every module has a new hash, and the old binaries would still be picked up by whoever lists the folder."""
+    keep = {m.path.stem for m in mods}
+    removed = 0
+    for f in jit.KERNEL_DIR.glob("evt_*"):
+        if f.suffix in (".so", ".hip") and f.stem not in keep:
+            f.unlink()
+            removed += 1
+    if verbose and removed:
+        print(f"[prebuild] removed {removed} files of modules no longer registered", flush=True)
+    return removed
+
+
+def build_all(jobs: int = 8, force: bool = False, verbose: bool = True, register=None,
+              with_tests: bool = False, prune: bool = False) -> List[jit.LazyModule]:
+    """`register`: further tracing to do before the build (a callable; it registers modules as a side effect).
+    `with_tests` (command line: --with-tests): the modules of the repository's tests as well, if tests/ is there.
+    `prune` (--prune): afterwards delete the binaries and sources of modules that were not registered."""
     mods = register_all()
+    if with_tests and register is None:
+        register = _register_tests()
+        if register is None and verbose:
+            print("[prebuild] no tests/ tree beside the package: building the benchmark's modules only", flush=True)
     if register is not None:
         register()
         mods = jit.registered_modules()
@@ -75,8 +106,10 @@ def build_all(jobs: int = 8, force: bool = False, verbose: bool = True, register
                 print(f"[prebuild] built {m.name} -> {m.path.name}", flush=True)
     if verbose:
         print(f"[prebuild] done in {time.time() - t0:.1f}s", flush=True)
+    if prune:
+        prune_stale(mods, verbose)
     return mods
 
 
 if __name__ == "__main__":
-    build_all(force="--force" in sys.argv)
+    build_all(force="--force" in sys.argv, with_tests="--with-tests" in sys.argv, prune="--prune" in sys.argv)

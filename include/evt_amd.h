@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define EVT_ABI_VERSION 4
+#define EVT_ABI_VERSION 5
 #define EVT_MAX_TENSORS 16
 #define EVT_MAX_SCALARS 16
 
@@ -36,6 +36,14 @@ extern "C" {
  * kernel, also where the last workgroup to arrive could do it inside the GEMM
  * kernel (a test switch: both forms give the same bits). */
 #define EVT_FLAG_TWO_KERNEL_REDUCE 1
+/* EvtArgs.flags bits 8..15, row-wise modules only (GEMM modules ignore them):
+ * workgroups per CU before the waves of a row kernel walk over several rows,
+ * stored plus one (0 = the module's own default; EVT_FLAG_ROW_WG_PER_CU(0) = a
+ * workgroup per group of rows, no walking).  The workspace size of a row module
+ * with a per-column reduction depends on it: pass the same flags to
+ * evt_workspace_bytes and evt_launch.  The modules read no environment. */
+#define EVT_FLAG_ROW_WG_PER_CU(n) ((((n) + 1) & 0xff) << 8)
+#define EVT_FLAG_ROW_WG_PER_CU_MASK 0xff00
 
 /* Error codes returned by evt_launch / evt_workspace_bytes (negative); a
  * positive value is a hipError_t reported by the runtime at launch. */
@@ -171,18 +179,22 @@ int evt_launch(const EvtArgs* args, void* workspace, int64_t workspace_bytes,
 
 /* `evt_launch` for callers that cannot allocate device memory or be handed a
  * workspace: code under HIP graph capture, tight serving loops, harnesses that
- * forbid hipMalloc.  It has no counterpart in the reference (whose callers
- * allocate and zero their reduction outputs per call, evt_fuser.py:217-225).
+ * forbid hipMalloc.  It has no counterpart in the reference.
  * The partial results, arrival counters and split-K tiles that `evt_launch`
  * keeps in the caller's workspace live in a device array that is part of the
- * module ("static_scratch_bytes" in the module spec: 1 MiB), which every GPU the module runs
- * on holds from the first such call until the process ends; the call itself
- * allocates nothing and frees nothing.  A problem whose workspace
- * (evt_workspace_bytes) exceeds the array is refused with EVT_ERR_SCRATCH
- * before anything is enqueued.  All calls on one GPU share that GPU's array,
- * so calls that may overlap in time (different streams) race; each call
- * clears what it needs on `stream` first (a fill kernel).  Inputs and outputs
- * are passed as for `evt_launch`. */
+ * module ("static_scratch_bytes" in the module spec: 1 MiB, or 0 for a module
+ * whose kernels never use a workspace and which therefore carries no array),
+ * which every GPU the module runs on holds from the first such call until the
+ * process ends; the call itself allocates nothing and frees nothing.  A
+ * problem whose workspace (evt_workspace_bytes) exceeds the array is refused
+ * with EVT_ERR_SCRATCH before anything is enqueued.  The array used is the one
+ * of the GPU `stream` belongs to (the current GPU for the null stream).  All
+ * calls on one GPU share that GPU's array, so calls that may overlap in time
+ * (different streams) race; each call clears the arrival counters it uses on
+ * `stream` first (fill kernels, no memset node).  The first call on each GPU
+ * looks the array's address up and must happen outside a stream capture;
+ * later calls may be captured.  Inputs and outputs are passed as for
+ * `evt_launch`. */
 int evt_launch_static(const EvtArgs* args, void* stream);
 
 #ifdef __cplusplus

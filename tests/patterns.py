@@ -976,3 +976,147 @@ def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
     g = torch.Generator(device="cpu").manual_seed(0x5EED + seed)
     return (REFERENCE_PATTERNS.get(name) or RANDOM_PATTERNS.get(name) or MULTI_ANCHOR_PATTERNS.get(name)
             or ROW_ANCHOR_PATTERNS[name])[1](g)
+
+
+# ---------------------------------------------------------------------------
+# The reference's tuner caches as a coverage checklist (tests/golden/reference_tuner_keys.json): every GEMM / BMM
+# problem key there names a shape, a layout pair and seven epilogue-node counts
+# (python/gtl/compiler/autotuner/tuner_base.py:107-152).  `CountedEpilogue` is a synthetic epilogue with exactly
+# those counts behind a product of that shape and layout.
+# ---------------------------------------------------------------------------
+
+class CountedEpilogue(torch.nn.Module):
+    """acc = A B; x = acc + aux_0 + ... + rowvec_0 + ..., times colvec_0 ...;
+    stores x, gelu(x), relu(x) ... (aux_store of them), sums over the rows of x,
+    x * x ... (row_reduction of them: [N] results, fp32) and sums along the rows
+    (column_reduction: [M] results, fp32).  row_store: a value of the [N]
+    vectors alone (the reference stores the transformed attention mask that
+    way, visitor_store.hpp:46-145); it does not depend on the product, so this
+    backend leaves it to an eager kernel outside the fused one.
+    forward(A, B, *aux, *rowvec, *colvec)."""
+
+    def __init__(self, counts, a_row: bool, b_row: bool, batched: bool):
+        super().__init__()
+        self.counts = tuple(int(c) for c in counts)
+        self.a_row, self.b_row, self.batched = a_row, b_row, batched
+
+    @staticmethod
+    def with_arity(counts, a_row: bool, b_row: bool, batched: bool) -> "CountedEpilogue":
+        """torch.fx traces positional parameters only: a subclass whose forward names every input."""
+        n = int(counts[0]) + int(counts[1]) + int(counts[2])
+        names = ", ".join(f"e{i}" for i in range(n))
+        scope: dict = {}
+        exec(f"def forward(self, A, B{', ' + names if n else ''}):\n    return self.body(A, B, [{names}])\n", scope)
+        cls = type(f"CountedEpilogue_{'_'.join(str(int(c)) for c in counts)}", (CountedEpilogue,), {"forward": scope["forward"]})
+        return cls(counts, a_row, b_row, batched)
+
+    def forward(self, A, B, *extra):
+        return self.body(A, B, list(extra))
+
+    def body(self, A, B, extra):
+        aux, rowb, colb, stores, rowred, colred, rowstore = self.counts
+        swap = [0, 2, 1] if self.batched else [1, 0]
+        a = A if self.a_row else aten.permute(A, swap)
+        b = B if self.b_row else aten.permute(B, swap)
+        x = aten.bmm(a, b) if self.batched else aten.mm(a, b)
+        extra = list(extra)
+        for _ in range(aux):
+            x = aten.add(x, extra.pop(0))
+        rows = [extra.pop(0) for _ in range(rowb)]
+        for r in rows:
+            x = aten.add(x, r)
+        for _ in range(colb):
+            x = aten.mul(x, extra.pop(0))
+        outs = []
+        variants = (lambda t: t, lambda t: aten.gelu(t, approximate="tanh"), aten.relu, aten.tanh)
+        for j in range(stores):
+            outs.append(variants[j % len(variants)](x))
+        if rowred or colred:
+            xf = aten._to_copy(x, dtype=torch.float32)
+            power = xf
+            for j in range(rowred):
+                outs.append(aten.sum(power, [-2]))
+                power = aten.mul(power, xf)
+            power = xf
+            for j in range(colred):
+                outs.append(aten.sum(power, [-1]))
+                power = aten.mul(power, xf)
+        for j in range(rowstore):
+            outs.append(aten.mul(rows[j % len(rows)], -10000.0))
+        return tuple(outs)
+
+
+def parse_reference_key(key: str, batched: bool):
+    """`M_N_K_h_h_R_C[_7 counts]` (`L_M_N_K_...` batched) -> dict(L, M, N, K, a_row, b_row, counts), counts None for
+    the keys of the reference tuner's first stage (no epilogue: a plain store)."""
+    parts = key.split("_")
+    nd = 4 if batched else 3
+    dims = [int(p) for p in parts[:nd]]
+    L = dims.pop(0) if batched else 1
+    M, N, K = dims
+    assert parts[nd] == parts[nd + 1] == "h", key
+    la, lb = parts[nd + 2], parts[nd + 3]
+    rest = parts[nd + 4:]
+    counts = tuple(int(c) for c in rest) if rest else None
+    assert counts is None or len(counts) == 7, key
+    return dict(L=L, M=M, N=N, K=K, a_row=la == "R", b_row=lb == "R", counts=counts)
+
+
+def counted_epilogue_shapes(case):
+    """(shape, dtype) of every input of CountedEpilogue for a parsed key."""
+    L, M, N, K = case["L"], case["M"], case["N"], case["K"]
+    counts = case["counts"] or (0, 0, 0, 1, 0, 0, 0)
+    lead = (L,) if case["L"] > 1 or case.get("batched") else ()
+    shapes = [(lead + ((M, K) if case["a_row"] else (K, M)), torch.half),
+              (lead + ((K, N) if case["b_row"] else (N, K)), torch.half)]
+    shapes += [(lead + (M, N), torch.half)] * counts[0]
+    shapes += [((N,), torch.half)] * counts[1]
+    shapes += [(lead + (M, 1), torch.half)] * counts[2]
+    return shapes
+
+
+def counted_epilogue(case):
+    """-> (module, meta inputs) for a parsed reference key."""
+    counts = case["counts"] or (0, 0, 0, 1, 0, 0, 0)
+    batched = bool(case.get("batched"))
+    mod = CountedEpilogue.with_arity(counts, case["a_row"], case["b_row"], batched)
+    metas = [torch.empty(s, dtype=d, device="meta") for s, d in counted_epilogue_shapes(case)]
+    return mod, metas
+
+
+def reference_key_cases():
+    """Every GEMM / BMM key of the committed fixture, parsed: [(table, key, case)]."""
+    import json
+    from pathlib import Path
+    doc = json.loads((Path(__file__).resolve().parent / "golden" / "reference_tuner_keys.json").read_text())
+    out = []
+    for table, batched in (("best_config_mm", False), ("best_config_bmm", True)):
+        for key in doc["tables"][table]:
+            case = parse_reference_key(key, batched)
+            case["batched"] = batched
+            out.append((table, key, case))
+    return out
+
+
+def reference_row_key_cases():
+    """The distinct (anchor, rows, columns) of the fixture's softmax / layer norm keys, each with the bare anchor
+    as a module and its meta inputs: [(key, anchor, rows, cols, module, metas)]."""
+    import json
+    from pathlib import Path
+    doc = json.loads((Path(__file__).resolve().parent / "golden" / "reference_tuner_keys.json").read_text())
+    half, f32 = torch.float16, torch.float32
+    seen, out = set(), []
+    for table, anchor in (("best_config_softmax", "softmax"), ("best_config_softmax_backward", "softmax_backward"),
+                          ("best_config_layernorm", "layernorm"), ("best_config_layernorm_backward", "layernorm_backward")):
+        for key in doc["tables"][table]:
+            rows, cols = (int(v) for v in key.partition(")")[0].strip("(").split(","))
+            if (anchor, rows, cols) in seen:
+                continue
+            seen.add((anchor, rows, cols))
+            x = torch.empty((rows, cols), dtype=half, device="meta")
+            stat = torch.empty((rows, 1), dtype=f32, device="meta")
+            mod, metas = {"softmax": (_BareSoftmax(), [x]), "softmax_backward": (_BareSoftmaxBackward(half), [x, x]),
+                          "layernorm": (_BareLayerNorm(cols), [x]),
+                          "layernorm_backward": (_BareLayerNormBackward(cols), [x, x, stat, stat])}[anchor]
+            out.append((key, anchor, rows, cols, mod, metas))
+    return out

@@ -105,6 +105,11 @@ def register_tests() -> None:
     cfg, shapes, tile = W.NO_ALLOC_TOO_BIG
     with force_tile(TileConfig(*tile)):
         W.fuse(W.CONFIGS[cfg].module(), _shapes_of(cfg, shapes))
+    # the reference's tuner-cache keys (tests/golden/reference_tuner_keys.json): one synthetic epilogue per key
+    for _table, _key, case in W.reference_key_cases():
+        W.fuse(*W.counted_epilogue(case))
+    for _key, _anchor, _rows, _cols, mod, metas in W.reference_row_key_cases():
+        W.fuse(mod, metas)
     for name, (cls, _) in W.REFERENCE_PATTERNS.items():
         if name in ("mm10", "mm11"):      # shapes only: their inputs are large
             shapes = {"mm10": [(16384, 1024), (1024, 4096)], "mm11": [(33792, 768), (33792, 768)]}[name]

@@ -44,10 +44,10 @@ def test_every_built_module_exports_the_abi():
         for sym in declared_symbols():
             assert hasattr(lib, sym), f"{p.name} lacks {sym}"
         lib.evt_abi_version.restype = ctypes.c_int
-        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 4
+        assert lib.evt_abi_version() == jit.EVT_ABI_VERSION == 5
         lib.evt_module_spec.restype = ctypes.c_char_p
         spec = json.loads(lib.evt_module_spec().decode())
-        assert spec["abi"] == 4
+        assert spec["abi"] == 5
         if "anchor" in spec:      # row-wise reduce-apply module
             assert spec["anchor"] in ("softmax", "softmax_backward", "layernorm", "layernorm_backward")
             assert spec["element"] in ("f16", "bf16", "f32") and spec["row"]["max_n"] >= 1
@@ -122,6 +122,17 @@ def test_argument_validation_happens_before_launch(module):
     assert km.lib.evt_launch(ctypes.byref(big), None, 0, None) == -3    # EVT_ERR_WORKSPACE
     with pytest.raises(RuntimeError, match="EVT_ERR_WORKSPACE"):
         km.launch(big, 0, 0, 0)
+
+
+def test_row_partials_must_fit_a_32_bit_offset(module):
+    """The partial state of a row is written at a 32-bit byte offset inside its (batch, part) block: a problem so
+    tall that M x state x 4 bytes reaches 2 GiB is refused, not wrapped."""
+    op, km = module
+    a = _args(op, km)
+    a.M = (0x7FFFFFFF // 12) + 1                       # three floats of state per row
+    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) == -4     # EVT_ERR_RANGE
+    a.M = 0x7FFFFFFF // 12 - 64
+    assert km.lib.evt_workspace_bytes(ctypes.byref(a)) >= 0
 
 
 def test_workspace_size_formula(module):

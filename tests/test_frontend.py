@@ -12,6 +12,8 @@ from evt_ae_amd.evt_fuser import EVTFuser, FusedBMM, FusedGEMM, target_name
 from oracle import evt_oracle
 from tests.util import fused_nodes, rand_slot, run_emulated
 
+aten = torch.ops.aten
+
 
 def _check(module_cls, inputs, n_fused=1, tol=2e-5):
     gm = W.fuse(module_cls(), inputs)
@@ -167,33 +169,54 @@ def test_random_patterns_lower_correctly():
     assert abs(keep - 0.3) < 5e-3
 
 
+class TwoDropoutLayers(torch.nn.Module):
+    """Two layers of the reference's dropout pattern (unittest/evt_fuser/dropout.py:33-46) in one graph: two
+    fused partitions whose rand_like tensors have the same shape."""
+    def forward(self, x, w1, b1, w2, b2):
+        h = aten.add(aten.mm(x, aten.permute(w1, [1, 0])), b1)
+        m1 = aten.ge(torch.rand_like(h), 0.7)
+        h = aten.mul(aten.mul(h, m1), 1. / (1 - 0.7))
+        y = aten.add(aten.mm(h, aten.permute(w2, [1, 0])), b2)
+        m2 = aten.ge(torch.rand_like(y), 0.7)
+        y = aten.mul(aten.mul(y, m2), 1. / (1 - 0.7))
+        return y, m1, m2
+
+
 def test_two_dropout_partitions_draw_unrelated_masks():
-    """Two fused ops whose rand_like tensors have the same shape (the hidden
-    dropouts of two layers) must not share a random stream: same seed, same
-    offset, same slot index, yet different masks -- every op mixes a stream id
-    of its own into the generator's counter.  And the seed is read when the op
-    is called, so torch.manual_seed after tracing still takes effect."""
+    """Two fused ops of one graph whose rand_like tensors have the same shape
+    (the hidden dropouts of two layers) must not share a random stream: same
+    seed, same offset, same slot index, yet different masks -- every op mixes a
+    stream id of its own into the generator's counter.  The id comes from the
+    anchor node's name, so tracing the same model again (in the same process,
+    whatever was traced in between) gives the same (seed, offset, salt) and
+    the same masks, as eager PyTorch does for a fixed seed.  And the seed is
+    read when the op is called, so torch.manual_seed after tracing still takes
+    effect."""
     g = torch.Generator().manual_seed(7)
     h = lambda *s: (torch.randn(*s, generator=g) * 0.5).half()   # noqa: E731
-    inputs = [h(1024, 32), h(1024, 32), h(1024), h(512, 2, 1024)]
-    ops = []
-    for _ in range(2):
-        gm = W.fuse(W.Dropout1(), inputs)
-        (n,) = fused_nodes(gm)
-        ops.append((gm, n.target))
-    assert ops[0][1].rand_stream != ops[1][1].rand_stream
-    torch.manual_seed(1234)
-    masks = []
-    for gm, op in ops:
+    inputs = [h(256, 128), h(128, 128), h(128), h(128, 128), h(128)]
+    runs = []
+    for trace in range(2):
+        gm = W.fuse(TwoDropoutLayers(), inputs)
+        ops = [n.target for n in fused_nodes(gm)]
+        assert len(ops) == 2
+        assert ops[0].rand_stream != ops[1].rand_stream
+        torch.manual_seed(1234)
         got = run_emulated(gm, inputs)
-        assert op.last_rand_state == (1234, 0)
-        masks.append([o for o in got if o.dtype == torch.bool][-1])
-    assert not torch.equal(masks[0], masks[1])
-    agree = (masks[0] == masks[1]).float().mean().item()      # independent masks with keep rate 0.3 agree on 58 %
-    assert abs(agree - (0.3 * 0.3 + 0.7 * 0.7)) < 1e-2
+        assert all(op.last_rand_state == (1234, 0) for op in ops)
+        m1, m2 = [o for o in got if o.dtype == torch.bool]
+        assert not torch.equal(m1, m2)
+        agree = (m1 == m2).float().mean().item()      # independent masks with keep rate 0.3 agree on 58 %
+        assert abs(agree - (0.3 * 0.3 + 0.7 * 0.7)) < 2e-2
+        runs.append((gm, ops, [op.rand_salt(0) for op in ops], (m1, m2)))
+        W.fuse(W.Dropout1(), W.pattern_inputs("dropout1"))     # an unrelated trace in between changes nothing
+    assert runs[0][2] == runs[1][2]
+    assert torch.equal(runs[0][3][0], runs[1][3][0]) and torch.equal(runs[0][3][1], runs[1][3][1])
+    gm, ops = runs[0][0], runs[0][1]
     torch.manual_seed(99)                                      # after tracing: a new seed, new numbers
-    again = [o for o in run_emulated(ops[0][0], inputs) if o.dtype == torch.bool][-1]
-    assert ops[0][1].last_rand_state == (99, 1)
+    again = [o for o in run_emulated(gm, inputs) if o.dtype == torch.bool]
+    assert ops[0].last_rand_state == (99, 1)
+    assert not torch.equal(again[0], runs[0][3][0])
 
 
 def test_pass_decomposition_rewrites():
@@ -304,7 +327,7 @@ def test_row_anchor_patterns_trace(name):
     assert K == 1 and N == inputs[0].shape[-1] and L * M * N == inputs[0].numel()
     assert op.row_spec.max_n >= N and op.row_spec.lpr in (8, 16, 32, 64) and 1 <= op.row_spec.ch <= 16
     spec = op.module.spec
-    assert spec["abi"] == 4 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
+    assert spec["abi"] == 5 and spec["anchor"] == kind and spec["row"]["max_n"] == op.row_spec.max_n
     assert op.num_anchor_inputs == {"softmax": 1, "softmax_backward": 2, "layernorm": 1, "layernorm_backward": 5}[kind]
     if kind == "layernorm":
         # eps travels as a scalar; mean and rstd are per-row stores

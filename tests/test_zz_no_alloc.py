@@ -94,3 +94,32 @@ def test_static_entry_point_of_a_row_anchor():
     plain, static = _launch_both(op, dev, idx)
     for name in plain:
         assert torch.equal(plain[name].view(torch.uint8), static[name].view(torch.uint8)), name
+
+
+def test_static_entry_point_is_graph_capturable():
+    """After one eager call on the device (which looks the array's address up), evt_launch_static can be recorded
+    into a HIP graph: it enqueues fill kernels and the fused kernel, nothing else.  Every replay, with eager work
+    and synchronisations in between, reproduces evt_launch bit for bit."""
+    tile = TileConfig(*W.NO_ALLOC_TILE)
+    op, dev, idx = _op_for(3, W.NO_ALLOC_SHAPES[3][0], tile)
+    plain, static = _launch_both(op, dev, idx)                  # the eager warm-up call, outside capture
+    args = [dev[i] for i in idx]
+    outs = op.allocate_outputs("cuda")
+    a, keep = op.build_arguments(outs, *args, block=op.new_argument_block())
+    module = op.module.ensure()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        rc = module.lib.evt_launch_static(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+    for rep in range(3):
+        for t in outs.values():
+            t.view(torch.uint8).fill_(0x5A)
+        _ = (dev[0].float().sum() + rep).item()                 # unrelated eager work and a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        for name in plain:
+            assert torch.equal(plain[name].view(torch.uint8), outs[name].view(torch.uint8)), (rep, name)
+    del keep

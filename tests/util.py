@@ -82,3 +82,25 @@ def rand_slot(op: FusedOpBase) -> int:
     """Generator salt (slot index + 16 x the op's stream id) of the op's single rand_like slot."""
     (k,) = [k for k, s in enumerate(op.ir.slots) if s.kind == "rand"]
     return op.rand_salt(k)
+
+
+def fake_argument_block(op: FusedOpBase):
+    """The op's argument block with made-up (aligned, non-null) pointers: what the host side of a module needs
+    to run its checks and size its workspace without any device memory."""
+    from evt_ae_amd.evt_fuser import FusedRowOp
+    a = op.new_argument_block()
+    M, N, K, L = op.problem
+    a.M, a.N, a.K, a.L = M, N, K, L
+    a.A, a.B = 0x7000_0000_0000, 0x7100_0000_0000
+    if isinstance(op, FusedRowOp):
+        a.lda = a.ldb = N
+        a.batch_stride_A = a.batch_stride_B = M * N
+    else:
+        a.lda, a.ldb = op.lda, op.ldb
+        a.batch_stride_A, a.batch_stride_B = getattr(op, "bsa", 0), getattr(op, "bsb", 0)
+        if isinstance(op, FusedBMM):
+            a.batch_div_A, a.batch_stride2_A = op.bdiva, op.bs2a
+            a.batch_div_B, a.batch_stride2_B = op.bdivb, op.bs2b
+    for k in range(a.num_tensors):
+        a.tensors[k].ptr = 0x7200_0000_0000 + (k << 36)
+    return a
