@@ -359,18 +359,21 @@ class MfmaProbe:
             os.replace(tmp, self.path)
         return self.path
 
-    def run(self, torch, operands, workgroups=256, iters=1 << 15, warm_launches=6):
-        """operands: contiguous CUDA fp16 tensor of >= 65536 elements.  Returns (TFLOP/s, shader MHz) of the last
-        of `warm_launches` + 1 back-to-back launches."""
+    def run(self, torch, operands, b_operands=None, variant=0, workgroups=256, iters=1 << 15, warm_launches=6):
+        """operands (and b_operands, for the B-side registers; default: the same buffer): contiguous CUDA fp16
+        tensors of >= 65536 elements.  variant 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_f32_16x16x32_f16.  Returns
+        (TFLOP/s, shader MHz) of the last of `warm_launches` + 1 back-to-back launches."""
         import ctypes
         if self._lib is None:
             self.build()
             self._lib = ctypes.CDLL(str(self.path), mode=ctypes.RTLD_LOCAL)
             self._lib.evt_mfma_probe_launch.restype = ctypes.c_int
-            self._lib.evt_mfma_probe_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
-                                                        ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
-        if operands.dtype != torch.float16 or operands.numel() < 65536 or not operands.is_contiguous():
-            raise ValueError("operands: contiguous fp16 tensor of at least 65536 elements")
+            self._lib.evt_mfma_probe_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        b_operands = operands if b_operands is None else b_operands
+        for t in (operands, b_operands):
+            if t.dtype != torch.float16 or t.numel() < 65536 or not t.is_contiguous():
+                raise ValueError("operands: contiguous fp16 tensors of at least 65536 elements")
         sink = torch.zeros(1024, dtype=torch.float32, device=operands.device)
         clk = torch.zeros(2, dtype=torch.int64, device=operands.device)
         stream = torch.cuda.current_stream().cuda_stream
@@ -378,8 +381,8 @@ class MfmaProbe:
         for i in range(warm_launches + 1):
             if i == warm_launches:
                 e0.record()
-            rc = self._lib.evt_mfma_probe_launch(operands.data_ptr(), sink.data_ptr(), clk.data_ptr(), workgroups, iters,
-                                                 ctypes.c_void_p(stream))
+            rc = self._lib.evt_mfma_probe_launch(operands.data_ptr(), b_operands.data_ptr(), sink.data_ptr(), clk.data_ptr(),
+                                                 workgroups, iters, variant, ctypes.c_void_p(stream))
             if rc != 0:
                 raise RuntimeError(f"HIP Error {rc} launching the MFMA probe")
         e1.record()
@@ -509,6 +512,7 @@ def main():
         return
     cfgs = [int(c) for c in args.configs.split(",")]
     details = {}
+    operand_chunks = {}
     for cfg in cfgs:
         case = Case(cfg, torch, W, fused_nodes)
         wl = case.wl
@@ -560,6 +564,8 @@ def main():
         if args.clock_probe:
             details[cfg]["clock_probe"] = case.clock_probe(jit)
         log(f"[bench] config {cfg} {wl.name}: {details[cfg]}")
+        # 64 Ki elements of each anchor operand, for the register-only MFMA loop below
+        operand_chunks[cfg] = tuple(t.reshape(-1)[:1 << 16].clone() for t in case.sets[0][1][:2])
         del case
         torch.cuda.empty_cache()
 
@@ -601,7 +607,21 @@ def main():
         t_zero, mhz_zero = probe.run(torch, torch.zeros_like(rnd))
         mfma_only = {"normal_operands_tflops": round(t_rnd, 1), "normal_operands_shader_mhz": round(mhz_rnd),
                      "zero_operands_tflops": round(t_zero, 1), "zero_operands_shader_mhz": round(mhz_zero)}
+        # the same loop on chunks of each config's own operands (A-side registers from its left operand, B-side
+        # from its right one: activations ~ N(0, 1) against weights ~ N(0, 0.02)), with the 32x32x16 instruction of
+        # the fused kernels and with 16x16x32
+        own = {}
+        for cfg in sorted(operand_chunks):
+            a_chunk, b_chunk = operand_chunks[cfg]
+            t32, mhz32 = probe.run(torch, a_chunk, b_chunk, variant=0)
+            t16, mhz16 = probe.run(torch, a_chunk, b_chunk, variant=1)
+            own[str(cfg)] = {"mfma_32x32x16_tflops": round(t32, 1), "mfma_32x32x16_shader_mhz": round(mhz32),
+                             "mfma_16x16x32_tflops": round(t16, 1), "mfma_16x16x32_shader_mhz": round(mhz16)}
+            if "clock_probe" in details[cfg]:
+                details[cfg]["frac_of_mfma_only_own_operands"] = round(details[cfg]["tflops"] / t32, 4)
+        mfma_only["own_operands"] = own
         clock["frac_of_mfma_only_normal_operands"] = round(dom_tflops / t_rnd, 4)
+        clock["frac_of_mfma_only_own_operands"] = round(dom_tflops / own[str(dom)]["mfma_32x32x16_tflops"], 4)
         log(f"[bench] register-only MFMA loop: {mfma_only}")
     traffic = measured_traffic_bytes(details[dom]["_key"])
     for d in details.values():

@@ -136,7 +136,11 @@ class AutoTunerBase:
             # one wave per SIMD (pipe 12): 64 x 64 wave tiles on 128 x 128 (measured 8-19 % faster than eight
             # waves on the 4096 x 1024 and 1024 x 4096 products of an encoder layer), 64 x 128 on the larger ones
             shapes += [(128, 128, 64, 2, 2, 3, 12), (128, 128, 64, 2, 2, 4, 12), (256, 128, 64, 2, 2, 3, 12),
-                       (128, 256, 64, 2, 2, 3, 12)]
+                       (128, 256, 64, 2, 2, 3, 12),
+                       # at most 80 KB of LDS and 256 registers: two such workgroups share a CU, one's epilogue runs
+                       # under the other's main loop (measured 1.36 x over one per CU on the classifier problem,
+                       # where the ping-pong tiles that walk still win)
+                       (128, 256, 32, 2, 2, 3, 12), (256, 128, 32, 4, 1, 3, 12), (128, 128, 64, 2, 2, 2, 12)]
             if self.N == 512:     # one tile spans the rows: row statistics complete inside the workgroup
                 shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0),
                            # 32 x 256 wave tiles: 8 columns per lane halve the cross-lane steps per element of a

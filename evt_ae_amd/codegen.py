@@ -321,6 +321,70 @@ class Codegen:
         e.dedent()
         e("}")
 
+    def onehot_label(self, r) -> str | None:
+        """A per-row sum of where(label == column index, x, 0) -- a gather along the row -- has at most one
+        non-zero term per row, and for most (wave, tile) pairs none: the name of the per-row `label` value if `r`
+        is such a sum and the label's value can be formed from per-row loads alone, else None."""
+        ir = self.ir
+        if r.axis != "row" or r.kind != "sum" or r.fold:
+            return None
+        n = ir.nodes[r.input]
+        if n.op != "where" or len(n.inputs) != 3:
+            return None
+        hit, _x, zero = (ir.nodes[i] for i in n.inputs)
+        if zero.op != "imm" or ir.scalars[zero.slot] != 0.0 or hit.op != "eq":
+            return None
+        a, b = hit.inputs
+        if ir.nodes[a].op == "colidx":
+            a, b = b, a
+        if ir.nodes[b].op != "colidx":
+            return None
+        for name in ir.closure([a]):
+            m = ir.nodes[name]
+            if self.var_n[name] or m.op in ("accum", "rres", "rowval", "anchorval", "colidx"):
+                return None
+            if m.op == "load" and ir.slots[m.slot].kind not in ("col", "scalar"):
+                return None
+            if m.op not in ("load", "imm", "where") and m.op not in _UNARY and m.op not in _BINARY:
+                return None
+        return a
+
+    def emit_onehot_vote(self, e: _Emitter, labels: List[str]):
+        """`oh_hit`: does the label of this lane's row(s) of the wave tile name one of this wave's columns?  (The
+        loads go out at the top of the tile; the vote over the wave is taken where the answer is needed.)"""
+        ir = self.ir
+        e("bool oh_hit = false;")
+        e("#pragma unroll")
+        e("for (int j = 0; j < (Cfg::TM + 63) / 64; ++j) {")
+        e.indent()
+        e("const int lr = t.lane + 64 * j, vr = t.row_u + lr;")
+        e("const bool vok = lr < Cfg::TM && vr < t.M;")
+        for name in ir.closure(labels):
+            n = ir.nodes[name]
+            c = "q" + _cname(name)
+            if n.op == "imm":
+                e(f"const float {c} = p.s[{n.slot}];")
+            elif n.op == "load":
+                k = n.slot
+                if ir.slots[k].kind == "col":
+                    e(f"const float {c} = vok ? evt::ld_f32(p.t{k}, bo_{k} + (int64_t)vr * p.t{k}_sm) : -1.f;")
+                else:
+                    e(f"const float {c} = evt::ld_f32(p.t{k}, 0);")
+            else:
+                a = ["q" + _cname(i) for i in n.inputs]
+                if n.op in _BINARY:
+                    ex = _BINARY[n.op].format(a=a[0], b=a[1])
+                elif n.op in _UNARY:
+                    ex = _UNARY[n.op].format(a=a[0])
+                else:
+                    ex = f"(({a[0]} != 0.f) ? {a[1]} : {a[2]})"
+                e(f"const float {c} = {ex};")
+        for lab in labels:
+            c = "q" + _cname(lab)
+            e(f"oh_hit |= vok && {c} >= (float)t.col_u && {c} < (float)(t.col_u + Cfg::TN);")
+        e.dedent()
+        e("}")
+
     def emit_tile(self, e: _Emitter):
         ir = self.ir
         tile_stores = [s for s in ir.stores if s.domain == "tile"]
@@ -329,7 +393,17 @@ class Codegen:
         roots = [s.input for s in tile_stores] + [r.input for r in ir.reduces.values()]
         need = ir.closure(roots)
         hoisted = [n for n in need if not self.var_m[n]]
-        inner = [n for n in need if self.var_m[n]]
+        # One-hot row sums (a gather along the row) are collected in a pass of their own, which a wave skips when
+        # none of its rows' labels names one of its columns (wave tiles of two or more 32-row blocks)
+        onehot: Dict[str, str] = {}
+        if self.spec is not None and self.spec.tile.bm // self.spec.tile.wm // 32 >= 2 and not col_reds:
+            for r in row_reds:
+                lab = self.onehot_label(r)
+                if lab is not None:
+                    onehot[r.name] = lab
+        main_roots = [s.input for s in tile_stores] + [r.input for r in ir.reduces.values() if r.name not in onehot]
+        inner = [n for n in ir.closure(main_roots) if self.var_m[n]]
+        oh_inner = [n for n in ir.closure([ir.reduces[name].input for name in onehot]) if self.var_m[n]]
 
         aux_nodes = [n for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "aux"]
         e("template <class Cfg, class Tile, bool FAST>")
@@ -345,7 +419,7 @@ class Codegen:
             e(f"[[maybe_unused]] const int64_t bo_{k} = evt::batch_offset(t.batch, p.t{k}_lm, p.t{k}_ld, p.t{k}_sl, p.t{k}_sl2);")
         self._tile_offsets = True
         # one value per row (column vectors): check-free path through buffer loads, the row's offset in a scalar
-        col_loads = sorted({ir.nodes[n].slot for n in inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "col"})
+        col_loads = sorted({ir.nodes[n].slot for n in inner + oh_inner if ir.nodes[n].op == "load" and ir.slots[ir.nodes[n].slot].kind == "col"})
         for k in col_loads:
             e(f"[[maybe_unused]] __amdgpu_buffer_rsrc_t rc_{k};")
             e(f"[[maybe_unused]] uint32_t vc_{k} = 0;")
@@ -357,6 +431,8 @@ class Codegen:
         # hoisted values
         for name in hoisted:
             self.emit_node(e, ir.nodes[name], hoisted=True)
+        if onehot:
+            self.emit_onehot_vote(e, sorted(set(onehot.values())))
         if col_reds:
             e(f"float cst[NI][{ir.col_state}];")
             e("#pragma unroll")
@@ -388,6 +464,8 @@ class Codegen:
         # With one 32-row block per wave (MI = 1) each row is reduced as it is produced (ROW_BY_ROW), which runs under
         # the row's stores; larger wave tiles collect the values and reduce all rows together afterwards
         e("constexpr bool ROW_BY_ROW = MI == 1;")
+        if onehot:
+            e('static_assert(!ROW_BY_ROW, "the separate pass of one-hot row sums is generated for wave tiles of two or more row blocks");')
         for r in row_reds:
             if r.kind in ("sum", "max"):
                 e(f"[[maybe_unused]] float rp_{_cname(r.name)}[16 * MI];")
@@ -456,7 +534,7 @@ class Codegen:
             self.emit_tile_store(e, k, arr)
             e.dedent()
             e("}")
-        if row_reds:
+        if row_reds and not onehot:
             e("if constexpr (ROW_BY_ROW) {")
             e.indent()
             e(f"float rst[{ir.row_state}];")
@@ -467,6 +545,8 @@ class Codegen:
             e("} else {")
             e.indent()
         for r in row_reds:
+            if r.name in onehot:
+                continue
             c, x = _cname(r.name), self.ref(r.input)
             if r.kind == "sum":
                 e(f"{{ float a = 0.f;\n#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) a += t.col_ok(ni) ? {x} : 0.f;\nrp_{c}[mi * 16 + v] = a; }}")
@@ -474,7 +554,7 @@ class Codegen:
                 e(f"{{ float a = -INFINITY;\n#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) a = t.col_ok(ni) ? fmaxf(a, {x}) : a;\nrp_{c}[mi * 16 + v] = a; }}")
             else:
                 e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) rx_{c}[mi * 16 + v][ni] = {x};")
-        if row_reds:
+        if row_reds and not onehot:
             e.dedent()
             e("}")
         for r in col_reds:
@@ -495,12 +575,56 @@ class Codegen:
         e("}")
         e.dedent()
         e("}")
+        if row_reds and onehot:      # the other reductions first: the vote's loads travel meanwhile
+            for r in row_reds:
+                if r.name in onehot:
+                    continue
+                c, o = _cname(r.name), r.state_offset
+                if r.kind in ("sum", "max"):
+                    e(f"evt::rows_simple<Cfg, {ir.row_state}, {'true' if r.kind == 'max' else 'false'}>(t, rp_{c}, {o});")
+                elif r.kind == "maxsumexp":
+                    e(f"evt::rows_maxsumexp<Cfg, {ir.row_state}, {ir.col_state}>(t, rx_{c}, {o});")
+                elif r.kind == "welford":
+                    e(f"evt::rows_welford<Cfg, {ir.row_state}, {ir.col_state}>(t, rx_{c}, {o});")
+                else:
+                    raise NotImplementedError(r.kind)
+        if onehot:
+            e("const bool oh_any = __builtin_amdgcn_ballot_w64(oh_hit) != 0;   // wave-uniform")
+            e("if (oh_any) {")
+            e.indent()
+            e("#pragma unroll")
+            e("for (int mi = 0; mi < MI; ++mi) {")
+            e.indent()
+            e("#pragma unroll")
+            e("for (int v = 0; v < 16; ++v) {")
+            e.indent()
+            e("const int row = t.row(mi, v);")
+            e("const bool rok = t.row_ok(row);")
+            for name in oh_inner:
+                self.emit_node(e, ir.nodes[name], hoisted=False)
+            for name in onehot:
+                r = ir.reduces[name]
+                c, x = _cname(r.name), self.ref(r.input)
+                e(f"{{ float a = 0.f;\n#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) a += t.col_ok(ni) ? {x} : 0.f;\nrp_{c}[mi * 16 + v] = a; }}")
+            e("(void)row; (void)rok;")
+            e.dedent()
+            e("}")
+            e.dedent()
+            e("}")
+            e.dedent()
+            e("}")
         if row_reds:
             e("if constexpr (!ROW_BY_ROW) {")
             e.indent()
         for r in row_reds:
             c, o = _cname(r.name), r.state_offset
-            if r.kind in ("sum", "max"):
+            if r.name in onehot:
+                # no label of this wave's rows names one of its columns: every term is zero
+                e(f"if (oh_any) evt::rows_simple<Cfg, {ir.row_state}, false>(t, rp_{c}, {o});")
+                e(f"else evt::rows_fill<Cfg, {ir.row_state}>(t, {o}, 0.f);")
+            elif onehot:
+                pass        # emitted above
+            elif r.kind in ("sum", "max"):
                 e(f"evt::rows_simple<Cfg, {ir.row_state}, {'true' if r.kind == 'max' else 'false'}>(t, rp_{c}, {o});")
             elif r.kind == "maxsumexp":
                 e(f"evt::rows_maxsumexp<Cfg, {ir.row_state}, {ir.col_state}>(t, rx_{c}, {o});")

@@ -1077,6 +1077,15 @@ EVT_DEV void rows_simple(const Tile& t, float (&part)[16 * Cfg::MI], int o) {   
   for (int e = 0; e < rows_owned<R>(); ++e) own[e] = part[e];
   rows_state_store<Cfg, RS>(t, o, own);
 }
+// component o of the rows' states when every term of a sum is known to be zero (a gather whose labels all lie
+// outside this wave's columns): the same stores as rows_simple, without the reduction
+template <class Cfg, int RS, class Tile>
+EVT_DEV void rows_fill(const Tile& t, int o, float value) {
+  float own[rows_owned<16 * Cfg::MI>()];
+#pragma unroll
+  for (int e = 0; e < rows_owned<16 * Cfg::MI>(); ++e) own[e] = value;
+  rows_state_store<Cfg, RS>(t, o, own);
+}
 template <class Cfg, int RS, int CS, class Tile>
 EVT_DEV void rows_maxsumexp(const Tile& t, const float (&x)[16 * Cfg::MI][Cfg::NI], int o) {
   constexpr int R = 16 * Cfg::MI;
@@ -1235,7 +1244,7 @@ EVT_DEV void run_epilogue(const GemmArgs& g, const typename Epi::Params& p, int 
 }
 
 template <class Cfg, class Epi>
-__global__ void __launch_bounds__(Cfg::THREADS) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
   // a walking workgroup keeps one running state per row behind the operand stages
   constexpr int WALK_BYTES = Cfg::WALK ? Cfg::BM * (Epi::ROW_STATE > 0 ? Epi::ROW_STATE : 1) * 4 : 0;
   __shared__ __attribute__((aligned(1024))) char smem[Cfg::LDS_BYTES + WALK_BYTES];

@@ -144,6 +144,10 @@ struct GemmCfg {
   static constexpr int B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  // One-wave-per-SIMD workgroups whose LDS leaves room for a second workgroup on the CU are compiled for two
+  // waves per SIMD (at most 256 registers): two such workgroups then share a CU and run out of step, one's
+  // epilogue under the other's main loop.
+  static constexpr int MIN_WAVES_PER_SIMD = (SOLO && LDS_BYTES <= 80 * 1024) ? 2 : 1;
   static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be 32-aligned");
   static_assert(STAGES >= 1 && STAGES <= 8, "1..8 stages");
