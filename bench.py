@@ -392,6 +392,41 @@ class MfmaProbe:
         flops = workgroups * 8 * iters * 8 * 32768.0
         return flops / (ms * 1e-3) / 1e12, 100.0 * cycles / max(ticks, 1)
 
+    def run_mix(self, torch, operands, b_operands, lds_reads, transfers, workgroups=256, iters=1 << 14, warm_launches=6):
+        """The 32x32x16 loop with `lds_reads` ds_read_b128 and `transfers` global -> LDS transfers (1 KiB per wave
+        each) between every 8 MFMAs.  Returns (TFLOP/s, shader MHz)."""
+        import ctypes
+        self.run(torch, operands, b_operands, iters=64, warm_launches=0)      # loads the library
+        fn = self._lib.evt_mfma_probe_launch_mix
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                       ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        sink = torch.zeros(1024, dtype=torch.float32, device=operands.device)
+        clk = torch.zeros(2, dtype=torch.int64, device=operands.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(warm_launches + 1):
+            if i == warm_launches:
+                e0.record()
+            rc = fn(operands.data_ptr(), b_operands.data_ptr(), operands.data_ptr(), sink.data_ptr(), clk.data_ptr(),
+                    workgroups, iters, lds_reads, transfers, ctypes.c_void_p(stream))
+            if rc != 0:
+                raise RuntimeError(f"error {rc} launching the MFMA / traffic mix ({lds_reads}, {transfers})")
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        cycles, ticks = (int(x) for x in clk.cpu())
+        flops = workgroups * 8 * iters * 8 * 32768.0
+        return flops / (ms * 1e-3) / 1e12, 100.0 * cycles / max(ticks, 1)
+
+
+def main_loop_traffic(tile):
+    """Per k-tile of one workgroup: (MFMAs 32x32x16, KiB read from LDS into fragments, KiB moved global -> LDS)."""
+    mfmas = (tile.bm // 32) * (tile.bn // 32) * (tile.bk // 16)
+    dma_kib = (tile.bm + tile.bn) * tile.bk * 2 / 1024.0
+    lds_kib = tile.wm * tile.wn * (tile.bm // tile.wm + tile.bn // tile.wn) * tile.bk * 2 / 1024.0
+    return mfmas, lds_kib, dma_kib
+
 
 # ---------------------------------------------------------------------------
 # HBM-side traffic of the fused kernels, from rocprofv3 counter runs of this script
@@ -512,7 +547,7 @@ def main():
         return
     cfgs = [int(c) for c in args.configs.split(",")]
     details = {}
-    operand_chunks = {}
+    operand_chunks, tiles = {}, {}
     for cfg in cfgs:
         case = Case(cfg, torch, W, fused_nodes)
         wl = case.wl
@@ -566,6 +601,7 @@ def main():
         log(f"[bench] config {cfg} {wl.name}: {details[cfg]}")
         # 64 Ki elements of each anchor operand, for the register-only MFMA loop below
         operand_chunks[cfg] = tuple(t.reshape(-1)[:1 << 16].clone() for t in case.sets[0][1][:2])
+        tiles[cfg] = case.op.tile
         del case
         torch.cuda.empty_cache()
 
@@ -620,6 +656,36 @@ def main():
             if "clock_probe" in details[cfg]:
                 details[cfg]["frac_of_mfma_only_own_operands"] = round(details[cfg]["tflops"] / t32, 4)
         mfma_only["own_operands"] = own
+        # What the traffic of a main loop costs next to its MFMAs on this data: the loop with LDS reads and global ->
+        # LDS transfers mixed in, on the dominant config's operands; the cost of a KiB of either kind, in units of one
+        # MFMA, follows from the rates (the part is power-bound on this data: rate ~ 1 / energy per MFMA).  With them,
+        # every config's main loop gets a predicted rate from its tile's traffic, beside the rate it reached.
+        a_chunk, b_chunk = operand_chunks[dom]
+        mix = {}
+        for r_, d_ in ((0, 0), (6, 0), (8, 0), (0, 2), (0, 3), (6, 3)):
+            t_, mhz_ = probe.run_mix(torch, a_chunk, b_chunk, r_, d_)
+            mix[f"{r_}_reads_{d_}_transfers_per_8_mfma"] = {"tflops": round(t_, 1), "shader_mhz": round(mhz_)}
+        base = mix["0_reads_0_transfers_per_8_mfma"]["tflops"]
+        e_lds = ((base / mix["8_reads_0_transfers_per_8_mfma"]["tflops"] - 1.0) / 1.0 +
+                 (base / mix["6_reads_0_transfers_per_8_mfma"]["tflops"] - 1.0) / 0.75) / 2.0
+        e_dma = ((base / mix["0_reads_3_transfers_per_8_mfma"]["tflops"] - 1.0) / 0.375 +
+                 (base / mix["0_reads_2_transfers_per_8_mfma"]["tflops"] - 1.0) / 0.25) / 2.0
+        both = base / (1.0 + 0.75 * e_lds + 0.375 * e_dma)
+        mfma_only["traffic_mix"] = {"rates": mix, "mfma_energies_per_kib_lds_read": round(e_lds, 3),
+                                    "mfma_energies_per_kib_global_to_lds": round(e_dma, 3),
+                                    "check_6_reads_3_transfers": {"predicted_tflops": round(both, 1),
+                                                                  "measured_tflops": mix["6_reads_3_transfers_per_8_mfma"]["tflops"]}}
+        for cfg in sorted(operand_chunks):
+            if "clock_probe" not in details[cfg]:
+                continue
+            mfmas, lds_kib, dma_kib = main_loop_traffic(tiles[cfg])
+            ceiling = own[str(cfg)]["mfma_32x32x16_tflops"]
+            predicted = ceiling / (1.0 + e_lds * lds_kib / mfmas + e_dma * dma_kib / mfmas)
+            reached = W.CONFIGS[cfg].flops / (details[cfg]["clock_probe"]["wg0_mainloop_us"] * 1e-6) / 1e12
+            details[cfg]["main_loop_model"] = {
+                "mfmas_per_k_tile": mfmas, "lds_read_kib_per_k_tile": round(lds_kib, 1), "global_to_lds_kib_per_k_tile": round(dma_kib, 1),
+                "mfma_only_tflops_own_operands": ceiling, "predicted_main_loop_tflops": round(predicted, 1),
+                "reached_main_loop_tflops": round(reached, 1), "reached_over_predicted": round(reached / predicted, 3)}
         clock["frac_of_mfma_only_normal_operands"] = round(dom_tflops / t_rnd, 4)
         clock["frac_of_mfma_only_own_operands"] = round(dom_tflops / own[str(dom)]["mfma_32x32x16_tflops"], 4)
         log(f"[bench] register-only MFMA loop: {mfma_only}")

@@ -73,6 +73,8 @@ def main():
     ap.add_argument("--short-list", action="store_true", help="only the tiles of SHORT_LIST")
     ap.add_argument("--cache", default=None, help="tuner cache file to write (default: the package's)")
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    ap.add_argument("--sigma", default=None, help="standard deviations of the timing operands, 'sigma_A,sigma_B' "
+                                                    "(default: 1.0,0.02, activations against weights)")
     args = ap.parse_args()
     # candidates must be enumerated without consulting an existing cache
     os.environ["EVT_TUNER_CACHE"] = "/nonexistent/tuner_cache.db"
@@ -102,20 +104,26 @@ def main():
         os.environ["EVT_TUNER_CACHE"] = args.cache
     else:
         os.environ.pop("EVT_TUNER_CACHE")
+    if args.sigma:
+        sigma = tuple(float(x) for x in args.sigma.split(","))
     for cfg, t in tuners:
         t.cache_file = default_cache_file()
-        results = []
-        for tile in t.candidates():
-            try:
-                us = t.profile(tile)
-            except RuntimeError as exc:
-                print(f"[tune] config {cfg} {tile.tag()}: {exc}", flush=True)
-                continue
-            results.append((us, tile))
-            print(f"[tune] config {cfg} {tile.tag():40s} {us:9.2f} us", flush=True)
-        us, best = min(results, key=lambda r: r[0])
+        if args.sigma:
+            t.operand_sigma = sigma
+
+        def report(tile, us, note, cfg=cfg):
+            if us is None:
+                print(f"[tune] config {cfg} {tile.tag():40s} FAILED: {note.splitlines()[0][:200]}", flush=True)
+            else:
+                print(f"[tune] config {cfg} {tile.tag():40s} {us:9.2f} us" + (f"  ({note})" if note else ""), flush=True)
+        results = t.sweep(report)
+        if not results:
+            print(f"[tune] config {cfg}: no candidate could be timed", flush=True)
+            continue
+        us, best = t.second_stage(results, report)
         t.store(best, us)
-        print(f"[tune] config {cfg} best {best.tag()} {us:.2f} us -> {t.cache_file}", flush=True)
+        print(f"[tune] config {cfg} best {best.tag()} {us:.2f} us -> {t.cache_file} "
+              f"(operands N(0, {t.operand_sigma[0]}) x N(0, {t.operand_sigma[1]}), {len(t.failed)} candidates failed)", flush=True)
 
 
 if __name__ == "__main__":

@@ -13,6 +13,7 @@ row or the analytic heuristic is used, so tracing never needs a device.
 from __future__ import annotations
 
 import json
+import logging
 import os
 import sqlite3
 from contextlib import contextmanager
@@ -52,16 +53,37 @@ def force_tile(tile: TileConfig):
         _FORCED_TILE = prev
 
 
+log = logging.getLogger("evt_ae_amd.tuner")
+
+
+def default_operand_sigma() -> Tuple[float, float]:
+    """Standard deviations the tuner draws its A and B operands with.  The clock the part holds, and with it the
+    ranking of tiles, depends on the bit activity of the operands, so candidates are timed on data distributed like
+    the workload's: activations against weights, N(0, 1) x N(0, 0.02), unless EVT_TUNE_SIGMA="sa,sb" says otherwise
+    (the fuser knows shapes, not distributions)."""
+    env = os.environ.get("EVT_TUNE_SIGMA")
+    if env:
+        sa, sb = (float(x) for x in env.split(","))
+        return sa, sb
+    return 1.0, 0.02
+
+
 class AutoTunerBase:
     table = "best_config"
     warmup_iterations = 10
     profile_iterations = 50
+    # second stage (reference: gemm_tuner.py:102-137, the best tiles timed again with the epilogue in place): the
+    # `second_stage_tiles` fastest candidates of the sweep are timed again, in turns, `second_stage_rounds` times
+    second_stage_tiles = 3
+    second_stage_rounds = 3
 
     def __init__(self, problem: Tuple[int, int, int, int], a_kc: bool, b_kc: bool, bf16: bool, dma: bool,
                  ir: EpilogueIR) -> None:
         self.M, self.N, self.K, self.L = problem
         self.a_kc, self.b_kc, self.bf16, self.dma, self.ir = a_kc, b_kc, bf16, dma, ir
         self.cache_file = default_cache_file()
+        self.operand_sigma = default_operand_sigma()      # (sigma_A, sigma_B) of the timing operands
+        self.failed: List[Tuple[TileConfig, str]] = []    # candidates that did not build or launch, and why
 
     # -- key (reference: tuner_base.py:107-152, gemm_tuner.py:95-100) -----------
     def epilogue_key(self) -> str:
@@ -218,8 +240,9 @@ class AutoTunerBase:
         dev = "cuda"
         dt = torch.bfloat16 if self.bf16 else torch.float16
         M, N, K, L = self.M, self.N, self.K, self.L
-        A = torch.randn(L, M, K, device=dev, dtype=dt) if self.a_kc else torch.randn(L, K, M, device=dev, dtype=dt)
-        B = torch.randn(L, N, K, device=dev, dtype=dt) if self.b_kc else torch.randn(L, K, N, device=dev, dtype=dt)
+        sa, sb = self.operand_sigma
+        A = (torch.randn((L, M, K) if self.a_kc else (L, K, M), device=dev, dtype=torch.float32) * sa).to(dt)
+        B = (torch.randn((L, N, K) if self.b_kc else (L, K, N), device=dev, dtype=torch.float32) * sb).to(dt)
         a = jit.EvtArgs()
         a.M, a.N, a.K, a.L = M, N, K, L
         a.A, a.lda, a.batch_stride_A = A.data_ptr(), (K if self.a_kc else M), M * K
@@ -271,17 +294,53 @@ class AutoTunerBase:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / self.profile_iterations
 
-    def tune(self) -> TileConfig:
-        best, best_us = None, None
+    def sweep(self, report=None) -> List[Tuple[float, TileConfig]]:
+        """Time every candidate once; a candidate that fails to build or to launch is recorded in `self.failed`
+        and logged, never dropped silently.  `report(tile, us or None, error or None)` is called per candidate."""
+        results = []
+        self.failed = []
         for tile in self.candidates():
             try:
                 us = self.profile(tile)
-            except RuntimeError:
+            except RuntimeError as exc:
+                self.failed.append((tile, str(exc)))
+                log.warning("tuner: candidate %s of %s failed: %s", tile.tag(), self.key(), str(exc).splitlines()[0][:300])
+                if report is not None:
+                    report(tile, None, str(exc))
                 continue
-            if best_us is None or us < best_us:
-                best, best_us = tile, us
-        if best is None:
+            results.append((us, tile))
+            if report is not None:
+                report(tile, us, None)
+        return results
+
+    def second_stage(self, results: List[Tuple[float, TileConfig]], report=None) -> Tuple[float, TileConfig]:
+        """The fastest few tiles of the sweep timed again, in turns (so that clock drift and neighbours on the
+        machine hit all of them alike); the winner is the tile with the lowest median."""
+        top = sorted(results, key=lambda r: r[0])[:max(1, self.second_stage_tiles)]
+        if len(top) == 1 or self.second_stage_rounds <= 0:
+            return top[0]
+        samples = {tile: [us] for us, tile in top}
+        for _ in range(self.second_stage_rounds):
+            for _, tile in top:
+                try:
+                    samples[tile].append(self.profile(tile))
+                except RuntimeError as exc:
+                    self.failed.append((tile, str(exc)))
+                    log.warning("tuner: candidate %s of %s failed in the second stage: %s", tile.tag(), self.key(),
+                                str(exc).splitlines()[0][:300])
+        med = {tile: sorted(v)[len(v) // 2] for tile, v in samples.items()}
+        best = min(med, key=med.get)
+        if report is not None:
+            for tile, us in med.items():
+                report(tile, us, "second stage")
+        return med[best], best
+
+    def tune(self) -> TileConfig:
+        results = self.sweep()
+        if not results:
+            log.warning("tuner: no candidate of %s could be timed (%d failed); using the modelled tile", self.key(), len(self.failed))
             return self.heuristic()
+        best_us, best = self.second_stage(results)
         self.store(best, best_us)
         return best
 

@@ -886,7 +886,7 @@ class Codegen:
         e("g.col_inkernel = (g.tiles_m * g.col_fold_count <= evt::kMaxInKernelPartials && !two_kernel_reduce) ? 1 : 0;")
         e("// Split-K: when the output tiles cannot fill the chip and K is long, several workgroups share a tile")
         e("// (EvtArgs.split_k: 0 = decide here, 1 = off, n = n splits)")
-        e("g.splits = 1; g.k_chunk = (a->K + Cfg::BK - 1) / Cfg::BK * Cfg::BK;")
+        e("g.splits = 1; g.split_group = 0; g.k_chunk = (a->K + Cfg::BK - 1) / Cfg::BK * Cfg::BK;")
         if t.stages > 1 and t.walk == 1:
             e("{")
             e("  const int want = a->split_k;")
@@ -896,16 +896,21 @@ class Codegen:
             e("  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * a->L;")
             e("  int s = 1;")
             e("  if (want > 1) s = want < kt ? want : kt;")
-            e("  // automatic: only small outputs -- every split writes and the last arriver reads a whole fp32 tile, which")
-            e("  // costs more than the idle CUs once the output runs to megabytes; at most 4 Mi elements over all splits")
-            e("  // (1024 x 1024 x 4096 measured 22 us with 4 splits, 40 us with 8, 30 us unsplit)")
-            e("  else if (want == 0 && tiles * 2 <= cus && kt >= 8 && (int64_t)a->M * a->N * a->L <= (1 << 20)) "
-              "{ s = (int)(cus / tiles); if (s > 8) s = 8; if (s > kt / 4) s = kt / 4;"
-              " const int64_t cap = (4 << 20) / ((int64_t)a->M * a->N * a->L); if (s > cap) s = cap < 1 ? 1 : (int)cap; }")
+            e("  // automatic: small outputs only, a split per CU the tiles leave idle, four k-tiles or more each, while the")
+            e("  // exchange stays small -- every split writes a whole fp32 tile and the last arrivers read them back, which")
+            e("  // costs more than idle CUs once it runs to megabytes: at most 4 Mi elements over all splits (1024 x 1024 x")
+            e("  // 4096 on 128 x 128 tiles measured 22 us with 4 splits, 40 us with 8, 30 us unsplit; 64 x 64 x 736389 takes")
+            e("  // a split per CU)")
+            e("  else if (want == 0 && tiles * 2 <= cus && kt >= 8 && (int64_t)a->M * a->N * a->L <= (1 << 20)) {")
+            e("    s = (int)(cus / tiles); if (s > kt / 4) s = kt / 4;")
+            e("    const int64_t cap = (4 << 20) / (tiles * Cfg::BM * Cfg::BN); if (s > cap) s = cap < 1 ? 1 : (int)cap;")
+            e("  }")
             e("  if (s >= 2) {")
             e("    const int chunk = (kt + s - 1) / s;")
             e("    g.splits = (kt + chunk - 1) / chunk;      // every split has work")
             e("    g.k_chunk = chunk * Cfg::BK;")
+            e("    // more than 16 splits meet in groups first: nobody reads more than 16 + 16 tiles alone")
+            e("    if (g.splits > 16) g.split_group = g.splits > 128 ? 16 : (g.splits + 7) / 8 < 4 ? 4 : (g.splits + 7) / 8;")
             e("  }")
             e("}")
         e("if ((int64_t)g.tiles_m * g.tiles_n * a->L * g.splits > 0x7fffffffLL) return EVT_ERR_RANGE;")
@@ -1046,16 +1051,17 @@ class RowSpec:
         return self.ch * self.lpr * self.wpr * 8
 
     @staticmethod
-    def registers(op: str, elt: str, ch: int, lookahead: bool) -> float:
+    def registers(op: str, elt: str, ch: int, lookahead: bool, col_state: int = 0) -> float:
         """Registers per lane that hold row data: the fp32 working copies (two
         for the backward anchors), the operands as loaded, twice when the next
-        row is fetched ahead, and layer norm backward's weight."""
+        row is fetched ahead, layer norm backward's weight, and the partials
+        of the epilogue's per-column reductions (`col_state` words per column)."""
         two = 2 if op in ("softmax_backward", "layernorm_backward") else 1
         weight = ch * 8 if op == "layernorm_backward" else 0      # this lane's columns of the weight, kept across rows
-        return ch * 8 * two * (1 + (1.0 if elt == "f32" else 0.5) * (2 if lookahead else 1)) + weight
+        return ch * 8 * two * (1 + (1.0 if elt == "f32" else 0.5) * (2 if lookahead else 1)) + weight + col_state * ch * 8
 
     @staticmethod
-    def for_row_length(op: str, n: int, elt: str) -> "RowSpec":
+    def for_row_length(op: str, n: int, elt: str, col_state: int = 0) -> "RowSpec":
         """Smallest lane group that holds the row in two chunks per lane (four
         for softmax), a full wave with up to 16 chunks for longer rows.  Rows longer
         than 8192 go over 2 .. 16 waves, as few as keep the row data within
@@ -1072,7 +1078,7 @@ class RowSpec:
             return RowSpec(op, ch, lpr, elt)
         for wpr, budget in ((2, 192), (4, 192), (8, 192), (16, 96)):
             ch = (n + wpr * 512 - 1) // (wpr * 512)
-            if ch <= 16 and RowSpec.registers(op, elt, ch, wpr < 16) <= budget:
+            if ch <= 16 and RowSpec.registers(op, elt, ch, wpr < 16, col_state) <= budget:
                 return RowSpec(op, ch, 64, elt, wpr)
         raise NotImplementedError(f"rows of {n} {elt} elements do not fit the register-cached {op} kernel")
 
@@ -1091,9 +1097,18 @@ class RowCodegen(Codegen):
             # the row would be a second pass over the anchor's own axis
             if r.axis != "col" or r.kind not in ("sum", "max"):
                 raise NotImplementedError(f"per-row reduction {r.name} behind a row-wise anchor")
-        if ir.col_state and (spec.wpr > 1 or ir.L != 1 or ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536):
-            raise NotImplementedError("per-column reduction behind a row-wise anchor: one batch and rows of at most "
-                                      f"{65536 // (4 * max(ir.col_state, 1))} elements")
+        if ir.col_state and ir.L != 1:
+            raise NotImplementedError("per-column reduction behind a row-wise anchor: the rows must form one batch")
+        if ir.col_state and spec.wpr == 1 and ir.col_state * spec.ch * spec.lpr * 8 * 4 > 65536:
+            raise NotImplementedError("per-column reduction behind a row-wise anchor: the waves' partials of a row of "
+                                      f"{spec.max_n} elements do not fit the LDS")
+        if ir.col_state and spec.wpr > 1:
+            # a row over several waves: every lane carries the partials of its own columns in registers, next to
+            # the row data (three quarters of the lane's registers at most, as for the row data alone)
+            budget = 96 if spec.wpr == 16 else 192
+            if RowSpec.registers(spec.op, spec.elt, spec.ch, spec.wpr < 16, ir.col_state) > budget:
+                raise NotImplementedError("per-column reduction behind a row-wise anchor: the partials of a row of "
+                                          f"{spec.max_n} elements over {spec.wpr} waves do not fit the registers")
         # a kernel that reduces over the rows runs 8 waves per workgroup: as many rows in flight per CU from half
         # the workgroups, so half the partials for the second phase (16 waves would cap a wave at 128 registers,
         # which spills the layer norm backward kernel)

@@ -492,14 +492,19 @@ __host__ __device__ inline WsLayout ws_layout(const GemmArgs& g) {
   w.split_counter_bytes = w.split_bytes = 0;
   return w;
 }
+// number of groups of a two-level split-K exchange (GemmArgs::split_group), 0 for one level
+__host__ __device__ inline int split_groups(const GemmArgs& g) {
+  return (g.split_group > 1 && g.split_group < g.splits) ? (g.splits + g.split_group - 1) / g.split_group : 0;
+}
 // with the split-K regions, which need the tile size
 template <class Cfg, int ROW_STATE, int COL_STATE>
 __host__ __device__ inline WsLayout ws_layout_split(const GemmArgs& g) {
   WsLayout w = ws_layout<ROW_STATE, COL_STATE>(g);
   if (g.splits > 1) {
     const int64_t tiles = (int64_t)g.L * g.tiles_m * g.tiles_n;
-    w.split_counter_bytes = (tiles * 4 + 255) / 256 * 256;
-    w.split_bytes = tiles * g.splits * Cfg::BM * Cfg::BN * 4;
+    const int groups = split_groups(g);      // 0: one level
+    w.split_counter_bytes = (tiles * (1 + groups) * 4 + 255) / 256 * 256;
+    w.split_bytes = tiles * (g.splits + groups) * Cfg::BM * Cfg::BN * 4;
   }
   return w;
 }
@@ -1189,36 +1194,64 @@ __device__ uint64_t evt_clock_probe[4];
 // (consecutive lanes write consecutive words); the one whose ticket is the last reads all of them back in split
 // order -- its own included, so the sum does not depend on who arrived last -- and returns true: it goes on to
 // the epilogue; the others are done.
-template <class Cfg, class Epi>
-EVT_DEV bool split_k_exchange(const GemmArgs& g, unsigned tile_id, int split, char* smem, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
-  const WsLayout wl = ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g);
-  char* region = g.workspace + wl.counter_bytes + wl.row_bytes + wl.col_bytes;
-  int* counter = (int*)region + tile_id;
-  constexpr int REGS = Cfg::MI * Cfg::NI * 16;
-  float* part = (float*)(region + wl.split_counter_bytes) + (int64_t)tile_id * g.splits * REGS * Cfg::THREADS;
-  float* mine = part + (int64_t)split * REGS * Cfg::THREADS + threadIdx.x;
+template <class Cfg>
+EVT_DEV void split_k_store(float* dst, const f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) st_device(mine + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS, acc[mi][ni][v]);
-  __syncthreads();                 // nobody still reads operand tiles from the LDS the flag lives in
-  if (!arrive_last(counter, g.splits, (int*)smem)) return false;
+      for (int v = 0; v < 16; ++v) st_device(dst + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS, acc[mi][ni][v]);
+}
+// acc = tiles[first] + ... + tiles[first + count - 1], added in that order
+template <class Cfg>
+EVT_DEV void split_k_sum(const float* tiles, int first, int count, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  constexpr int REGS = Cfg::MI * Cfg::NI * 16;
 #pragma unroll
   for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
     for (int ni = 0; ni < Cfg::NI; ++ni)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
-  for (int sp = 0; sp < g.splits; ++sp) {
-    const float* src = part + (int64_t)sp * REGS * Cfg::THREADS + threadIdx.x;
+  for (int sp = first; sp < first + count; ++sp) {
+    const float* src = tiles + (int64_t)sp * REGS * Cfg::THREADS + threadIdx.x;
 #pragma unroll
     for (int mi = 0; mi < Cfg::MI; ++mi)
 #pragma unroll
       for (int ni = 0; ni < Cfg::NI; ++ni)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[mi][ni][v] += ld_device(src + ((mi * Cfg::NI + ni) * 16 + v) * Cfg::THREADS);
+  }
+}
+// With groups (split_groups(g) > 0) the exchange has two levels: the last workgroup of a group of consecutive splits
+// adds the group's tiles up in split order and leaves the sum as the group's tile, the last group to finish adds the
+// groups' tiles up in group order.  Which workgroup does either is a matter of timing; what is added, and in which
+// order, is not.
+template <class Cfg, class Epi>
+EVT_DEV bool split_k_exchange(const GemmArgs& g, unsigned tile_id, int split, char* smem, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  const WsLayout wl = ws_layout_split<Cfg, Epi::ROW_STATE, Epi::COL_STATE>(g);
+  char* region = g.workspace + wl.counter_bytes + wl.row_bytes + wl.col_bytes;
+  const int groups = split_groups(g);
+  const int64_t tiles_total = (int64_t)g.L * g.tiles_m * g.tiles_n;
+  int* counter = (int*)region + tile_id;
+  constexpr int REGS = Cfg::MI * Cfg::NI * 16;
+  float* part = (float*)(region + wl.split_counter_bytes) + (int64_t)tile_id * (g.splits + groups) * REGS * Cfg::THREADS;
+  split_k_store<Cfg>(part + (int64_t)split * REGS * Cfg::THREADS + threadIdx.x, acc);
+  __syncthreads();                 // nobody still reads operand tiles from the LDS the flag lives in
+  if (groups == 0) {
+    if (!arrive_last(counter, g.splits, (int*)smem)) return false;
+    split_k_sum<Cfg>(part, 0, g.splits, acc);
+  } else {
+    const int grp = split / g.split_group, first = grp * g.split_group;
+    const int count = g.splits - first < g.split_group ? g.splits - first : g.split_group;
+    int* group_counter = (int*)region + tiles_total + (int64_t)tile_id * groups + grp;
+    if (!arrive_last(group_counter, count, (int*)smem)) return false;
+    split_k_sum<Cfg>(part, first, count, acc);
+    __syncthreads();               // everybody has read the flag
+    if (threadIdx.x == 0) __hip_atomic_store(group_counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    split_k_store<Cfg>(part + (int64_t)(g.splits + grp) * REGS * Cfg::THREADS + threadIdx.x, acc);
+    if (!arrive_last(counter, groups, (int*)smem)) return false;
+    split_k_sum<Cfg>(part, g.splits, groups, acc);
   }
   __syncthreads();
   if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch

@@ -72,6 +72,10 @@ struct GemmArgs {
   // they leave their accumulators in the workspace and the last one to arrive adds them up in split order and
   // runs the epilogue.  splits == 1: one workgroup per tile, nothing goes through the workspace.
   int splits, k_chunk;
+  // Many splits meet in two levels: `split_group` consecutive splits form a group whose last arriver adds the
+  // group's tiles up and leaves one tile; the last group to finish adds up the groups' tiles.  The last arriver of a
+  // one-level exchange would read every tile alone.  0 or >= splits: one level.
+  int split_group;
   // GemmCfg::WALK: a workgroup computes `walk` consecutive tiles of a row block, left to right, and a per-row
   // reduction leaves one partial per workgroup: parts_n = ceil(tiles_n / walk) of them per row.  Elsewhere
   // walk = 1 and parts_n = tiles_n.

@@ -539,7 +539,6 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
   t.sub = Cfg::WPR > 1 ? (int)threadIdx.x : lane % Cfg::LPR;
   __shared__ float xch[2 * 16];
   RowReduce<Cfg> red{xch, 0};
-  static_assert(CS == 0 || Cfg::WPR == 1, "per-column reductions need a row per wave");
   // (batch, row in the batch) of the walker's present row: kept up to date by addition, since the rows of a run
   // follow each other (a 64-bit division per visit costs more instructions than the rest of a short row's work).
   // Batches shorter than 64 rows take the division.
@@ -679,7 +678,20 @@ __global__ __launch_bounds__(Cfg::THREADS) void evt_row_kernel(RowArgs g, typena
       }
     }
   }
-  if constexpr (CS > 0) {
+  if constexpr (CS > 0 && Cfg::WPR > 1) {
+    // A row over the whole workgroup: every thread has carried the partials of its own columns over all the rows
+    // the workgroup visited, so there is nothing to combine inside the workgroup.  One partial per (workgroup,
+    // column) goes to the workspace, as below.
+#pragma unroll
+    for (int k = 0; k < CS; ++k)
+#pragma unroll
+      for (int c = 0; c < Cfg::CH; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int n = c * Cfg::SPAN + t.sub * 8 + j;
+          if (n < g.N) g.colws[((int64_t)blockIdx.x * CS + k) * g.N + n] = cst[k][c][j];
+        }
+  } else if constexpr (CS > 0) {
     // Column partials of the workgroup: first across the row groups of a wave (lanes that hold the same
     // columns of different rows), then across the waves, which add their share into one LDS copy one after
     // the other in wave order; one partial per (workgroup, column) goes to the workspace and a second kernel

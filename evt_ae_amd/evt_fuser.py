@@ -707,7 +707,9 @@ class FusedRowOp(FusedOpBase):
         if dtype not in (torch.float16, torch.bfloat16, torch.float32):
             raise NotImplementedError(f"{self.row_op} operands of dtype {dtype}")
         self.problem = (v.M, v.N, 1, v.L)
-        self.row_spec = RowSpec.for_row_length(self.row_op, v.N, DTYPE_NAMES[dtype])
+        # (a per-column reduction of the epilogue keeps its partials in registers next to the row: rows over several
+        # waves then take more waves)
+        self.row_spec = RowSpec.for_row_length(self.row_op, v.N, DTYPE_NAMES[dtype], self.ir.col_state)
         self.spec = self.row_spec
         self.module = jit.load_module(self.ir, self.row_spec)
 
@@ -1446,8 +1448,10 @@ class EVTFuser:
             raise NotImplementedError(
                 f"{node.name}: reduces over something other than the N axis (optionally with batches folded) "
                 f"or exactly the M axis")
-        if fold and kind not in ("sum", "max"):
-            raise NotImplementedError(f"{node.name}: {kind} reduction that also folds batches")
+        if fold and axis == "col" and kind not in ("sum", "max"):
+            raise NotImplementedError(f"{node.name}: per-column {kind} reduction that also folds batches")
+        # (a per-row reduction of any kind may fold batches: the partial states of the batches that share a result
+        # go through the workspace and are merged with the kind's own combine operator, in batch order)
         for other in self.ir.reduces.values():
             if other.axis == axis and (other.fold, other.fold_step, other.fold_count) != (fold, fold_step, fold_count):
                 raise NotImplementedError(f"{node.name}: per-{axis} reductions of one epilogue fold batches differently")

@@ -89,31 +89,38 @@ def interpret(ir, accum: torch.Tensor, slot_tensors: Dict[int, torch.Tensor]) ->
         elif node.op == "rres":
             r = ir.reduces[node.reduce]
             x = val[r.input].expand(L, M, N)
-            dim = 2 if r.axis == "row" else 1
+            fold = getattr(r, "fold", "")
+            if fold:
+                # Batches that share a result are reduced together: bring them side by side in front of the reduced
+                # axis ([groups, members, M, N]), reduce over members and the axis, and let every member carry the
+                # total.  'mod': batch l = j * step + key belongs to group key; 'div': l = key * count + j.
+                cnt = r.fold_count
+                g4 = x.reshape(cnt, L // cnt, M, N).transpose(0, 1) if fold == "mod" else x.reshape(L // cnt, cnt, M, N)
+                dims = (1, 3) if r.axis == "row" else (1, 2)
+            else:
+                g4 = x.reshape(L, 1, M, N)
+                dims = (1, 3) if r.axis == "row" else (1, 2)
             if r.kind == "sum":
-                out = x.sum(dim, keepdim=True)
+                out = g4.sum(dims, keepdim=True)
             elif r.kind == "max":
-                out = x.amax(dim, keepdim=True)
+                out = g4.amax(dims, keepdim=True)
             elif r.kind == "maxsumexp":
-                mx = x.amax(dim, keepdim=True)
-                out = mx if node.comp == 0 else torch.exp(x - mx).sum(dim, keepdim=True)
+                mx = g4.amax(dims, keepdim=True)
+                out = mx if node.comp == 0 else torch.exp(g4 - mx).sum(dims, keepdim=True)
             elif r.kind == "welford":
-                cnt = x.shape[dim]
-                mean = x.mean(dim, keepdim=True)
-                out = (torch.full_like(mean, float(cnt)) if node.comp == 0 else mean if node.comp == 1
-                       else ((x - mean) ** 2).sum(dim, keepdim=True))
+                cnt_el = g4.shape[dims[0]] * g4.shape[dims[1]]
+                mean = g4.mean(dims, keepdim=True)
+                out = (torch.full_like(mean, float(cnt_el)) if node.comp == 0 else mean if node.comp == 1
+                       else ((g4 - mean) ** 2).sum(dims, keepdim=True))
             else:
                 raise NotImplementedError(r.kind)
-            if getattr(r, "fold", ""):
-                # batches that share a result are reduced together; every one of them then carries the total
-                if r.kind not in ("sum", "max"):
-                    raise NotImplementedError(f"folded {r.kind}")
-                cnt = r.fold_count
-                tail = (M, 1) if r.axis == "row" else (1, N)
-                grouped = out.view(cnt, L // cnt, *tail) if r.fold == "mod" else out.view(L // cnt, cnt, *tail)
-                axis = 0 if r.fold == "mod" else 1
-                tot = grouped.sum(axis, keepdim=True) if r.kind == "sum" else grouped.amax(axis, keepdim=True)
-                out = tot.expand_as(grouped).reshape(L, *tail)
+            tail = (M, 1) if r.axis == "row" else (1, N)
+            if fold:
+                members = g4.shape[1]
+                out = out.expand(g4.shape[0], members, *tail)
+                out = out.transpose(0, 1).reshape(L, *tail) if fold == "mod" else out.reshape(L, *tail)
+            else:
+                out = out.reshape(L, *tail)
             val[name] = out
         else:
             val[name] = _apply(node.op, [val[i] for i in node.inputs])

@@ -264,6 +264,29 @@ class FoldConsecutiveBatches(torch.nn.Module):
         return y, aten.mul(s, 0.5)
 
 
+class FoldedLogSumExp(torch.nn.Module):
+    """Not a reference test: log-sum-exp and (biased) variance / mean of a BMM result along its rows and over
+    pairs of consecutive batches -- reductions with a two- and a three-word state that fold batches."""
+    def forward(self, a, b, r):
+        bmm = aten.bmm(a, b)
+        y = aten.add(bmm, r)
+        v = aten._to_copy(aten.view(y, [3, 2, 40, 72]), dtype=torch.float32)
+        lse = aten.logsumexp(v, [1, 3])
+        vm = aten.var_mean(v, [1, 3], correction=0, keepdim=False)
+        return y, lse, operator.getitem(vm, 0), operator.getitem(vm, 1)
+
+
+class FoldedModuloVariance(torch.nn.Module):
+    """The same statistics over the batches that agree modulo 3 (batch l = i * 3 + j, reduced over i)."""
+    def forward(self, a, b, r):
+        bmm = aten.bmm(a, b)
+        y = aten.add(bmm, r)
+        v = aten._to_copy(aten.view(y, [2, 3, 40, 72]), dtype=torch.float32)
+        vm = aten.var_mean(v, [0, 3], correction=0, keepdim=False)
+        lse = aten.logsumexp(v, [0, 3])
+        return y, operator.getitem(vm, 0), operator.getitem(vm, 1), lse
+
+
 def fold_consecutive_inputs():
     g = torch.Generator(device="cpu").manual_seed(17)
     return [_h(g, (6, 40, 24), 0.3), _h(g, (6, 24, 72), 0.3), _h(g, (6, 40, 72), 0.3)]
@@ -599,6 +622,10 @@ ROW_ANCHOR_PATTERNS = {
     "softmax_column_broadcast": (SoftmaxColumnBroadcast, lambda g: [_h(g, (16384, 512)), _h(g, (16384, 1))]),
     "softmax_column_reduce": (SoftmaxColumnReduce, lambda g: [_h(g, (16, 512))]),
     "softmax_column_reduce_tall": (SoftmaxColumnReduce, lambda g: [_h(g, (40000, 512))]),
+    # rows over several waves of a workgroup with a sum over all rows behind them (every lane carries the partials
+    # of its own columns): 12288 columns, and a vocabulary-sized row whose length is no multiple of 8
+    "softmax_column_reduce_wide": (SoftmaxColumnReduce, lambda g: [_h(g, (300, 12288))]),
+    "softmax_column_reduce_vocab": (SoftmaxColumnReduce, lambda g: [_h(g, (70, 30522))]),
     "softmax_ragged": (SoftmaxRagged, lambda g: [_h(g, (3, 5, 37, 203), 3.0), _h(g, (37, 1))]),
     "softmax_backward": (SoftmaxBackward, lambda g: [_h(g, (4, 16, 512, 512)), _softmax_out(g, (4, 16, 512, 512))]),
     "layernorm1": (LayerNormPattern1, lambda g: [_h(g, (512, 2, 1024)) + 1., _h(g, (1024,)), _h(g, (1024,))]),

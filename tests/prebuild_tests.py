@@ -27,6 +27,8 @@ def register_tests() -> None:
     for name, (cls, _) in W.RANDOM_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
     W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
+    W.fuse(W.FoldedLogSumExp(), _meta(W.fold_consecutive_inputs()))
+    W.fuse(W.FoldedModuloVariance(), _meta(W.fold_consecutive_inputs()))
     for name, (cls, _) in W.MULTI_ANCHOR_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
     for name, (cls, _) in W.ROW_ANCHOR_PATTERNS.items():

@@ -214,3 +214,41 @@ def test_shipped_tuner_cache_is_read():
         (n,) = fused_nodes(gm)
         picked.add(n.target.tile)
     assert picked <= set(rows.values())
+
+
+def test_tuner_reports_candidates_that_fail(monkeypatch, caplog):
+    """A candidate that does not build or launch is logged and listed in `failed`, the others are still ranked, the
+    fastest few are timed again (second stage), and the timing operands are drawn like the workload's: activations
+    N(0, 1) against weights N(0, 0.02) unless the caller says otherwise."""
+    import logging
+    from evt_ae_amd.autotuner.gemm_tuner import MMTuner
+    from evt_ae_amd.codegen import TileConfig
+    monkeypatch.setenv("EVT_TUNER_CACHE", "/nonexistent/tuner_cache.db")
+    inputs = W.make_inputs(1, W.GOLDEN_SHAPES[1])
+    (n,) = fused_nodes(W.fuse(W.CONFIGS[1].module(), [t.to("meta") for t in inputs]))
+    tuner = MMTuner((512, 512, 256, 1), True, False, False, True, n.target.ir)
+    assert tuner.operand_sigma == (1.0, 0.02)
+    monkeypatch.setenv("EVT_TUNE_SIGMA", "0.5,0.25")
+    assert MMTuner((512, 512, 256, 1), True, False, False, True, n.target.ir).operand_sigma == (0.5, 0.25)
+    tiles = [TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2), TileConfig(128, 128, 64, 2, 2, 3, True, 4, 12),
+             TileConfig(64, 64, 64, 2, 2, 2, True, 4, 0), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 3)]
+    times = {tiles[0]: [30.0, 31.0, 29.0, 30.5], tiles[2]: [50.0], tiles[3]: [29.5, 33.0, 34.0, 35.0]}
+    calls = []
+
+    def fake_profile(self, tile):
+        calls.append(tile)
+        if tile == tiles[1]:
+            raise RuntimeError("hipcc failed for evt_x.hip:\nerror: too many registers")
+        seq = times[tile]
+        return seq[min(calls.count(tile) - 1, len(seq) - 1)]
+    monkeypatch.setattr(MMTuner, "candidates", lambda self: list(tiles))
+    monkeypatch.setattr(MMTuner, "profile", fake_profile)
+    stored = []
+    monkeypatch.setattr(MMTuner, "store", lambda self, tile, us: stored.append((tile, us)))
+    with caplog.at_level(logging.WARNING, logger="evt_ae_amd.tuner"):
+        best = tuner.tune()
+    assert [t for t, _ in tuner.failed] == [tiles[1]] and "too many registers" in tuner.failed[0][1]
+    assert any("failed" in r.getMessage() and tiles[1].tag() in r.getMessage() for r in caplog.records)
+    # the sweep alone would have picked tiles[3] (29.5 us); timed again in turns its median is 34 us against 30.5
+    assert best == tiles[0] and stored == [(tiles[0], 30.5)]
+    assert calls.count(tiles[0]) == 1 + tuner.second_stage_rounds and calls.count(tiles[1]) == 1

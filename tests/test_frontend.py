@@ -107,6 +107,17 @@ def test_batch_folded_row_reductions_lower_correctly():
     (red,) = n.target.ir.reduces.values()
     assert (red.fold, red.fold_count) == ("div", 2)
 
+    # reductions with a two- and a three-word state fold batches as well: (max, sum-exp) and (count, mean, M2)
+    # states of the batches that share a result are merged with their own combine operators
+    gm = _check(W.FoldedLogSumExp, W.fold_consecutive_inputs())
+    (n,) = fused_nodes(gm)
+    assert sorted((r.kind, r.fold, r.fold_count) for r in n.target.ir.reduces.values()) == \
+        [("maxsumexp", "div", 2), ("welford", "div", 2)]
+    gm = _check(W.FoldedModuloVariance, W.fold_consecutive_inputs())
+    (n,) = fused_nodes(gm)
+    assert sorted((r.kind, r.fold, r.fold_step, r.fold_count) for r in n.target.ir.reduces.values()) == \
+        [("maxsumexp", "mod", 3, 2), ("welford", "mod", 3, 2)]
+
 
 def test_fit_strides_batch_terms():
     from evt_ae_amd.ir import Coord, accum_coord, fit_strides

@@ -270,7 +270,9 @@ def test_batch_folded_row_reductions(two_kernel, monkeypatch):
     the finalize kernel."""
     if two_kernel:
         monkeypatch.setenv("EVT_TWO_KERNEL_REDUCE", "1")
-    cases = [(W.FoldConsecutiveBatches, W.fold_consecutive_inputs()), (W.BMMPartition2, W.pattern_inputs("bmm2"))]
+    cases = [(W.FoldConsecutiveBatches, W.fold_consecutive_inputs()), (W.BMMPartition2, W.pattern_inputs("bmm2")),
+             # (max, sum-exp) and (count, mean, M2) states folding consecutive batches / batches modulo 3
+             (W.FoldedLogSumExp, W.fold_consecutive_inputs()), (W.FoldedModuloVariance, W.fold_consecutive_inputs())]
     for cls, inputs in cases:
         gm = W.fuse(cls(), inputs)
         (node,) = fused_nodes(gm)
@@ -278,9 +280,9 @@ def test_batch_folded_row_reductions(two_kernel, monkeypatch):
         outs = list(gm(*[t.cuda() for t in inputs]))
         again = list(gm(*[t.cuda() for t in inputs]))
         refs = evt_oracle.eval_fp32(cls(), inputs)
-        for o, o2, r in zip(outs, again, refs):
+        for i, (o, o2, r) in enumerate(zip(outs, again, refs)):
             assert torch.equal(o, o2)
-            assert evt_oracle.max_rel_err(o, r) <= FP16_TOL
+            assert evt_oracle.max_rel_err(o, r) <= (FP16_TOL if o.dtype != torch.float32 else evt_oracle.REDUCTION_TOL), (cls.__name__, i)
 
 
 def test_launch_is_graph_capturable():
@@ -448,7 +450,11 @@ def test_row_anchor_patterns(name):
         assert torch.allclose(o.float(), e.float(), atol=atol, rtol=1e-2), f"{name} output {k} vs eager"
         stat = o.dtype == torch.float32 and o.numel() * 8 <= inputs[0].numel()      # per-row mean / rstd
         err = evt_oracle.max_rel_err(o, r)
-        assert err <= (REDUCTION_TOL if stat else FP16_TOL), f"{name} output {k}: max rel err {err:.3e}"
+        # the probabilities of a vocabulary-sized softmax lie below fp16's normal range (6.1e-5), where the output
+        # format's spacing is 2^-24 whatever the value: there the bound is the relative one plus half that spacing
+        d, rr = (o.float().cpu() - r).abs(), r.abs()
+        denormal_ok = o.dtype == torch.float16 and bool((d <= FP16_TOL * rr + 2.0 ** -25).all())
+        assert err <= (REDUCTION_TOL if stat else FP16_TOL) or denormal_ok, f"{name} output {k}: max rel err {err:.3e}"
 
 
 @pytest.mark.parametrize("dtype", W.ROW_EDGE_DTYPES, ids=lambda d: str(d).split(".")[-1])
@@ -630,8 +636,8 @@ def test_split_k(cfg, tile, monkeypatch):
     """Few output tiles and a long K: several workgroups share a tile, leave their
     accumulators in the workspace and the last to arrive adds them in split order
     and runs the epilogue (with its own per-row / per-column reductions).  Checked
-    against the oracle with the automatic split, with a forced odd split and with
-    splitting off; repeated launches are bit-identical (the order of the sum is
+    against the oracle with the automatic split, with a forced odd split, with as
+    many splits as there are k-tiles (which meet in two levels) and with splitting off; repeated launches are bit-identical (the order of the sum is
     fixed), and the automatic choice really splits.  With the tuner's tile, a
     ping-pong tile and a one-wave-per-SIMD tile."""
     shapes = W.SPLIT_K_SHAPES[cfg]
@@ -648,7 +654,7 @@ def test_split_k(cfg, tile, monkeypatch):
     (node,) = fused_nodes(gm)
     op = node.target
     results = {}
-    for mode in ("auto", "3", "1"):
+    for mode in ("auto", "3", "40", "1"):     # "40": more than 16 splits meet in groups first (two levels)
         if mode == "auto":
             monkeypatch.delenv("EVT_SPLIT_K", raising=False)
         else:
