@@ -482,6 +482,56 @@ def summarize_traffic(fetch_csv, write_csv, out_path=TRAFFIC_FILE):
     return lines
 
 
+def _short_kernel_name(name):
+    import re
+    m = re.search(r"evt_gemm_kernel<evt::GemmCfg<([^>]*)>", name)
+    if m:
+        return "evt_gemm_kernel<" + m.group(1).replace(" ", "") + ">"
+    m = re.search(r"evt_row_kernel<evt::RowCfg<([^>]*)>.*?, (\d)>", name)
+    if m:
+        return "evt_row_kernel<" + m.group(1).replace(" ", "") + ";fast=" + m.group(2) + ">"
+    m = re.search(r"(evt_\w+_kernel)", name)
+    if m:
+        return m.group(1)
+    if "neg_kernel" in name:
+        return "at::native neg kernel (calibration: 256 MiB in, 256 MiB out)"
+    return name[:76]
+
+
+def summarize_profiles(root):
+    """Text summary of the rocprofv3 output folders under `root`: for every sub-folder that holds a
+    *_kernel_stats.csv (a --kernel-trace --stats run) the calls and average / minimum / maximum duration of each
+    kernel, and for every one that holds a *_counter_collection.csv (a --pmc run) the mean of each counter per
+    dispatch of each kernel of this package (and of the calibration kernel).  No GPU work."""
+    import csv
+    from collections import defaultdict
+    out = [f"# written by `bench.py --profile-summary {root}` from the rocprofv3 CSV files under that folder"]
+    for sub in sorted(p for p in Path(root).iterdir() if p.is_dir()):
+        for stats in sorted(sub.rglob("*_kernel_stats.csv")):
+            out += ["", f"[{sub.name}] kernel trace ({stats.relative_to(root)}): calls, average / minimum / maximum duration in us, share of the run's kernel time",
+                    f"{'kernel':<92} {'calls':>6} {'avg':>9} {'min':>9} {'max':>9} {'%':>6}"]
+            with open(stats, newline="") as f:
+                rows = list(csv.DictReader(f))
+            for r in rows:
+                short = _short_kernel_name(r["Name"])
+                if float(r["Percentage"]) < 0.3 and not short.startswith("evt_"):
+                    continue
+                out.append(f"{short:<92} {r['Calls']:>6} {float(r['AverageNs']) / 1e3:9.2f} {float(r['MinNs']) / 1e3:9.2f} "
+                           f"{float(r['MaxNs']) / 1e3:9.2f} {float(r['Percentage']):6.2f}")
+        for cc in sorted(sub.rglob("*_counter_collection.csv")):
+            vals = defaultdict(list)
+            with open(cc, newline="") as f:
+                for r in csv.DictReader(f):
+                    short = _short_kernel_name(r["Kernel_Name"])
+                    if short.startswith("evt_") or short.startswith("at::native neg"):
+                        vals[(short, int(r["Grid_Size"]), r["Counter_Name"])].append(float(r["Counter_Value"]))
+            out += ["", f"[{sub.name}] counters ({cc.relative_to(root)}): mean per dispatch",
+                    f"{'kernel':<92} {'grid':>9} {'counter':<30} {'n':>6} {'mean':>14}"]
+            for (short, grid, counter), v in sorted(vals.items()):
+                out.append(f"{short:<92} {grid:>9} {counter:<30} {len(v):>6} {sum(v) / len(v):14.6g}")
+    return out
+
+
 def measured_traffic_bytes(key, path=TRAFFIC_FILE):
     """HBM-side bytes per launch of the kernel `key`, scaled by the calibration; None when the file does not hold
     the kernel, or holds it at several grid sizes (then the entry cannot be told apart from here)."""
@@ -526,7 +576,13 @@ def main():
     ap.add_argument("--traffic-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
                     help="no GPU work: condense the counter files of two rocprofv3 --pmc runs of this script "
                          f"(FETCH_SIZE, WRITE_SIZE) into {TRAFFIC_FILE.relative_to(ROOT)} and exit")
+    ap.add_argument("--profile-summary", metavar="DIR", default=None,
+                    help="no GPU work: print a text summary of the rocprofv3 output folders under DIR (kernel statistics "
+                         "and per-dispatch counter means) and exit")
     args = ap.parse_args()
+    if args.profile_summary:
+        print("\n".join(summarize_profiles(args.profile_summary)))
+        return
     if args.traffic_summary:
         print("\n".join(summarize_traffic(*args.traffic_summary)))
         return
