@@ -130,6 +130,68 @@ def spin_up(torch, fn, seconds=0.15):
         torch.cuda.synchronize()
 
 
+class PowerMeter:
+    """Socket power of GPU 0 as the amdgpu driver reports it (hwmon `power1_input`, or `power1_average`, in
+    microwatts; `power1_cap` is the limit the part regulates to), read while a launch loop keeps the GPU busy.
+    Telemetry the box does not expose reads as None; nothing here changes a setting."""
+
+    def __init__(self, torch):
+        import glob
+        self.torch = torch
+        self.path = self.cap_w = None
+        cards = sorted(glob.glob("/sys/class/drm/card*/device"))
+        try:
+            p = torch.cuda.get_device_properties(0)
+            want = "%04x:%02x:%02x." % (getattr(p, "pci_domain_id", 0), p.pci_bus_id, p.pci_device_id)
+            mine = [c for c in cards if os.path.basename(os.path.realpath(c)).startswith(want)]
+        except Exception:
+            mine = []
+        for card in mine or (cards if len(cards) == 1 else []):
+            for hw in sorted(glob.glob(card + "/hwmon/hwmon*")):
+                for name in ("power1_input", "power1_average"):
+                    if self._read(os.path.join(hw, name)) is not None:
+                        self.path = os.path.join(hw, name)
+                        cap = self._read(os.path.join(hw, "power1_cap"))
+                        self.cap_w = None if cap is None else round(cap / 1e6, 1)
+                        return
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return int(f.read().strip())
+        except (OSError, ValueError):
+            return None
+
+    def under_load(self, fn, seconds=2.0, batch=40):
+        """Keep `fn(i)` launches queued for `seconds` (at most two batches ahead of the GPU) and read the power
+        after every batch; the report covers the readings of the second half, when the sensor's average has
+        caught up with the load."""
+        if self.path is None:
+            return None
+        torch = self.torch
+        events, readings, i = [], [], 0
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(batch):
+                fn(i)
+                i += 1
+            ev = torch.cuda.Event()
+            ev.record()
+            events.append(ev)
+            if len(events) > 2:
+                events.pop(0).synchronize()
+            w = self._read(self.path)
+            if w is not None:
+                readings.append((time.perf_counter() - t0, w / 1e6))
+        torch.cuda.synchronize()
+        late = sorted(w for t, w in readings if t >= seconds / 2)
+        if not late:
+            return None
+        return {"socket_w": round(late[len(late) // 2], 1), "socket_w_max": round(late[-1], 1), "cap_w": self.cap_w,
+                "readings": len(late), "seconds": seconds, "source": os.path.basename(self.path)}
+
+
 def time_loop(torch, fn, steps, warmup, repeats=1):
     """ms per call: `steps` back-to-back calls between two HIP events on the launch stream, after a clock
     spin-up and `warmup` untimed calls; the median of `repeats` such regions."""
@@ -573,6 +635,9 @@ def main():
     ap.add_argument("--no-clock-probe", dest="clock_probe", action="store_false",
                     help="skip the diagnostic build of each kernel that reports the shader clock it ran at and "
                          "workgroup 0's main-loop / epilogue split (per_config[*].clock_probe, roofline.shader_mhz)")
+    ap.add_argument("--no-power", dest="power", action="store_false",
+                    help="skip the socket-power readings taken while each config and the MFMA probe run for two seconds "
+                         "(per_config[*].power, roofline.mfma_only.power)")
     ap.add_argument("--traffic-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
                     help="no GPU work: condense the counter files of two rocprofv3 --pmc runs of this script "
                          f"(FETCH_SIZE, WRITE_SIZE) into {TRAFFIC_FILE.relative_to(ROOT)} and exit")
@@ -602,6 +667,7 @@ def main():
         print(json.dumps({"encoder_layer_step": bench_encoder_step(torch, W, only=args.only_encoder_step)}), flush=True)
         return
     cfgs = [int(c) for c in args.configs.split(",")]
+    meter = PowerMeter(torch) if args.power else None
     details = {}
     operand_chunks, tiles = {}, {}
     for cfg in cfgs:
@@ -654,6 +720,8 @@ def main():
             details[cfg]["unfused_addmm_gelu_us"] = round(ms_unf_lib * 1e3, 2)
         if args.clock_probe:
             details[cfg]["clock_probe"] = case.clock_probe(jit)
+        if meter is not None:
+            details[cfg]["power"] = meter.under_load(case.launch)
         log(f"[bench] config {cfg} {wl.name}: {details[cfg]}")
         # 64 Ki elements of each anchor operand, for the register-only MFMA loop below
         operand_chunks[cfg] = tuple(t.reshape(-1)[:1 << 16].clone() for t in case.sets[0][1][:2])
@@ -699,6 +767,13 @@ def main():
         t_zero, mhz_zero = probe.run(torch, torch.zeros_like(rnd))
         mfma_only = {"normal_operands_tflops": round(t_rnd, 1), "normal_operands_shader_mhz": round(mhz_rnd),
                      "zero_operands_tflops": round(t_zero, 1), "zero_operands_shader_mhz": round(mhz_zero)}
+        if meter is not None:
+            # the same loop held for two seconds: what the socket draws with the matrix cores busy on random data,
+            # where the clock falls, and on zeros, where it does not
+            zeros = torch.zeros_like(rnd)
+            mfma_only["power"] = {
+                "normal_operands": meter.under_load(lambda i: probe.run(torch, rnd, warm_launches=0), batch=4),
+                "zero_operands": meter.under_load(lambda i: probe.run(torch, zeros, warm_launches=0), batch=4)}
         # the same loop on chunks of each config's own operands (A-side registers from its left operand, B-side
         # from its right one: activations ~ N(0, 1) against weights ~ N(0, 0.02)), with the 32x32x16 instruction of
         # the fused kernels and with 16x16x32
