@@ -390,7 +390,8 @@ class Codegen:
         tile_stores = [s for s in ir.stores if s.domain == "tile"]
         row_reds = [r for r in ir.reduces.values() if r.axis == "row"]
         col_reds = [r for r in ir.reduces.values() if r.axis == "col"]
-        roots = [s.input for s in tile_stores] + [r.input for r in ir.reduces.values()]
+        vec_stores = [s for s in ir.stores if s.domain == "nvec"]
+        roots = [s.input for s in tile_stores] + [r.input for r in ir.reduces.values()] + [s.input for s in vec_stores]
         need = ir.closure(roots)
         hoisted = [n for n in need if not self.var_m[n]]
         # One-hot row sums (a gather along the row) are collected in a pass of their own, which a wave skips when
@@ -431,6 +432,18 @@ class Codegen:
         # hoisted values
         for name in hoisted:
             self.emit_node(e, ir.nodes[name], hoisted=True)
+        if vec_stores:
+            # one value per column, formed from [N] vectors and scalars alone: written once per batch, by the
+            # lanes that hold row 0
+            e("if (t.row(0, 0) == 0) {")
+            e.indent()
+            for s_ in vec_stores:
+                k = s_.slot
+                e("#pragma unroll")
+                e(f"for (int ni = 0; ni < NI; ++ni) if (t.col_ok(ni)) "
+                  f"evt::st_f32(p.t{k}, bo_{k} + (int64_t)t.col(ni) * p.t{k}_sn, {self.ref(s_.input)});")
+            e.dedent()
+            e("}")
         if onehot:
             self.emit_onehot_vote(e, sorted(set(onehot.values())))
         if col_reds:

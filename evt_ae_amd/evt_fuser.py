@@ -1112,9 +1112,25 @@ class EVTFuser:
         shape, dtype = node_shape_dtype(out)
         if dtype not in DTYPE_NAMES:
             raise NotImplementedError(f"output dtype {dtype}")
+        if out not in self.ir_name or out not in self.coords:
+            # an output no other node of the epilogue reads and that does not depend on the accumulator: its
+            # elements as the accumulator's coordinates see them
+            coord = accum_coord(self.L, self.M, self.N, self.ir.batched).restrict(shape)
+            self.ir_name[out] = self._materialize(out, coord)
+            self.coords.setdefault(out, coord)
         value = self.ir_name[out]
         domain = self.ir.nodes[value].domain
-        if domain not in ("tile", "row", "col"):
+        if domain == "flex":
+            # formed from the epilogue's inputs alone.  One value per column (the reference's row store,
+            # visitor_store.hpp:46-145: BERT's transformed attention mask leaves its first use that way) is
+            # written by the tiles that hold row 0; anything else stays outside
+            st0 = fit_strides(self.coords[out], self.L, self.M, self.N)
+            if (st0 is None or st0.stride_m != 0 or st0.stride_n == 0 or self.M <= 0
+                    or packet(self.anchor.target) in self.row_targets):
+                raise NotImplementedError(
+                    f"output {out.name} does not depend on the accumulator; keep it outside the partition")
+            domain = "nvec"
+        if domain not in ("tile", "row", "col", "nvec"):
             raise NotImplementedError(
                 f"output {out.name} does not depend on the accumulator; keep it outside the partition")
         # find the tensor to materialise: the output itself, or (if its layout
@@ -1149,7 +1165,7 @@ class EVTFuser:
             store_key[key] = name
             self.output2store[name] = name
             self.store_meta[name] = (tuple(sshape), dtype)
-            kind = {"tile": "aux", "row": "col", "col": "row"}[domain]
+            kind = {"tile": "aux", "row": "col", "col": "row", "nvec": "row"}[domain]
             k = self.ir.add_slot(Slot(name, "store", DTYPE_NAMES[dtype], domain, kind, st, tuple(sshape)))
             self.ir.stores.append(Store(k, value, domain))
         if post:

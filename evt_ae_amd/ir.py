@@ -326,7 +326,7 @@ class Slot:
     name: str            # name of the fx node that is loaded / produced
     role: str            # 'load' | 'store'
     dtype: str           # key of DTYPE_CTYPES
-    domain: str          # 'tile' | 'row' | 'col' : where it is accessed
+    domain: str          # 'tile' | 'row' | 'col' : where it is accessed; stores also 'nvec' (see Store)
     kind: str            # loads: 'aux' | 'row' | 'col' | 'scalar' | 'rand' (no storage: generated); stores: 'aux' | 'row' | 'col'
     strides: Strides
     shape: Tuple[int, ...] = ()
@@ -362,7 +362,10 @@ class Reduce:
 class Store:
     slot: int
     input: str
-    domain: str          # 'tile' | 'row' | 'col'
+    # 'tile' | 'row' (one value per row: a reduction along the row) | 'col' (one per column: a reduction over the
+    # rows) | 'nvec' (one per column, formed from [N] vectors and scalars alone: the reference's row store,
+    # visitor_store.hpp:46-145 -- written once per batch by the tiles that hold row 0)
+    domain: str
 
 
 class EpilogueIR:
@@ -484,6 +487,8 @@ class EpilogueIR:
             return False
         if any(n.op == "colidx" for n in self.nodes.values()):
             return False            # there is no row-index value to take its place
+        if any(st.domain == "nvec" for st in self.stores):
+            return False            # a per-column vector store has no per-row counterpart
         for r in self.reduces.values():
             if r.axis == "row" and (r.kind not in ("sum", "max") or r.fold == "div"):
                 return False        # per-column reductions are sums and maxima, folded modulo only
@@ -548,10 +553,10 @@ class EpilogueIR:
                 raise NotImplementedError(f"per-column {r.kind} reduction")
         for s in self.stores:
             have = self.nodes[s.input].domain
-            if have != s.domain:
+            if have != ("flex" if s.domain == "nvec" else s.domain):
                 raise NotImplementedError(
                     f"store of {s.input}: value domain {have} does not match tensor domain {s.domain}")
-        for dom, bad_stride in (("row", "stride_n"), ("col", "stride_m")):
+        for dom, bad_stride in (("row", "stride_n"), ("col", "stride_m"), ("nvec", "stride_m")):
             for name in self.closure([s.input for s in self.stores if s.domain == dom]):
                 n = self.nodes[name]
                 if n.op == "load" and getattr(self.slots[n.slot].strides, bad_stride) != 0:
@@ -594,7 +599,7 @@ class EpilogueIR:
         (tuner_base.py:120-131): aux_load, row_broadcast, column_broadcast,
         aux_store, row_reduction ([N] result), column_reduction ([M] result),
         row_store."""
-        c = {"aux_load": 0, "row": 0, "col": 0, "aux_store": 0, "rowred": 0, "colred": 0}
+        c = {"aux_load": 0, "row": 0, "col": 0, "aux_store": 0, "rowred": 0, "colred": 0, "rowstore": 0}
         for s in self.slots:
             if s.role == "load":
                 if s.kind == "aux":
@@ -606,8 +611,10 @@ class EpilogueIR:
             else:
                 if s.domain == "tile":
                     c["aux_store"] += 1
+                elif s.domain == "nvec":
+                    c["rowstore"] += 1
                 elif s.domain == "col":
                     c["rowred"] += 1      # reference naming: RowReduction -> [N] vector
                 else:
                     c["colred"] += 1      # ColumnReduction -> [M] vector
-        return (c["aux_load"], c["row"], c["col"], c["aux_store"], c["rowred"], c["colred"], 0)
+        return (c["aux_load"], c["row"], c["col"], c["aux_store"], c["rowred"], c["colred"], c["rowstore"])

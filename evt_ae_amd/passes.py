@@ -37,6 +37,9 @@ FUSIBLE_TGT = {
     "detach", "alias", "contiguous", "rand_like",
 }
 _SMALL_SIDE = FUSIBLE_TGT - {"sum", "amax", "mean", "logsumexp", "var_mean", "gather", "one_hot", "getitem"}
+# layout-only and generated values: nothing a kernel would compute once and hand to other kernels
+LAYOUT_SIDE = {"view", "_unsafe_view", "reshape", "unsqueeze", "squeeze", "permute", "clone", "expand", "detach", "alias",
+               "contiguous", "getitem", "rand_like"}
 
 
 def _fusible(node: Node) -> bool:
@@ -119,10 +122,44 @@ def _private_operand_chains(graph_module: GraphModule) -> None:
         graph_module.recompile()
 
 
-def _absorb_side_expressions(anchor: Node, inside: Set[Node], desc: Set[Node], taken: Set[Node]) -> None:
+def _vector_along_n(node: Node) -> bool:
+    """[N], [1, N], [B, 1, N], [B, 1, 1, N]: one value per column (and batch)."""
+    tm = node.meta.get("tensor_meta")
+    if tm is None or not hasattr(tm, "shape"):
+        return False
+    shape = [int(d) for d in tm.shape]
+    if not shape or shape[-1] <= 1:
+        return False
+    middle = shape[1:-1] if len(shape) >= 3 else shape[:-1]
+    return all(d == 1 for d in middle)
+
+
+def _ancestors(nodes: Set[Node], stop: Node) -> Set[Node]:
+    """Everything the `nodes` are computed from, not looking through `stop`."""
+    seen: Set[Node] = set()
+    work = [i for n in nodes for i in n.all_input_nodes if i is not stop]
+    while work:
+        n = work.pop()
+        if n in seen or n is stop:
+            continue
+        seen.add(n)
+        work.extend(n.all_input_nodes)
+    return seen
+
+
+def _absorb_side_expressions(anchor: Node, inside: Set[Node], desc: Set[Node], taken: Set[Node],
+                             shared: Set[Node] = None) -> None:
     """Broadcast-side expressions (e.g. a mask built from a small tensor) whose
     every user is inside the partition join it.  They are not downstream of the
-    anchor, so this cannot close a cycle between partitions."""
+    anchor, so this cannot close a cycle between partitions.
+
+    With `shared` (a set that receives them), a per-column vector that has users
+    outside the partition as well joins it too and leaves the kernel as an
+    output of its own -- the reference's row store (visitor_store.hpp:46-145):
+    BERT's transformed attention mask is computed by the first attention
+    product's kernel and read by the others.  None of its outside users may
+    feed the partition; the caller checks the planned partitions as a whole
+    for cycles."""
     # producers of the anchor's operands inside the partition (layout chains read through strides): what feeds
     # them is the operand's source tensor, never a side expression of the epilogue
     pre: Set[Node] = set()
@@ -146,9 +183,45 @@ def _absorb_side_expressions(anchor: Node, inside: Set[Node], desc: Set[Node], t
                 if all(u in inside for u in i.users):
                     inside.add(i)
                     changed = True
+                elif (shared is not None and _vector_along_n(i) and same_phase(i, anchor)
+                      and target_name(i.target) not in LAYOUT_SIDE
+                      and not any(u in _ancestors(inside | {i}, i) for u in i.users if u not in inside)):
+                    inside.add(i)
+                    shared.add(i)
+                    changed = True
 
 
-def _grow(anchor: Node, taken: Set[Node]) -> List[Node]:
+def _quotient_is_acyclic(graph: Graph, groups: Sequence[Set[Node]]) -> bool:
+    """Do the planned partitions, each taken as one node, leave the graph orderable?"""
+    gid = {}
+    for k, members in enumerate(groups):
+        for n in members:
+            gid[n] = ("p", k)
+    succ, indeg = {}, {}
+    for n in graph.nodes:
+        a = gid.get(n, n)
+        succ.setdefault(a, set())
+        indeg.setdefault(a, 0)
+    for n in graph.nodes:
+        b = gid.get(n, n)
+        for i in n.all_input_nodes:
+            a = gid.get(i, i)
+            if a != b and b not in succ[a]:
+                succ[a].add(b)
+                indeg[b] += 1
+    ready = [a for a, d in indeg.items() if d == 0]
+    done = 0
+    while ready:
+        a = ready.pop()
+        done += 1
+        for b in succ[a]:
+            indeg[b] -= 1
+            if indeg[b] == 0:
+                ready.append(b)
+    return done == len(indeg)
+
+
+def _grow(anchor: Node, taken: Set[Node], shared: Set[Node] = None) -> List[Node]:
     part: List[Node] = _mainloop_permutes(anchor, taken)
     part.append(anchor)
     inside = set(part)
@@ -177,7 +250,7 @@ def _grow(anchor: Node, taken: Set[Node]) -> List[Node]:
                     if u in inside:
                         inside.discard(u)
                         part.remove(u)
-    _absorb_side_expressions(anchor, inside, desc, taken)
+    _absorb_side_expressions(anchor, inside, desc, taken, shared)
     return [n for n in anchor.graph.nodes if n in inside]
 
 
@@ -246,26 +319,37 @@ class Partitioning:
         except NotImplementedError:
             return False
 
-    def plan_greedy(self, graph_module: GraphModule, anchors: List[Node]) -> List[List[str]]:
+    def plan_greedy(self, graph_module: GraphModule, anchors: List[Node], share: bool = True) -> List[List[str]]:
         taken: Set[Node] = set()
         planned: List[List[str]] = []
+        by_name = {n.name: n for n in graph_module.graph.nodes}
+        any_shared = False
         for anchor in anchors:
             if anchor in taken:
                 continue
-            part = _grow(anchor, taken)
+            shared: Set[Node] = set()
+            part = _grow(anchor, taken, shared if share else None)
             names = [n.name for n in part]
+            if shared and not self._accepted(graph_module, names):
+                # the fuser cannot write that vector from this kernel: it stays an input
+                part = _grow(anchor, taken)
+                names = [n.name for n in part]
+                shared = set()
             while EVTFuser.fusible(names, graph_module):
                 if self._accepted(graph_module, names):
                     planned.append(names)
                     taken.update(n for n in part if n.name in names)
+                    any_shared |= bool(shared)
                     break
                 # drop the last epilogue node (never the anchor or its operand permutes)
                 if len(names) - 1 <= names.index(anchor.name):
                     break
                 names = names[:-1]
+        if any_shared and not _quotient_is_acyclic(graph_module.graph, [{by_name[x] for x in names} for names in planned]):
+            return self.plan_greedy(graph_module, anchors, share=False)
         return planned
 
-    def plan_ilp(self, graph_module: GraphModule, anchors: List[Node]) -> List[List[str]]:
+    def plan_ilp(self, graph_module: GraphModule, anchors: List[Node], share: bool = True) -> List[List[str]]:
         from .partitioner import AnchorPartitionILP
         reserved = {}
         for anchor in anchors:
@@ -279,21 +363,35 @@ class Partitioning:
             taken = set(reserved) | set(anchors)
             for s in anchors:
                 taken.update(assign[s])
-            planned, rejected = [], False
+            planned, rejected, any_shared = [], False, False
             for s in anchors:
                 if s in dead:
                     continue
-                inside = {s, *assign[s], *(p for p, a in reserved.items() if a is s)}
-                _absorb_side_expressions(s, inside, ilp._desc[s], taken)
+                base = {s, *assign[s], *(p for p, a in reserved.items() if a is s)}
+                inside, shared = set(base), set()
+                _absorb_side_expressions(s, inside, ilp._desc[s], taken, shared if share else None)
                 names = [n.name for n in order if n in inside]
-                if self._accepted(graph_module, names):
+                ok = self._accepted(graph_module, names)
+                if not ok and shared:
+                    # the fuser cannot write that vector from this kernel: it stays an input
+                    inside, shared = set(base), set()
+                    _absorb_side_expressions(s, inside, ilp._desc[s], taken)
+                    names = [n.name for n in order if n in inside]
+                    ok = self._accepted(graph_module, names)
+                if ok:
                     planned.append(names)
+                    taken.update(shared)         # one kernel writes it, the others read it
+                    any_shared |= bool(shared)
                 elif assign[s]:
                     ilp.ban(assign[s][-1], s)
                     rejected = True
                 else:
                     dead.add(s)
             if not rejected:
+                if any_shared:
+                    by_name = {n.name: n for n in order}
+                    if not _quotient_is_acyclic(graph_module.graph, [{by_name[x] for x in names} for names in planned]):
+                        return self.plan_ilp(graph_module, anchors, share=False)
                 self.ilp = ilp
                 return planned
         raise RuntimeError("partitioning did not settle: the fuser kept turning partitions down")

@@ -1006,6 +1006,57 @@ def pattern_inputs(name: str, seed: int = 0) -> List[torch.Tensor]:
 
 
 # ---------------------------------------------------------------------------
+# A per-column vector computed in an epilogue and read by other kernels (the reference's row store,
+# visitor_store.hpp:46-145): BERT turns its attention mask into (1 - mask) * -10000 once; the first attention
+# product's kernel computes and writes it, the later ones load it.
+# ---------------------------------------------------------------------------
+
+class MaskedScores(torch.nn.Module):
+    """scores[B*H, S, S] = q k^T / 8 + (1 - mask[B, 1, 1, S]) * -10000; the transformed mask is an output too."""
+    DIMS = (2, 3, 40, 16)
+    GPU_DIMS = ((2, 3, 40, 16), (2, 2, 264, 64), (3, 2, 512, 64))     # unaligned; several row tiles, ragged; aligned
+
+    def __init__(self, dims=None):
+        super().__init__()
+        self.B, self.H, self.S, self.D = dims or self.DIMS
+
+    def forward(self, q, k, mask):
+        B, H, S = self.B, self.H, self.S
+        ext = aten.mul(aten.rsub(mask, 1.0), -10000.0)
+        sc = aten.view(aten.bmm(q, aten.permute(k, [0, 2, 1])), [B, H, S, S])
+        sc = aten.add(aten.div(sc, 8.0), ext)
+        return aten.view(sc, [B * H, S, S]), ext
+
+    @classmethod
+    def inputs(cls, seed=0, dims=None):
+        g = torch.Generator().manual_seed(seed)
+        B, H, S, D = dims or cls.DIMS
+        q = torch.randn(B * H, S, D, generator=g).half()
+        k = torch.randn(B * H, S, D, generator=g).half()
+        mask = (torch.rand(B, 1, 1, S, generator=g) > 0.3).half()
+        return [q, k, mask]
+
+
+class TwoMaskedLayers(torch.nn.Module):
+    """Two products that add the same transformed [N] mask: one kernel writes it, the other reads it."""
+
+    def forward(self, x, w1, w2, mask):
+        ext = aten.mul(aten.rsub(mask, 1.0), -100.0)
+        h = aten.relu(aten.add(aten.mm(x, w1), ext))
+        y = aten.add(aten.mm(h, w2), ext)
+        return y
+
+    @staticmethod
+    def inputs(seed=0, m=72, n=48):
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(m, n, generator=g).half()
+        w1 = (torch.randn(n, n, generator=g) * n ** -0.5).half()
+        w2 = (torch.randn(n, n, generator=g) * n ** -0.5).half()
+        mask = (torch.rand(n, generator=g) > 0.3).half()
+        return [x, w1, w2, mask]
+
+
+# ---------------------------------------------------------------------------
 # The reference's tuner caches as a coverage checklist (tests/golden/reference_tuner_keys.json): every GEMM / BMM
 # problem key there names a shape, a layout pair and seven epilogue-node counts
 # (python/gtl/compiler/autotuner/tuner_base.py:107-152).  `CountedEpilogue` is a synthetic epilogue with exactly
@@ -1017,9 +1068,10 @@ class CountedEpilogue(torch.nn.Module):
     stores x, gelu(x), relu(x) ... (aux_store of them), sums over the rows of x,
     x * x ... (row_reduction of them: [N] results, fp32) and sums along the rows
     (column_reduction: [M] results, fp32).  row_store: a value of the [N]
-    vectors alone (the reference stores the transformed attention mask that
-    way, visitor_store.hpp:46-145); it does not depend on the product, so this
-    backend leaves it to an eager kernel outside the fused one.
+    vectors alone that the epilogue uses and that leaves the kernel as well
+    (the reference stores BERT's transformed attention mask that way,
+    (1 - mask) * -10000: visitor_store.hpp:46-145): the first row_store row
+    vectors enter x in that form, and the transformed vectors are outputs.
     forward(A, B, *aux, *rowvec, *colvec)."""
 
     def __init__(self, counts, a_row: bool, b_row: bool, batched: bool):
@@ -1050,7 +1102,8 @@ class CountedEpilogue(torch.nn.Module):
         for _ in range(aux):
             x = aten.add(x, extra.pop(0))
         rows = [extra.pop(0) for _ in range(rowb)]
-        for r in rows:
+        masks = [aten.mul(aten.rsub(r, 1.0), -10000.0) for r in rows[:rowstore]]
+        for r in masks + rows[len(masks):]:
             x = aten.add(x, r)
         for _ in range(colb):
             x = aten.mul(x, extra.pop(0))
@@ -1068,8 +1121,7 @@ class CountedEpilogue(torch.nn.Module):
             for j in range(colred):
                 outs.append(aten.sum(power, [-1]))
                 power = aten.mul(power, xf)
-        for j in range(rowstore):
-            outs.append(aten.mul(rows[j % len(rows)], -10000.0))
+        outs.extend(masks)
         return tuple(outs)
 
 

@@ -26,6 +26,10 @@ def register_tests() -> None:
                                                device="meta") for t in _shapes_of(1, W.SMALL_SHAPES[1])])
     for name, (cls, _) in W.RANDOM_PATTERNS.items():
         W.fuse(cls(), _meta(W.pattern_inputs(name)))
+    for dims in W.MaskedScores.GPU_DIMS:
+        W.fuse(W.MaskedScores(dims), _meta(W.MaskedScores.inputs(dims=dims)))
+    W.fuse(W.TwoMaskedLayers(), _meta(W.TwoMaskedLayers.inputs()))
+    W.fuse(W.TwoMaskedLayers(), _meta(W.TwoMaskedLayers.inputs(m=1000, n=520)))
     W.fuse(W.FoldConsecutiveBatches(), _meta(W.fold_consecutive_inputs()))
     W.fuse(W.FoldedLogSumExp(), _meta(W.fold_consecutive_inputs()))
     W.fuse(W.FoldedModuloVariance(), _meta(W.fold_consecutive_inputs()))

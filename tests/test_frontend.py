@@ -538,3 +538,48 @@ def test_walk_tiles_are_offered_and_refused_where_they_should(monkeypatch):
     assert "_n4_kx" in node.target.module.name
     with pytest.raises(NotImplementedError):           # a module that must also take a K with a partial k-tile
         jit.LazyModule(node.target.ir, replace(node.target.spec, k_exact=False))
+
+
+def test_a_vector_of_the_epilogue_leaves_the_kernel_as_a_row_store():
+    """(1 - mask) * -10000 feeds the scores and is an output of its own: the kernel computes it per column, adds
+    it, and the tiles that hold row 0 write it (one store per batch row of the mask, l // H)."""
+    inputs = W.MaskedScores.inputs()
+    gm = _check(W.MaskedScores, inputs)
+    (node,) = fused_nodes(gm)
+    ir = node.target.ir
+    assert ir.epilogue_counts() == (0, 1, 0, 1, 0, 0, 1)
+    (vec,) = [sl for sl in ir.slots if sl.role == "store" and sl.domain == "nvec"]
+    assert (vec.strides.stride_m, vec.strides.stride_n, vec.strides.l_div) == (0, 1, W.MaskedScores.DIMS[1])
+    assert not any(n.op == "call_function" and n.target in (aten.mul, aten.rsub) for n in gm.graph.nodes)
+    assert "t.row(0, 0) == 0" in node.target.module.source
+
+
+def test_one_kernel_writes_a_shared_vector_and_the_next_reads_it():
+    inputs = W.TwoMaskedLayers.inputs()
+    gm = _check(W.TwoMaskedLayers, inputs, n_fused=2)
+    first, second = fused_nodes(gm)
+    assert first.target.ir.epilogue_counts()[6] == 1 and second.target.ir.epilogue_counts()[6] == 0
+    # the second kernel's row vector is the first one's output
+    src = [a for a in second.args if isinstance(a, torch.fx.Node) and a.op == "call_function"]
+    assert any(first in (a, *a.all_input_nodes, *(i for b in a.all_input_nodes for i in b.all_input_nodes)) for a in src)
+    assert not any(n.op == "call_function" and n.target in (aten.mul, aten.rsub) for n in gm.graph.nodes)
+
+
+def test_a_vector_that_feeds_the_partition_through_its_other_users_stays_outside():
+    """If another user of the side expression is an ancestor of the partition, writing it from the kernel would
+    close a cycle: it stays an eager node."""
+    class Loop(torch.nn.Module):
+        def forward(self, x, w, mask):
+            ext = aten.mul(aten.rsub(mask, 1.0), -100.0)
+            x2 = aten.add(x, ext)                    # reads ext and feeds the product
+            return aten.add(aten.mm(x2, w), ext)
+    g = torch.Generator().manual_seed(3)
+    inputs = [torch.randn(40, 32, generator=g).half(), (torch.randn(32, 32, generator=g) * 0.2).half(),
+              (torch.rand(32, generator=g) > 0.5).half()]
+    gm = W.fuse(Loop(), inputs)
+    (node,) = fused_nodes(gm)
+    assert node.target.ir.epilogue_counts()[6] == 0
+    assert any(n.op == "call_function" and n.target is aten.mul for n in gm.graph.nodes)
+    # the eager nodes in front of the product round to fp16, which the product amplifies: a loose bound
+    (got,), (ref,) = run_emulated(gm, inputs), evt_oracle.eval_fp32(Loop(), inputs)
+    assert evt_oracle.max_rel_err(got.float(), ref) <= 5e-2

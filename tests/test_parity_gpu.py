@@ -387,6 +387,43 @@ def test_multi_anchor_graphs(name):
         assert err <= (REDUCTION_TOL if red else FP16_TOL), f"{name} output {k}: max rel err {err:.3e}"
 
 
+@pytest.mark.parametrize("dims", W.MaskedScores.GPU_DIMS, ids=lambda d: "x".join(map(str, d)))
+def test_row_store_of_a_shared_mask(dims):
+    """BERT's transformed attention mask, (1 - mask[B, 1, 1, S]) * -10000, is computed in the epilogue of the
+    scores' product, added there, and written by the tiles that hold row 0 (the reference's row store,
+    visitor_store.hpp:46-145): both outputs against the oracle, the stored vector exactly (one fp16 rounding of
+    an exact value), and nothing but the fused kernel left in the graph."""
+    inputs = W.MaskedScores.inputs(seed=5, dims=dims)
+    mod = W.MaskedScores(dims)
+    gm = W.fuse(mod, inputs)
+    (node,) = fused_nodes(gm)
+    assert node.target.ir.epilogue_counts() == (0, 1, 0, 1, 0, 0, 1)
+    scores, ext = gm(*[t.cuda() for t in inputs])
+    torch.cuda.synchronize()
+    ref_scores, ref_ext = evt_oracle.eval_fp32(mod, inputs)
+    assert tuple(ext.shape) == tuple(ref_ext.shape) and ext.dtype == torch.float16
+    assert torch.equal(ext.cpu().float(), ref_ext.float())
+    err = evt_oracle.max_rel_err(scores, ref_scores)
+    assert err <= FP16_TOL, err
+    again_scores, again_ext = gm(*[t.cuda() for t in inputs])
+    torch.cuda.synchronize()
+    assert torch.equal(again_scores, scores) and torch.equal(again_ext, ext)
+
+
+@pytest.mark.parametrize("m,n", [(72, 48), (1000, 520)])
+def test_one_kernel_writes_a_vector_the_next_one_reads(m, n):
+    inputs = W.TwoMaskedLayers.inputs(seed=2, m=m, n=n)
+    gm = W.fuse(W.TwoMaskedLayers(), inputs)
+    first, second = fused_nodes(gm)
+    assert first.target.ir.epilogue_counts()[6] == 1 and second.target.ir.epilogue_counts()[6] == 0
+    out = gm(*[t.cuda() for t in inputs])
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    torch.cuda.synchronize()
+    (ref,) = evt_oracle.eval_fp32(W.TwoMaskedLayers(), inputs)
+    err = evt_oracle.max_rel_err(out, ref)
+    assert err <= FP16_TOL, err
+
+
 @pytest.mark.parametrize("entry", ["aot_module", "torch.compile"])
 def test_aot_training_step(entry):
     """A whole training step through AOT autograd, as the reference's model tests

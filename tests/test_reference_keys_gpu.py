@@ -6,7 +6,8 @@
   * `736389_64_128_h_h_R_C_0_1_0_1_0_0_0`     odd M, 2877 or more row tiles, one narrow column tile;
   * `16384_1024_30528_h_h_R_R_1_0_2_1_2_0_0`  K = 30528, two [M] vectors, two per-column reductions;
   * `64_64_736389_h_h_C_R_0_0_0_1_0_0_0`      one output tile, K = 736389 (odd: a K tail in the last k-tile);
-  * `512_512_512_64_h_h_R_R_0_1_0_1_0_0_1`    the batched key with a row store (kept outside the fused kernel).
+  * `512_512_512_64_h_h_R_R_0_1_0_1_0_0_1`    the batched key with a row store ([N] values the epilogue forms, uses
+    and writes from the tiles that hold row 0).
 
 The oracle (PyTorch fp32 on the CPU, oracle/evt_oracle.py) is evaluated on the same inputs restricted to sampled
 rows / columns -- first and last tiles, the columns on either side of the 2^31-byte boundary -- where the whole
@@ -169,11 +170,12 @@ def test_one_tile_with_an_odd_k_of_736389():
     assert torch.equal(out, again)
 
 
-def test_batched_key_with_a_row_store_outside_the_kernel():
+def test_batched_key_with_a_row_store():
     key = "512_512_512_64_h_h_R_R_0_1_0_1_0_0_1"
     case = W.parse_reference_key(key, True); case["batched"] = True
     inputs = _inputs(case, 15)
     mod, gm, op = _fused(case, inputs)
+    assert op.ir.epilogue_counts() == case["counts"]
     out, rowvec = gm(*inputs)
     torch.cuda.synchronize()
     ref_out, ref_vec = evt_oracle.eval_fp32(mod, [t.cpu() for t in inputs])
