@@ -1,5 +1,7 @@
-"""The extreme problems of the reference's tuner caches at their real sizes
-(tests/golden/reference_tuner_keys.json), one launch each through the C ABI:
+"""The problems of the reference's tuner caches at their real sizes
+(tests/golden/reference_tuner_keys.json), one launch each through the C ABI: every GEMM / BMM key and every
+softmax / layer norm problem against the oracle (the tests at the end of this file), and the extreme ones with
+checks of their own:
 
   * `2048_670208_512_h_h_R_C_1_1_0_1_1_0_0`  a 2.75 GB fp16 output and a 2.75 GB residual (byte offsets past
     2^31), a [N] vector, a per-column sum over 8 row tiles;
@@ -181,3 +183,105 @@ def test_batched_key_with_a_row_store():
     ref_out, ref_vec = evt_oracle.eval_fp32(mod, [t.cpu() for t in inputs])
     _check("scores", out, ref_out, False)
     _check("row store", rowvec, ref_vec, False)
+
+
+# ---------------------------------------------------------------------------
+# every GEMM / BMM key of the catalogue at its real size
+# ---------------------------------------------------------------------------
+
+_ALL_KEYS = [(table, key) for table, key, _ in W.reference_key_cases()]
+
+
+def _split_outputs(counts, outs):
+    """CountedEpilogue's outputs by kind: ([M, N] stores, [N] sums over the rows, [M] sums along the rows, [N] masks)."""
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    a, b, c = counts[3], counts[3] + counts[4], counts[3] + counts[4] + counts[5]
+    return outs[:a], outs[a:b], outs[b:c], outs[c:]
+
+
+@pytest.mark.parametrize("table,key", _ALL_KEYS, ids=[k for _, k in _ALL_KEYS])
+def test_every_reference_key_at_its_size(table, key):
+    """One launch per key of the reference's tuner caches, on the problem size the key names, against the oracle:
+    on the whole problem where that is at most 2e10 flop, else on sampled rows (all columns: the stores and the
+    sums along the rows) and sampled columns (all rows: the stores and the sums over the rows), first and last
+    tiles included."""
+    batched = table == "best_config_bmm"
+    case = W.parse_reference_key(key, batched); case["batched"] = batched
+    counts = case["counts"] or (0, 0, 0, 1, 0, 0, 0)
+    L, M, N, K = case["L"], case["M"], case["N"], case["K"]
+    lead = 1 if batched else 0
+    inputs = _inputs(case, 100 + len(key))
+    mod, gm, op = _fused(case, inputs)
+    assert op.ir.epilogue_counts() == tuple(counts), key
+    outs = gm(*inputs)
+    torch.cuda.synchronize()
+    stores, over_rows, along_rows, masks = _split_outputs(counts, outs)
+    if 2.0 * L * M * N * K <= 2e10:
+        refs = _split_outputs(counts, evt_oracle.eval_fp32(mod, [t.cpu() for t in inputs]))
+        for kind, got, ref in zip(("store", "sum over rows", "sum along rows", "row store"), (stores, over_rows, along_rows, masks), refs):
+            for j, (o, r) in enumerate(zip(got, ref)):
+                _check(f"{key} {kind} {j}", o, r, kind.startswith("sum"))
+        return
+    g = torch.Generator().manual_seed(len(key))
+    rows = torch.unique(torch.cat([torch.tensor([0, 1, M - 1]), torch.randint(0, M, (9,), generator=g)])).cuda()
+    cols = torch.unique(torch.cat([torch.arange(0, 4), torch.arange(N - 4, N), torch.randint(0, N, (16,), generator=g)])).cuda()
+    r_stores, _, r_along, r_masks = _split_outputs(counts, evt_oracle.eval_fp32(mod, _restrict(case, inputs, rows=rows)))
+    for j, (o, r) in enumerate(zip(stores, r_stores)):
+        _check(f"{key} store {j} rows", o.index_select(lead, rows), r, False)
+    for j, (o, r) in enumerate(zip(along_rows, r_along)):
+        _check(f"{key} sum along rows {j}", o.index_select(lead, rows), r, True)
+    for j, (o, r) in enumerate(zip(masks, r_masks)):
+        _check(f"{key} row store {j}", o, r, False)
+    c_stores, c_over, _, _ = _split_outputs(counts, evt_oracle.eval_fp32(mod, _restrict(case, inputs, cols=cols)))
+    for j, (o, r) in enumerate(zip(stores, c_stores)):
+        _check(f"{key} store {j} columns", o.index_select(lead + 1, cols), r, False)
+    for j, (o, r) in enumerate(zip(over_rows, c_over)):
+        _check(f"{key} sum over rows {j}", o.index_select(lead, cols), r, True)
+
+
+_ROW_KEYS = W.reference_row_key_cases()
+
+
+@pytest.mark.parametrize("case", _ROW_KEYS, ids=[f"{c[1]}-{c[2]}x{c[3]}" for c in _ROW_KEYS])
+def test_every_reference_row_key_at_its_size(case):
+    """The softmax / layer norm problems of the reference's tuner caches (2 columns to 30528, 32 rows to 736392) on
+    the row-wise kernels at their real size.  Rows do not interact in these anchors, so the oracle is evaluated
+    on the first and last 64 rows and 1000 random ones."""
+    key, anchor, rows, cols, mod, metas = case
+    g = torch.Generator(device="cuda").manual_seed(rows % 9973 + cols)
+    half = torch.float16
+
+    def randn():
+        t = torch.empty((rows, cols), dtype=half, device="cuda")
+        flat, step = t.view(-1), 1 << 28
+        for lo in range(0, flat.numel(), step):
+            n = min(step, flat.numel() - lo)
+            flat[lo:lo + n] = torch.randn(n, generator=g, device="cuda").to(half)
+        return t
+    x = randn()
+    if anchor == "softmax":
+        inputs = [x]
+    elif anchor == "softmax_backward":
+        inputs = [randn(), torch.softmax(x.float(), -1).to(half)]
+    elif anchor == "layernorm":
+        inputs = [x]
+    else:
+        var, mean = torch.var_mean(x.float(), -1, unbiased=False, keepdim=True)
+        inputs = [randn(), x, mean, torch.rsqrt(var + 1e-5)]
+    gm = W.fuse(mod, [t.to("meta") for t in inputs])
+    (node,) = fused_nodes(gm)
+    outs = gm(*inputs)
+    outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+    torch.cuda.synchronize()
+    pick = torch.Generator().manual_seed(cols)
+    idx = torch.unique(torch.cat([torch.arange(0, min(64, rows)), torch.arange(max(rows - 64, 0), rows),
+                                  torch.randint(0, rows, (1000,), generator=pick)])).cuda()
+    refs = evt_oracle.eval_fp32(mod, [t.index_select(0, idx).cpu() for t in inputs])
+    assert len(refs) == len(outs)
+    for j, (o, r) in enumerate(zip(outs, refs)):
+        got = o.index_select(0, idx).cpu()
+        ok, err = evt_oracle.check(got, r, reduction=o.dtype == torch.float32)
+        # the probabilities of a vocabulary-sized softmax lie below fp16's normal range (6.1e-5), where the output
+        # format's spacing is 2^-24 whatever the value: there the bound is the relative one plus half that spacing
+        denormal_ok = o.dtype == half and bool(((got.float() - r).abs() <= 2e-2 * r.abs() + 2.0 ** -25).all())
+        assert ok or denormal_ok, (key, anchor, j, err)
