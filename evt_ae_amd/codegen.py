@@ -940,13 +940,14 @@ class Codegen:
                 e("if (a->K & 7) return EVT_ERR_ALIGNMENT;")
                 e("if ((int64_t)Cfg::BM * a->lda * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
             else:
-                e("if (a->M & 7) return EVT_ERR_ALIGNMENT;")
+                e("// whole 8-element chunks are read along M: rows padded to a multiple of 8 make room for the last one")
+                e("if ((a->M & 7) && a->lda < ((a->M + 7) & ~(int64_t)7)) return EVT_ERR_ALIGNMENT;")
                 e("if ((int64_t)Cfg::BK * a->lda * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
             if sp.b_kc:
                 e("if (a->K & 7) return EVT_ERR_ALIGNMENT;")
                 e("if ((int64_t)Cfg::BN * a->ldb * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
             else:
-                e("if (a->N & 7) return EVT_ERR_ALIGNMENT;")
+                e("if ((a->N & 7) && a->ldb < ((a->N + 7) & ~(int64_t)7)) return EVT_ERR_ALIGNMENT;")
                 e("if ((int64_t)Cfg::BK * a->ldb * 2 >= 0x7fffffffLL) return EVT_ERR_RANGE;")
         for k, s in enumerate(ir.slots):
             ct = DTYPE_CTYPES[s.dtype]

@@ -211,6 +211,7 @@ class FusedOpBase:
         next call; a caller that keeps several argument sets side by side
         passes a block of its own (`new_argument_block()`) for each."""
         M, N, K, L = self.problem
+        K = getattr(self, "kernel_k", K)         # operands padded along K (FusedGEMM.pad)
         A, lda, bsa, B, ldb, bsb = self.operands(args[-2], args[-1])
         a = block if block is not None else self.argument_block()
         a.M, a.N, a.K, a.L = M, N, K, L
@@ -481,6 +482,7 @@ class FusedGEMM(FusedOpBase):
     __name__ = "cutlass_gemm_with_visitor"
     target = aten.mm
     mainloop_fusion_targets = [aten.permute]
+    pad_min_flops = 1e9          # products below this keep the element-wise path: the copies would cost more
 
     def __init__(self, node: Node, epilogue_visitor: "EVTFuser") -> None:
         super().__init__(node, epilogue_visitor)
@@ -512,13 +514,25 @@ class FusedGEMM(FusedOpBase):
         self.lda = K if self.a_kc else M
         self.ldb = K if self.b_kc else N
         dma = _dma_ok(self.a_kc, self.b_kc, M, N, K, self.lda, self.ldb, 0, 0)
+        # Extents that break the transfer path's 16-byte rule (ViT's patch embedding: K = 588) would fall back to the
+        # element-wise path, several times slower.  A product large enough to pay for two copy kernels runs on
+        # zero-padded copies of its operands instead: rows padded to a multiple of 8 elements, K to a multiple of 8
+        # (zero columns / rows add nothing to the product; the output keeps its M and N).
+        self.pad = None
+        if not dma and 2.0 * M * N * K >= self.pad_min_flops:
+            r8 = lambda v: (v + 7) & ~7      # noqa: E731
+            Kp = r8(K) if (self.a_kc or self.b_kc) else K
+            self.pad = (Kp, Kp if self.a_kc else r8(M), Kp if self.b_kc else r8(N))
+            self.kernel_k, self.lda, self.ldb = self.pad
+            dma = True
+            K = Kp
 
         self.align_A = self.get_alignment(K if self.a_kc else M)
         self.align_B = self.get_alignment(K if self.b_kc else N)
         self.align_C = self.get_alignment(N)
 
         with (_pop_mode_temporarily() if _len_torch_dispatch_stack() > 0 else nullcontext()):
-            tuner = MMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
+            tuner = MMTuner((M, N, K, 1), self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
             tile = tuner.get_best_config()
             self.tile = tile
             self.spec = KernelSpec.for_problem(K, self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
@@ -527,6 +541,19 @@ class FusedGEMM(FusedOpBase):
     def operands(self, A, B):
         A = A.contiguous()
         B = B.contiguous()
+        if self.pad is not None:
+            M, N, K, _ = self.problem
+            Kp, lda, ldb = self.pad
+            pad = torch.nn.functional.pad
+            # (last-axis padding, then rows): one copy kernel per operand that needs it
+            if self.a_kc:
+                A = pad(A, (0, lda - K)) if lda != K else A
+            elif lda != M or Kp != K:
+                A = pad(A, (0, lda - M, 0, Kp - K))
+            if self.b_kc:
+                B = pad(B, (0, ldb - K)) if ldb != K else B
+            elif ldb != N or Kp != K:
+                B = pad(B, (0, ldb - N, 0, Kp - K))
         if self.tile.dma:
             # the global->LDS path moves 16-byte chunks: a contiguous view that starts at an odd storage offset is
             # copied into a fresh (aligned) allocation instead of failing the launch, as eager would simply work

@@ -90,6 +90,15 @@ typedef struct EvtTensorArg {
  * dimensions of each operand is contiguous is a compile-time property of the
  * module (see evt_module_spec).  `lda`/`ldb` are the strides, in elements, of
  * the non-contiguous dimension; batch strides are in elements and may be 0.
+ * Modules with "tile"."dma": true in their spec move 16-byte chunks: A, B, lda, ldb
+ * and the batch strides must be multiples of 8 elements (16 bytes), and so
+ * must K where an operand is contiguous along K.  An operand that is
+ * contiguous along M (A) or N (B) is read in whole chunks of 8 along that
+ * dimension: if M (N) is not a multiple of 8, lda (ldb) must be at least M (N)
+ * rounded up to 8 and every row, the last one included, readable to that
+ * extent (what lies there does not reach the output).  Anything else is
+ * refused with EVT_ERR_ALIGNMENT; modules with "tile"."dma": false take any
+ * alignment.
  * Replaces GemmArguments / BmmArguments2x (evt_fuser.py:539-544, bmm.py:23-64).
  *
  * Row-wise modules (module spec has "anchor": softmax, softmax_backward,

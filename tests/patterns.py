@@ -1125,6 +1125,22 @@ class CountedEpilogue(torch.nn.Module):
         return tuple(outs)
 
 
+# products whose extents break the 16-byte rule of the transfer path, run on zero-padded copies of their operands
+# (FusedGEMM.pad): (M, N, K, A row-major, B row-major, the seven epilogue counts)
+PADDED_GEMM_CASES = [
+    (203, 141, 589, True, True, (1, 1, 0, 1, 1, 1, 0)),
+    (203, 141, 589, True, False, (0, 1, 1, 2, 0, 1, 0)),
+    (203, 141, 589, False, True, (1, 0, 0, 1, 1, 0, 0)),
+    (203, 141, 589, False, False, (0, 1, 0, 1, 0, 0, 0)),
+    (520, 588, 1028, True, True, (0, 1, 0, 1, 1, 0, 0)),
+]
+
+
+def padded_gemm_case(i):
+    M, N, K, a_row, b_row, counts = PADDED_GEMM_CASES[i]
+    return dict(L=1, M=M, N=N, K=K, a_row=a_row, b_row=b_row, counts=counts, batched=False)
+
+
 def parse_reference_key(key: str, batched: bool):
     """`M_N_K_h_h_R_C[_7 counts]` (`L_M_N_K_...` batched) -> dict(L, M, N, K, a_row, b_row, counts), counts None for
     the keys of the reference tuner's first stage (no epilogue: a plain store)."""

@@ -116,6 +116,14 @@ def register_tests() -> None:
         W.fuse(*W.counted_epilogue(case))
     for _key, _anchor, _rows, _cols, mod, metas in W.reference_row_key_cases():
         W.fuse(mod, metas)
+    from evt_ae_amd.evt_fuser import FusedGEMM
+    floor = FusedGEMM.pad_min_flops
+    try:
+        for FusedGEMM.pad_min_flops in (0.0, float("inf")):      # padded operands, and the element-wise path
+            for i in range(len(W.PADDED_GEMM_CASES)):
+                W.fuse(*W.counted_epilogue(W.padded_gemm_case(i)))
+    finally:
+        FusedGEMM.pad_min_flops = floor
     for name, (cls, _) in W.REFERENCE_PATTERNS.items():
         if name in ("mm10", "mm11"):      # shapes only: their inputs are large
             shapes = {"mm10": [(16384, 1024), (1024, 4096)], "mm11": [(33792, 768), (33792, 768)]}[name]

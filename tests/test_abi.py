@@ -111,6 +111,11 @@ def test_argument_validation_happens_before_launch(module):
     assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -2    # EVT_ERR_ALIGNMENT
     bad = _args(op, km); bad.lda += 1
     assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -2
+    # B is contiguous along N and read in whole chunks of 8: an N that is no multiple of 8 needs rows padded to one
+    bad = _args(op, km); bad.N -= 4
+    assert km.lib.evt_workspace_bytes(ctypes.byref(bad)) >= 0            # ldb still has room for the last chunk
+    bad.ldb = bad.N + 4 - 8
+    assert km.lib.evt_workspace_bytes(ctypes.byref(bad)) == -2
     bad = _args(op, km); bad.tensors[0].l_div = 0
     assert km.lib.evt_launch(ctypes.byref(bad), None, 0, None) == -1
     bad = _args(op, km); bad.tensors[0].l_mod = -3

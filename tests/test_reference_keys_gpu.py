@@ -285,3 +285,33 @@ def test_every_reference_row_key_at_its_size(case):
         # format's spacing is 2^-24 whatever the value: there the bound is the relative one plus half that spacing
         denormal_ok = o.dtype == half and bool(((got.float() - r).abs() <= 2e-2 * r.abs() + 2.0 ** -25).all())
         assert ok or denormal_ok, (key, anchor, j, err)
+
+
+@pytest.mark.parametrize("i", range(len(W.PADDED_GEMM_CASES)), ids=lambda i: "_".join(map(str, W.PADDED_GEMM_CASES[i][:5])))
+def test_misaligned_extents_run_on_padded_operands(i, monkeypatch):
+    """Odd M, N and K in every operand layout: the fused op copies its operands into zero-padded buffers and runs
+    the transfer-path kernel (ViT's K = 588 patch embedding takes this route at its real size); outputs, sums over
+    the rows and along the rows against the oracle -- the padding must not reach any of them."""
+    from evt_ae_amd.evt_fuser import FusedGEMM
+    monkeypatch.setattr(FusedGEMM, "pad_min_flops", 0.0)
+    case = W.padded_gemm_case(i)
+    inputs = _inputs(case, 40 + i)
+    mod, gm, op = _fused(case, inputs)
+    assert op.pad is not None and op.tile.dma and (op.kernel_k % 8 == 0 or not (op.a_kc or op.b_kc))
+    outs = gm(*inputs)
+    torch.cuda.synchronize()
+    counts = case["counts"]
+    got = _split_outputs(counts, outs)
+    ref = _split_outputs(counts, evt_oracle.eval_fp32(mod, [t.cpu() for t in inputs]))
+    for kind, gs, rs in zip(("store", "sum over rows", "sum along rows", "row store"), got, ref):
+        for j, (o, r) in enumerate(zip(gs, rs)):
+            assert tuple(o.shape) == tuple(r.shape)
+            _check(f"{kind} {j}", o, r, kind.startswith("sum"))
+    # the same product on the element-wise path gives the same values up to the order of the K sum
+    monkeypatch.setattr(FusedGEMM, "pad_min_flops", float("inf"))
+    _, gm2, op2 = _fused(case, inputs)
+    assert op2.pad is None and not op2.tile.dma
+    outs2 = gm2(*inputs)
+    torch.cuda.synchronize()
+    for o, o2 in zip(outs if isinstance(outs, (tuple, list)) else [outs], outs2 if isinstance(outs2, (tuple, list)) else [outs2]):
+        assert evt_oracle.max_rel_err(o, o2.float().cpu()) <= 2e-2

@@ -90,7 +90,7 @@ def fake_argument_block(op: FusedOpBase):
     from evt_ae_amd.evt_fuser import FusedRowOp
     a = op.new_argument_block()
     M, N, K, L = op.problem
-    a.M, a.N, a.K, a.L = M, N, K, L
+    a.M, a.N, a.K, a.L = M, N, getattr(op, "kernel_k", K), L
     a.A, a.B = 0x7000_0000_0000, 0x7100_0000_0000
     if isinstance(op, FusedRowOp):
         a.lda = a.ldb = N
