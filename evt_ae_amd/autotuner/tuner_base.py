@@ -163,6 +163,15 @@ class AutoTunerBase:
                        # under the other's main loop (measured 1.36 x over one per CU on the classifier problem,
                        # where the ping-pong tiles that walk still win)
                        (128, 256, 32, 2, 2, 3, 12), (256, 128, 32, 4, 1, 3, 12), (128, 128, 64, 2, 2, 2, 12)]
+            # narrow outputs (GCN's 736389 x 64 products): a tile wider than the problem leaves every tile partial,
+            # which costs the epilogue its check-free path and the main loop half its MFMAs; measured on
+            # 736389 x 64 x 64 with two residual loads 459 us on 256 x 128 tiles, 61 us on 128 x 64
+            if self.N <= 64 or self.N % 128 == 64:
+                shapes += [(128, 64, 64, 4, 1, 2, 0), (128, 64, 64, 2, 2, 2, 0), (256, 64, 64, 4, 1, 2, 0),
+                           (256, 64, 64, 4, 2, 2, 0)]
+            if self.M <= 64 or self.M % 128 == 64:
+                shapes += [(64, 128, 64, 1, 4, 2, 0), (64, 128, 64, 2, 2, 2, 0), (64, 256, 64, 1, 4, 2, 0),
+                           (64, 256, 64, 2, 4, 2, 0)]
             if self.N == 512:     # one tile spans the rows: row statistics complete inside the workgroup
                 shapes += [(128, 512, 64, 2, 4, 2, 0), (64, 512, 64, 1, 8, 2, 0),
                            # 32 x 256 wave tiles: 8 columns per lane halve the cross-lane steps per element of a
@@ -204,7 +213,8 @@ class AutoTunerBase:
     def heuristic(self) -> TileConfig:
         """Pick the candidate with the lowest modelled time: number of
         workgroup rounds on 256 CUs x work per tile / efficiency of the tile."""
-        eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3}
+        eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3,
+               (128, 64): 0.5, (64, 128): 0.5, (256, 64): 0.45, (64, 256): 0.45}
         best, best_cost = None, None
         for t in self.candidates():
             tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
@@ -218,6 +228,8 @@ class AutoTunerBase:
                 wg_per_cu = 1       # one workgroup per CU at most: nothing shares a CU's throughput
             rounds = -(-tiles // (NUM_CUS * wg_per_cu))
             cost = rounds * wg_per_cu * t.bm * t.bn / (eff.get((t.bm, t.bn), 0.5) * (1.3 if solo else 1.15 if t.pipe == 2 else 1.0))
+            if t.bn > self.N or t.bm > self.M:
+                cost *= 2.0         # no tile is whole: every epilogue access is checked (measured 3-7 x on narrow outputs)
             # few tiles, a long K and a small output: the kernel splits K over several workgroups per tile (the
             # rule of the generated host code); the exchange of partial tiles eats about half of the gain, and
             # more than four splits are not rewarded here
