@@ -221,13 +221,18 @@ class AutoTunerBase:
             # untuned default: a ping-pong tile or the plain double-buffered ring, or, for one round of 128 x 128
             # tiles with a CU each, the one-wave-per-SIMD loop (measured 8-19 % faster there than eight waves)
             solo = t.pipe == 12 and (t.bm, t.bn, t.stages) == (128, 128, 3) and tiles <= NUM_CUS and self.K >= 4 * t.bk
-            if (t.pipe not in (0, 2) and not solo) or t.stages == 1 or t.walk > 1:
+            # the one-barrier ping-pong loops with the options that won the sweeps of the reference's large
+            # products: 256 x 256 with 2 x 4 waves and pipe 7 (within 1 % of the best on every one of twelve
+            # shapes and layouts, 5-20 % ahead of 4 x 2 waves with two barriers), pipe 5 / 10 on the half tiles
+            tuned = (t.pipe, t.bm, t.bn, t.stages) in ((7, 256, 256, 2), (5, 256, 128, 3), (10, 128, 256, 3))
+            if (t.pipe not in (0, 2) and not solo and not tuned) or t.stages == 1 or t.walk > 1:
                 continue
             wg_per_cu = max(1, min(2, LDS_LIMIT // t.lds_bytes())) if t.bm * t.bn <= 128 * 128 else 1
             if tiles <= NUM_CUS:
                 wg_per_cu = 1       # one workgroup per CU at most: nothing shares a CU's throughput
             rounds = -(-tiles // (NUM_CUS * wg_per_cu))
-            cost = rounds * wg_per_cu * t.bm * t.bn / (eff.get((t.bm, t.bn), 0.5) * (1.3 if solo else 1.15 if t.pipe == 2 else 1.0))
+            loop = 1.3 if solo else 1.2 if tuned else 1.15 if t.pipe == 2 else 1.0
+            cost = rounds * wg_per_cu * t.bm * t.bn / (eff.get((t.bm, t.bn), 0.5) * loop)
             if t.bn > self.N or t.bm > self.M:
                 cost *= 2.0         # no tile is whole: every epilogue access is checked (measured 3-7 x on narrow outputs)
             # few tiles, a long K and a small output: the kernel splits K over several workgroups per tile (the
@@ -240,7 +245,9 @@ class AutoTunerBase:
             # latency and epilogue, and two 2-stage workgroups fit where one 4-stage one does), more stages when a
             # workgroup has its CU to itself (measured both ways on 128 x 128 tiles)
             stage_pref = 0.005 * (t.stages - 2) if tiles > NUM_CUS else -0.005 * (t.stages - 2)
-            cost *= 1.0 + 0.01 * (64 // t.bk - 1) + stage_pref + (0.002 if t.wm < t.wn else 0.0)
+            # 256 x 256: 2 x 4 waves (128 x 64 wave tiles) ahead of 4 x 2 in every layout measured
+            wave_pref = (-0.03 if t.wm < t.wn else 0.0) if (t.bm, t.bn) == (256, 256) else (0.002 if t.wm < t.wn else 0.0)
+            cost *= 1.0 + 0.01 * (64 // t.bk - 1) + stage_pref + wave_pref
             if best_cost is None or cost < best_cost:
                 best, best_cost = t, cost
         return best

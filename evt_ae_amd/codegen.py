@@ -490,29 +490,42 @@ class Codegen:
         # rows are processed in batches of MB x 16: the full-tensor loads of a batch are all issued before its
         # arithmetic and stores (loads do not move above stores by themselves), so a batch costs one round trip
         # to HBM; two 32-row blocks per batch keep the staging registers bounded on the largest wave tiles
-        e("constexpr int MB = MI >= 2 ? 2 : 1;")
+        # The staging registers of a batch sit next to the accumulators (16 MI NI per lane) and the epilogue's own
+        # values: with several full tensors to read, a batch shrinks to one 32-row block, then to 8 or 4 of its 16
+        # rows per lane, so that nothing spills (three residuals on a 256 x 256 tile spilled 576 bytes per lane with
+        # fixed batches of two blocks and ran 118 us where the unfused sequence takes 81)
+        stage_words = " + ".join(f"(int)sizeof({DTYPE_CTYPES[ir.slots[ir.nodes[n].slot].dtype]})" for n in aux_nodes) or "0"
+        e(f"constexpr int STAGE_BYTES_PER_ROW = NI * ({stage_words});     // per lane and row of the wave tile")
+        e("constexpr int STAGE_BUDGET = (256 - 16 * MI * NI - 104 > 16 ? 256 - 16 * MI * NI - 104 : 16) * 4;   // bytes per lane")
+        e("constexpr int STAGE_ROWS = STAGE_BYTES_PER_ROW == 0 ? 32 : STAGE_BUDGET / STAGE_BYTES_PER_ROW;")
+        e("constexpr int MB = (MI >= 2 && STAGE_ROWS >= 32) ? 2 : 1;")
+        e("constexpr int VB = STAGE_ROWS >= 16 ? 16 : STAGE_ROWS >= 8 ? 8 : 4;    // rows of a block per batch")
         e('static_assert(MI % MB == 0, "row blocks per wave must be 1 or even");')
         e("#pragma unroll")
         e("for (int mb = 0; mb < MI; mb += MB) {")
         e.indent()
+        e("#pragma unroll")
+        e("for (int vb = 0; vb < 16; vb += VB) {")
+        e.indent()
         if aux_nodes:
             for name in aux_nodes:
                 k = ir.nodes[name].slot
-                e(f"{DTYPE_CTYPES[ir.slots[k].dtype]} rb_{_cname(name)}[MB][16][NI];")
+                e(f"{DTYPE_CTYPES[ir.slots[k].dtype]} rb_{_cname(name)}[MB][VB][NI];")
             e("#pragma unroll")
             e("for (int mo = 0; mo < MB; ++mo) {")
             e.indent()
             e("#pragma unroll")
-            e("for (int v = 0; v < 16; ++v) {")
+            e("for (int vi = 0; vi < VB; ++vi) {")
             e.indent()
+            e("const int v = vb + vi;")
             e("const int row = t.row(mb + mo, v);")
             e("const bool rok = t.row_ok(row);")
             for name in aux_nodes:
                 k = ir.nodes[name].slot
                 e(f"if constexpr (FAST) evt::row_load<Tile>(rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mb + mo, v) * rp_{k}, "
-                  f"rb_{_cname(name)}[mo][v]);")
+                  f"rb_{_cname(name)}[mo][vi]);")
                 e(f"else evt::aux_load<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
-                  f"p.t{k}_sn, p.t{k}_vec, rok, rb_{_cname(name)}[mo][v]);")
+                  f"p.t{k}_sn, p.t{k}_vec, rok, rb_{_cname(name)}[mo][vi]);")
             e.dedent()
             e("}")
             e.dedent()
@@ -523,10 +536,11 @@ class Codegen:
         e("const int mi = mb + mo;")
         for name in aux_nodes:
             k = ir.nodes[name].slot
-            e(f"const {DTYPE_CTYPES[ir.slots[k].dtype]} (&r_{_cname(name)})[16][NI] = rb_{_cname(name)}[mo];")
+            e(f"const {DTYPE_CTYPES[ir.slots[k].dtype]} (&r_{_cname(name)})[VB][NI] = rb_{_cname(name)}[mo];")
         e("#pragma unroll")
-        e("for (int v = 0; v < 16; ++v) {")
+        e("for (int vi = 0; vi < VB; ++vi) {")
         e.indent()
+        e("const int v = vb + vi;")
         e("const int row = t.row(mi, v);")
         e("const bool rok = t.row_ok(row);")
         for name in inner:
@@ -582,6 +596,8 @@ class Codegen:
                 e(f"cst[ni][{o}] = (rok && t.col_ok(ni)) ? fmaxf(cst[ni][{o}], {x()}) : cst[ni][{o}];")
             e.dedent()
             e("}")
+        e.dedent()
+        e("}")
         e.dedent()
         e("}")
         e.dedent()
@@ -716,7 +732,7 @@ class Codegen:
                   f"{base} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, p.t{k}_sn, {c});")
             elif s.kind == "aux":
                 e(f"float {c}[NI];")
-                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = (float)r_{c}[v][ni];")
+                e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = (float)r_{c}[vi][ni];")
             elif s.kind == "row":
                 e(f"float {c}[NI];")
                 e(f"#pragma unroll\nfor (int ni = 0; ni < NI; ++ni) {c}[ni] = t.col_ok(ni) ? "

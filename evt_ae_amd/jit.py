@@ -41,6 +41,11 @@ HIPCC_FLAGS = [
     # packed-fp32 VALU forms are kept off on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-value", "-Wno-unknown-attributes",
+    # The epilogue's row loops are written to be unrolled in full: the accumulators are indexed by their loop
+    # counters and must stay in registers.  Past the compiler's default size limit for `#pragma unroll` a loop
+    # stays rolled and the accumulators go to scratch memory (three residual loads on a 128 x 64 wave tile: 576
+    # bytes of scratch per lane, 114 us instead of 53)
+    "-mllvm", "-pragma-unroll-threshold=1000000",
 ] + os.environ.get("EVT_HIPCC_EXTRA", "").split()
 
 

@@ -193,7 +193,9 @@ def test_untuned_problems_get_a_modelled_tile(monkeypatch):
         picks[problem] = t = tuner.heuristic()
         assert tuner.fits(t) and t in tuner.candidates()
     big, solo_a, solo_b, short_k = picks.values()
-    assert (big.bm, big.bn, big.pipe) == (256, 256, 2)
+    assert (big.bm, big.bn, big.wm, big.wn, big.pipe) == (256, 256, 2, 4, 7)     # what the sweeps of large products settle on
+    narrow = MMTuner((736389, 64, 64, 1), True, True, False, True, n.target.ir).heuristic()
+    assert (narrow.bm, narrow.bn) == (128, 64)      # never a tile wider than the problem
     assert (solo_a.bm, solo_a.bn, solo_a.wm * solo_a.wn, solo_a.pipe) == (128, 128, 4, 12) and solo_a == solo_b
     assert short_k.pipe != 12       # two k-tiles do not fill a three-stage ring
 
