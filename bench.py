@@ -373,6 +373,62 @@ def bench_encoder_step(torch, W, iters=20, only=None):
     return out
 
 
+def bench_reference_keys(torch, steps=30, only=None):
+    """Every GEMM / BMM problem of the reference's tuner caches (tests/golden/reference_tuner_keys.json: shape,
+    operand layouts and the seven node counts of its epilogue) at its real size: a synthetic epilogue with the
+    key's counts, fused (the tile the tuner cache or the model picks), against the same module run unfused by
+    PyTorch and against the library's GEMM alone.  µs per call, median of 3 regions of `steps` calls each."""
+    from tests import patterns as P
+    from evt_ae_amd.workloads import fused_nodes
+    rows = []
+    for table, key, case in P.reference_key_cases():
+        if only and not any(o in key for o in only):
+            continue
+        g = torch.Generator(device="cuda").manual_seed(1234)
+        ins = []
+        for i, (shape, dt) in enumerate(P.counted_epilogue_shapes(case)):
+            t = torch.empty(shape, dtype=dt, device="cuda")
+            flat = t.view(-1)
+            for lo in range(0, flat.numel(), 1 << 28):      # in pieces: the largest operands run to gigabytes
+                n = min(1 << 28, flat.numel() - lo)
+                flat[lo:lo + n] = (torch.randn(n, generator=g, device="cuda") * (0.02 if i == 1 else 1.0)).to(dt)
+            ins.append(t)
+        mod, _ = P.counted_epilogue(case)
+        gm = P.fuse(mod, [t.to("meta") for t in ins])
+        (node,) = fused_nodes(gm)
+        outs = gm(*ins)
+        with torch.no_grad():
+            refs = mod(*ins)
+        torch.cuda.synchronize()
+        worst = 0.0
+        for o, r in zip(outs, refs):      # a spot check against the unfused fp16 result; parity proper is the tests' job
+            o, r = o.float().reshape(-1), r.float().reshape(-1)
+            idx = torch.randint(0, o.numel(), (1 << 18,), device="cuda")
+            worst = max(worst, float((o[idx] - r[idx]).abs().max() / r[idx].abs().max().clamp_min(1e-6)))
+        if worst > 5e-2:
+            sys.exit(f"bench.py: reference key {key}: fused and unfused results differ ({worst:.3e})")
+        a, b = ins[0], ins[1]
+        swap = (1, 2) if case["batched"] else (0, 1)
+        A = a if case["a_row"] else a.transpose(*swap)
+        B = b if case["b_row"] else b.transpose(*swap)
+        mm = torch.bmm if case["batched"] else torch.mm
+        us = time_loop(torch, lambda i: gm(*ins), steps, 10, 3) * 1e3
+        with torch.no_grad():
+            us_eager = time_loop(torch, lambda i: mod(*ins), steps, 10, 3) * 1e3
+        us_lib = time_loop(torch, lambda i: mm(A, B), steps, 10, 3) * 1e3
+        rows.append({"key": key, "tile": node.target.tile.tag(), "us": round(us, 2), "unfused_us": round(us_eager, 2),
+                     "library_gemm_alone_us": round(us_lib, 2)})
+        log(f"[bench] {key} {rows[-1]}")
+        del ins, outs, refs, gm, a, b, A, B
+        torch.cuda.empty_cache()
+    import math
+    tot = {k: round(sum(r[k] for r in rows), 1) for k in ("us", "unfused_us", "library_gemm_alone_us")}
+    return {"keys": len(rows), "total_us": tot,
+            "geomean_speedup_vs_unfused": round(math.exp(sum(math.log(r["unfused_us"] / r["us"]) for r in rows) / max(len(rows), 1)), 3),
+            "slower_than_unfused": [r["key"] for r in rows if r["us"] > r["unfused_us"]],
+            "rows": rows}
+
+
 def cpu_baseline(torch, W, evt_oracle, cfgs, reps=3):
     """PyTorch fp32 eager evaluation of the same subgraphs on the host cores."""
     torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
@@ -635,6 +691,10 @@ def main():
     ap.add_argument("--no-clock-probe", dest="clock_probe", action="store_false",
                     help="skip the diagnostic build of each kernel that reports the shader clock it ran at and "
                          "workgroup 0's main-loop / epilogue split (per_config[*].clock_probe, roofline.shader_mhz)")
+    ap.add_argument("--reference-keys", nargs="*", metavar="SUBSTRING", default=None,
+                    help="run nothing but the GEMM / BMM problems of the reference's tuner caches (all of them, or "
+                         "those whose key contains one of the substrings) at their real sizes: fused, unfused and the "
+                         "library's GEMM alone; prints one JSON line")
     ap.add_argument("--no-power", dest="power", action="store_false",
                     help="skip the socket-power readings taken while each config and the MFMA probe run for two seconds "
                          "(per_config[*].power, roofline.mfma_only.power)")
@@ -665,6 +725,9 @@ def main():
     torch.cuda.set_device(0)
     if args.only_encoder_step:
         print(json.dumps({"encoder_layer_step": bench_encoder_step(torch, W, only=args.only_encoder_step)}), flush=True)
+        return
+    if args.reference_keys is not None:
+        print(json.dumps({"reference_keys": bench_reference_keys(torch, only=args.reference_keys or None)}), flush=True)
         return
     cfgs = [int(c) for c in args.configs.split(",")]
     meter = PowerMeter(torch) if args.power else None
