@@ -21,6 +21,7 @@ the Infinity Cache does not stand in for HBM.
 """
 import argparse
 import json
+import operator
 import os
 import sys
 import time
@@ -113,9 +114,12 @@ class Case:
         ret = out_node.args[0]
         ret = list(ret) if isinstance(ret, (tuple, list)) else [ret]
         order = []
-        for r in ret:   # each is view(getitem(fused, idx))
-            gi = r.args[0]
-            order.append(res[gi.args[1]].view(r.args[1]))
+        for r in ret:   # each is getitem(fused, idx), or a view of one
+            if r.target is operator.getitem:
+                order.append(res[r.args[1]])
+            else:
+                gi = r.args[0]
+                order.append(res[gi.args[1]].view(r.args[1]))
         return order
 
 

@@ -139,12 +139,27 @@ def launch_switches() -> Tuple[int, int]:
     EVT_TWO_KERNEL_REDUCE=1 finishes cross-tile reductions in the finalize
     kernel, EVT_ROW_WG_PER_CU=n sets the workgroups per CU of the row-wise
     kernels.  The kernel modules themselves read no environment."""
-    split = os.environ.get("EVT_SPLIT_K")
-    flags = jit.EVT_FLAG_TWO_KERNEL_REDUCE if os.environ.get("EVT_TWO_KERNEL_REDUCE") == "1" else 0
-    per_cu = os.environ.get("EVT_ROW_WG_PER_CU")
+    if _ENV_BYTES:      # the usual case, nothing set: three dictionary look-ups
+        d = _ENV_DATA
+        if d.get(b"EVT_SPLIT_K") is None and d.get(b"EVT_TWO_KERNEL_REDUCE") is None and d.get(b"EVT_ROW_WG_PER_CU") is None:
+            return 0, 0
+    split, two, per_cu = _env("EVT_SPLIT_K"), _env("EVT_TWO_KERNEL_REDUCE"), _env("EVT_ROW_WG_PER_CU")
+    flags = jit.EVT_FLAG_TWO_KERNEL_REDUCE if two == "1" else 0
     if per_cu:
         flags |= jit.evt_flag_row_wg_per_cu(max(0, min(254, int(per_cu))))
     return (max(0, int(split)) if split else 0), flags
+
+
+_ENV_DATA = getattr(os.environ, "_data", None)        # the mapping behind os.environ (bytes keys on POSIX)
+_ENV_BYTES = isinstance(_ENV_DATA, dict) and os.name == "posix"
+
+
+def _env(name: str) -> Optional[str]:
+    """os.environ.get(name) without its per-call encoding and wrapping: these switches are read at every launch."""
+    if isinstance(_ENV_DATA, dict):
+        v = _ENV_DATA.get(name.encode() if os.name == "posix" else name.upper())
+        return None if v is None else (v.decode() if isinstance(v, bytes) else v)
+    return os.environ.get(name)
 
 
 class FusedOpBase:
@@ -285,11 +300,11 @@ class FusedOpBase:
         ws_bytes = cached[1]
         if not ws_bytes:
             return 0, 0
-        key = stream.cuda_stream
+        key = stream if isinstance(stream, int) else stream.cuda_stream      # a raw stream handle or a torch stream
         ws = self._workspace.get(key)
         if ws is None or ws.numel() < ws_bytes:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
-            self.module.workspace_init(ws.data_ptr(), ws_bytes, stream.cuda_stream)
+            self.module.workspace_init(ws.data_ptr(), ws_bytes, key)
             self._workspace[key] = ws
         return ws.data_ptr(), ws_bytes
 
@@ -300,12 +315,21 @@ class FusedOpBase:
                 for name, (shape, dtype) in self.store_meta.items()}
 
     def call(self, visitor_args: Dict[str, torch.Tensor], stream, *args) -> Any:
+        """`stream`: a torch stream or a raw HIP stream handle."""
         a, keep = self.build_arguments(visitor_args, *args)
         ws_ptr, ws_bytes = self.workspace_for(a, stream, keep[0].device)
-        self.module.launch(a, ws_ptr, ws_bytes, stream.cuda_stream)
+        self.module.launch(a, ws_ptr, ws_bytes, stream if isinstance(stream, int) else stream.cuda_stream)
 
     def get_output_name(self, output: Node) -> str:
         return "accum" if output is self.node else output.name
+
+    def result_shape(self, name: str) -> Tuple[int, ...]:
+        """Shape of the tensor `__call__` returns for output `name`: the stored tensor's, seen through the views
+        and permutes that follow the store."""
+        shape = tuple(self.store_meta[self.output2store[name]][0])
+        for op, arg in self.post_reshape_permute.get(name, ()):
+            shape = tuple(int(d) for d in arg) if op == "view" else tuple(shape[int(i)] for i in arg)
+        return shape
 
     def __call__(self, *args_):
         if not _hip_device_present():
@@ -313,12 +337,14 @@ class FusedOpBase:
         # every microsecond here is paid per launch: no copies of what is contiguous already, no stream context
         # unless the op has a stream of its own, the result plan (store, views / permutes) worked out once
         args = [a if (not isinstance(a, torch.Tensor) or a.is_contiguous()) else a.contiguous() for a in args_]
-        default_stream = torch.cuda.current_stream()
         if self.stream is not None:
-            self.stream.wait_stream(default_stream)
+            self.stream.wait_stream(torch.cuda.current_stream())
             stream = self.stream
         else:
-            stream = default_stream
+            # the current stream's raw handle: torch.cuda.current_stream() builds a Stream object and resolves
+            # the device three times over, 8 us per call where this takes a fraction of one
+            index = args[-1].device.index
+            stream = _raw_current_stream(torch.cuda.current_device() if index is None else index)
 
         with (torch.cuda.stream(stream) if self.stream is not None else nullcontext()):
             visitor_args = self.allocate_outputs(args[-1].device)
@@ -451,6 +477,10 @@ def operand_strides(chain: Sequence[Node], shape3: Sequence[int]) -> Optional[St
 
 
 _HIP_PRESENT: Optional[bool] = None
+
+
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
+    lambda index: torch.cuda.current_stream(index).cuda_stream)
 
 
 def _hip_device_present() -> bool:
@@ -925,9 +955,16 @@ class EVTFuser:
             graph_module.graph.inserting_after(get_item_node)
             shape, dtype = node_shape_dtype(output_node)
             get_item_node.meta = {"tensor_meta": _tensor_meta(shape, dtype), **carried}
-            view_node = graph_module.graph.call_function(aten.view, args=(get_item_node, list(shape)))
-            view_node.meta = {k: v for k, v in output_node.meta.items()
-                              if k in ("tensor_meta", "val", "partitioner_tag", "seq_nr", "autograd_backward")}
+            out_meta = {k: v for k, v in output_node.meta.items()
+                        if k in ("tensor_meta", "val", "partitioner_tag", "seq_nr", "autograd_backward")}
+            name = "accum" if output_node is anchor else output_node.name
+            if tuple(fused_kernel.result_shape(name)) == tuple(shape):
+                # the kernel's result has the node's shape already: no view node (an aten call per output and launch)
+                get_item_node.meta.update(out_meta)
+                view_node = get_item_node
+            else:
+                view_node = graph_module.graph.call_function(aten.view, args=(get_item_node, list(shape)))
+                view_node.meta = out_meta
             if output_node is anchor:
                 for user in list(anchor.users):
                     if user not in epi_set and user is not fused_node:
