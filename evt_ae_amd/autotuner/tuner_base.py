@@ -166,10 +166,10 @@ class AutoTunerBase:
             # narrow outputs (GCN's 736389 x 64 products): a tile wider than the problem leaves every tile partial,
             # which costs the epilogue its check-free path and the main loop half its MFMAs; measured on
             # 736389 x 64 x 64 with two residual loads 459 us on 256 x 128 tiles, 61 us on 128 x 64
-            if self.N <= 64 or self.N % 128 == 64:
+            if self.N <= 64 or self.N % 128 == 64 or self.K <= 64:
                 shapes += [(128, 64, 64, 4, 1, 2, 0), (128, 64, 64, 2, 2, 2, 0), (256, 64, 64, 4, 1, 2, 0),
                            (256, 64, 64, 4, 2, 2, 0)]
-            if self.M <= 64 or self.M % 128 == 64:
+            if self.M <= 64 or self.M % 128 == 64 or self.K <= 64:
                 shapes += [(64, 128, 64, 1, 4, 2, 0), (64, 128, 64, 2, 2, 2, 0), (64, 256, 64, 1, 4, 2, 0),
                            (64, 256, 64, 2, 4, 2, 0)]
             if self.N == 512:     # one tile spans the rows: row statistics complete inside the workgroup
@@ -215,9 +215,30 @@ class AutoTunerBase:
         workgroup rounds on 256 CUs x work per tile / efficiency of the tile."""
         eff = {(256, 256): 1.0, (256, 128): 0.85, (128, 256): 0.85, (128, 128): 0.7, (64, 64): 0.3,
                (128, 64): 0.5, (64, 128): 0.5, (256, 64): 0.45, (64, 256): 0.45}
+        # K fits one k-tile: nothing to pipeline and next to no arithmetic, the launch streams its operands in and its
+        # output out.  What counts is the area the tiles cover (the edge tiles of a 264 x 264 batch cost a whole
+        # workgroup each) and how many workgroups a CU holds; measured on the reference's batched K = 64 problems,
+        # single-stage 128 x 64 tiles with 4 x 1 waves lead or tie everywhere (1536 x 264 x 264 x 64: 128 us
+        # against 155 on 128 x 128 and 178 on 64 x 64; 512 x 512 x 512 x 64: 59.7 against 72.4 and 68.2 on the
+        # ping-pong 256 x 256)
+        one_k_tile = self.dma and self.K <= 64
+        eff_stream = {(128, 64): 1.0, (256, 64): 0.95, (64, 128): 0.95, (128, 512): 0.95, (256, 128): 0.9,
+                      (128, 256): 0.9, (128, 128): 0.85, (256, 256): 0.8, (64, 64): 0.7}
         best, best_cost = None, None
         for t in self.candidates():
             tiles = -(-self.M // t.bm) * -(-self.N // t.bn) * self.L
+            if one_k_tile:
+                if t.stages != 1 or t.pipe != 0 or t.walk > 1:
+                    continue
+                cost = tiles * t.bm * t.bn / eff_stream.get((t.bm, t.bn), 0.6)
+                if t.bn > self.N or t.bm > self.M:
+                    cost *= 2.0
+                if self.ir.row_state and t.bn >= self.N:
+                    cost *= 0.6         # the whole row in one tile: its statistics finish inside the workgroup
+                cost *= 1.0 + (0.002 if t.wm < t.wn else 0.0)
+                if best_cost is None or cost < best_cost:
+                    best, best_cost = t, cost
+                continue
             # untuned default: a ping-pong tile or the plain double-buffered ring, or, for one round of 128 x 128
             # tiles with a CU each, the one-wave-per-SIMD loop (measured 8-19 % faster there than eight waves)
             solo = t.pipe == 12 and (t.bm, t.bn, t.stages) == (128, 128, 3) and tiles <= NUM_CUS and self.K >= 4 * t.bk
@@ -250,6 +271,13 @@ class AutoTunerBase:
             cost *= 1.0 + 0.01 * (64 // t.bk - 1) + stage_pref + wave_pref
             if best_cost is None or cost < best_cost:
                 best, best_cost = t, cost
+        if best is None and one_k_tile:      # no single-stage tile holds this epilogue: the general model
+            one_k_tile_was, self_k = True, self.K
+            try:
+                self.K = 65
+                return self.heuristic()
+            finally:
+                self.K = self_k
         return best
 
     # -- timing ----------------------------------------------------------------------

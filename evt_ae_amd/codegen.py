@@ -522,7 +522,7 @@ class Codegen:
             e("const bool rok = t.row_ok(row);")
             for name in aux_nodes:
                 k = ir.nodes[name].slot
-                e(f"if constexpr (FAST) evt::row_load<Tile>(rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mb + mo, v) * rp_{k}, "
+                e(f"if constexpr (FAST) evt::row_load<Tile>(t, rok, rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mb + mo, v) * rp_{k}, "
                   f"rb_{_cname(name)}[mo][vi]);")
                 e(f"else evt::aux_load<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
                   f"p.t{k}_sn, p.t{k}_vec, rok, rb_{_cname(name)}[mo][vi]);")
@@ -705,7 +705,7 @@ class Codegen:
 
     def emit_tile_store(self, e: _Emitter, k: int, arr: str):
         """Store the NI values `arr` of row (mi, v) to tile slot k (inside the row loops)."""
-        e(f"if constexpr (FAST) evt::row_store<Tile, {DTYPE_CTYPES[self.ir.slots[k].dtype]}>(rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mi, v) * rp_{k}, {arr});")
+        e(f"if constexpr (FAST) evt::row_store<Tile, {DTYPE_CTYPES[self.ir.slots[k].dtype]}>(t, rok, rs_{k}, vo_{k}, (uint32_t)Tile::row_step(mi, v) * rp_{k}, {arr});")
         e(f"else evt::aux_store<false>(t, p.t{k}, {self.slot_off(k)} + (int64_t)row * p.t{k}_sm + (int64_t)t.col0 * p.t{k}_sn, "
           f"p.t{k}_sn, p.t{k}_vec, rok, {arr});")
 
@@ -743,7 +743,7 @@ class Codegen:
                 else:
                     ct = DTYPE_CTYPES[s.dtype]
                     e(f"float {c};")
-                    e(f"if constexpr (FAST) {c} = evt::buffer_ld_f32<{ct}>(rc_{k}, vc_{k}, (uint32_t)Tile::row_step(mi, v) * cp_{k});")
+                    e(f"if constexpr (FAST) {c} = evt::buffer_ld_f32<{ct}>(rc_{k}, (Tile::FULL || rok) ? vc_{k} : evt::kOobOffset, (uint32_t)Tile::row_step(mi, v) * cp_{k});")
                     e(f"else {c} = rok ? evt::ld_f32(p.t{k}, {base} + (int64_t)row * p.t{k}_sm) : 0.f;")
             else:
                 e(f"const float {c} = evt::ld_f32(p.t{k}, 0);")

@@ -269,9 +269,16 @@ EVT_DEV float buffer_ld_f32(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t s
   }
 }
 
+// On a tile that is not whole (Tile::FULL false) the same instructions serve: a lane whose row or columns lie
+// outside the matrix gets an offset beyond the buffer's range, which the hardware answers with zeros (loads) or
+// drops (stores) -- no branch, no per-element address arithmetic.  The caller has checked that valid columns
+// come in whole vectors (N a multiple of NI) where a lane's NI columns move as one access.
 template <class Tile, class T>
-EVT_DEV void row_load(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, T (&out)[Tile::NI]) {
+EVT_DEV void row_load(const Tile& t, bool rok, __amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, T (&out)[Tile::NI]) {
   constexpr int NI = Tile::NI;
+  if constexpr (!Tile::FULL) {
+    if (!rok || (row_is_vector<Tile, T>() && t.col0 + NI > t.N)) voff = kOobOffset;
+  }
   if constexpr (row_is_vector<Tile, T>() && NI == 8) {
     const u32x4 raw = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
     const T* e = (const T*)&raw;
@@ -289,7 +296,7 @@ EVT_DEV void row_load(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, T
   } else {
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
-      out[ni] = buffer_load_elem<T>(rs, voff + (uint32_t)(ni * Tile::COL_STEP * (int)sizeof(T)), soff);
+      out[ni] = buffer_load_elem<T>(rs, t.col_ok(ni) ? voff + (uint32_t)(ni * Tile::COL_STEP * (int)sizeof(T)) : kOobOffset, soff);
   }
 }
 
@@ -329,8 +336,12 @@ EVT_DEV void buffer_store_elem(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_
   }
 }
 template <class Tile, class T>
-EVT_DEV void row_store(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, const float (&val)[Tile::NI]) {
+EVT_DEV void row_store(const Tile& t, bool rok, __amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff,
+                       const float (&val)[Tile::NI]) {
   constexpr int NI = Tile::NI;
+  if constexpr (!Tile::FULL) {
+    if (!rok || (row_is_vector<Tile, T>() && t.col0 + NI > t.N)) voff = kOobOffset;
+  }
   if constexpr (row_is_vector<Tile, T>()) {
     T e[NI];
 #pragma unroll
@@ -341,7 +352,7 @@ EVT_DEV void row_store(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff, 
   } else {
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
-      buffer_store_elem<T>(rs, voff + (uint32_t)(ni * Tile::COL_STEP * (int)sizeof(T)), soff, val[ni]);
+      buffer_store_elem<T>(rs, t.col_ok(ni) ? voff + (uint32_t)(ni * Tile::COL_STEP * (int)sizeof(T)) : kOobOffset, soff, val[ni]);
   }
 }
 
@@ -1268,6 +1279,12 @@ EVT_DEV void run_epilogue(const GemmArgs& g, const typename Epi::Params& p, int 
     t.init(g, batch, tm, tn, smem);
     if constexpr (Cfg::WALK) t.set_walk(part, g.parts_n, first, last, state);
     Epi::template tile<Cfg, TileCtx<Cfg, true>, true>(p, t, g, acc);
+  } else if (p.fast && (!Cfg::ADJACENT || g.N % Cfg::NI == 0)) {
+    // a tile on the matrix's edge: the same buffer accesses, lanes outside the matrix masked by their offsets
+    TileCtx<Cfg, false> t;
+    t.init(g, batch, tm, tn, smem);
+    if constexpr (Cfg::WALK) t.set_walk(part, g.parts_n, first, last, state);
+    Epi::template tile<Cfg, TileCtx<Cfg, false>, true>(p, t, g, acc);
   } else {
     TileCtx<Cfg, false> t;
     t.init(g, batch, tm, tn, smem);
