@@ -106,6 +106,7 @@ def main():
                     help="only the tiles of SHORT_LIST (with their single-stage forms where K fits one tile, and walking "
                          "forms where the candidates have them)")
     ap.add_argument("--cache", default=None, help="tuner cache file to write (default: the package's)")
+    ap.add_argument("--resume", action="store_true", help="skip problems the cache file already has a row for")
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     ap.add_argument("--sigma", default=None, help="standard deviations of the timing operands, 'sigma_A,sigma_B' "
                                                     "(default: 1.0,0.02, activations against weights)")
@@ -129,7 +130,8 @@ def main():
     mods = []
     for cfg, t in tuners:
         for tile in t.candidates():
-            mods.append(jit.load_module(t.ir, KernelSpec.for_problem(t.K, t.a_kc, t.b_kc, t.bf16, tile)))
+            mods.append(jit.load_module(t.ir, KernelSpec.for_problem(t.K, t.a_kc, t.b_kc, t.bf16, tile, t.M, t.N)))
+    mods = list({str(m.path): m for m in mods}.values())       # problems with one epilogue structure share modules
     todo = [m for m in mods if not m.path.exists()]
     print(f"[tune] {len(mods)} candidate modules, {len(todo)} to compile", flush=True)
     with ThreadPoolExecutor(args.jobs) as pool:
@@ -149,6 +151,9 @@ def main():
         t.cache_file = default_cache_file()
         if args.sigma:
             t.operand_sigma = sigma
+        if args.resume and t.fetch_cached() is not None:
+            print(f"[tune] config {cfg}: already in {t.cache_file}", flush=True)
+            continue
 
         def report(tile, us, note, cfg=cfg):
             if us is None:

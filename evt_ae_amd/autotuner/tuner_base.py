@@ -288,12 +288,16 @@ class AutoTunerBase:
         dt = torch.bfloat16 if self.bf16 else torch.float16
         M, N, K, L = self.M, self.N, self.K, self.L
         sa, sb = self.operand_sigma
-        A = (torch.randn((L, M, K) if self.a_kc else (L, K, M), device=dev, dtype=torch.float32) * sa).to(dt)
-        B = (torch.randn((L, N, K) if self.b_kc else (L, K, N), device=dev, dtype=torch.float32) * sb).to(dt)
+        # rows padded to the transfer path's 8 elements where an extent is no multiple of 8 (what the fused op's
+        # padded copies look like, FusedGEMM.pad)
+        r8 = (lambda v: (v + 7) & ~7) if self.dma else (lambda v: v)
+        lda, ldb = r8(K if self.a_kc else M), r8(K if self.b_kc else N)
+        A = (torch.randn((L, M, lda) if self.a_kc else (L, K, lda), device=dev, dtype=torch.float32) * sa).to(dt)
+        B = (torch.randn((L, N, ldb) if self.b_kc else (L, K, ldb), device=dev, dtype=torch.float32) * sb).to(dt)
         a = jit.EvtArgs()
         a.M, a.N, a.K, a.L = M, N, K, L
-        a.A, a.lda, a.batch_stride_A = A.data_ptr(), (K if self.a_kc else M), M * K
-        a.B, a.ldb, a.batch_stride_B = B.data_ptr(), (K if self.b_kc else N), N * K
+        a.A, a.lda, a.batch_stride_A = A.data_ptr(), lda, A.shape[1] * lda
+        a.B, a.ldb, a.batch_stride_B = B.data_ptr(), ldb, B.shape[1] * ldb
         a.num_tensors, a.num_scalars = len(self.ir.slots), len(self.ir.scalars)
         keep = [A, B]
         nbytes = (A.numel() + B.numel()) * 2
@@ -325,7 +329,7 @@ class AutoTunerBase:
 
     def profile(self, tile: TileConfig) -> float:
         from .. import jit
-        module = jit.load_module(self.ir, KernelSpec.for_problem(self.K, self.a_kc, self.b_kc, self.bf16, tile))
+        module = jit.load_module(self.ir, KernelSpec.for_problem(self.K, self.a_kc, self.b_kc, self.bf16, tile, self.M, self.N))
         sets = self.argument_sets()
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = module.workspace_bytes(sets[0][0])

@@ -1279,7 +1279,7 @@ EVT_DEV void run_epilogue(const GemmArgs& g, const typename Epi::Params& p, int 
     t.init(g, batch, tm, tn, smem);
     if constexpr (Cfg::WALK) t.set_walk(part, g.parts_n, first, last, state);
     Epi::template tile<Cfg, TileCtx<Cfg, true>, true>(p, t, g, acc);
-  } else if (p.fast && (!Cfg::ADJACENT || g.N % Cfg::NI == 0)) {
+  } else if (Epi::EDGE_TILES && p.fast && (!Cfg::ADJACENT || g.N % Cfg::NI == 0)) {
     // a tile on the matrix's edge: the same buffer accesses, lanes outside the matrix masked by their offsets
     TileCtx<Cfg, false> t;
     t.init(g, batch, tm, tn, smem);

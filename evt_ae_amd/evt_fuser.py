@@ -565,7 +565,8 @@ class FusedGEMM(FusedOpBase):
             tuner = MMTuner((M, N, K, 1), self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
             tile = tuner.get_best_config()
             self.tile = tile
-            self.spec = KernelSpec.for_problem(K, self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
+            self.spec = KernelSpec.for_problem(K, self.a_kc, self.b_kc, dtype == torch.bfloat16, tile,
+                                               self.problem[0], self.problem[1])
             self.module = jit.load_module(self.ir, self.spec)
 
     def operands(self, A, B):
@@ -670,7 +671,8 @@ class FusedBMM(FusedOpBase):
             tuner = BMMTuner(self.problem, self.a_kc, self.b_kc, dtype == torch.bfloat16, dma, self.ir)
             tile = tuner.get_best_config()
             self.tile = tile
-            self.spec = KernelSpec.for_problem(K, self.a_kc, self.b_kc, dtype == torch.bfloat16, tile)
+            self.spec = KernelSpec.for_problem(K, self.a_kc, self.b_kc, dtype == torch.bfloat16, tile,
+                                               self.problem[0], self.problem[1])
             self.module = jit.load_module(self.ir, self.spec)
 
     # kept for callers that ask which 3-D permutation an operand went through
