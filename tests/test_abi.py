@@ -259,3 +259,38 @@ def test_tuner_reports_candidates_that_fail(monkeypatch, caplog):
     # the sweep alone would have picked tiles[3] (29.5 us); timed again in turns its median is 34 us against 30.5
     assert best == tiles[0] and stored == [(tiles[0], 30.5)]
     assert calls.count(tiles[0]) == 1 + tuner.second_stage_rounds and calls.count(tiles[1]) == 1
+
+
+def test_in_step_stage_keeps_what_the_step_prefers(tmp_path, monkeypatch):
+    """The tuner's third stage for a model's cache: a problem's best few tiles are tried inside the model's step, and
+    a row changes only when the kernels it touches get faster by more than the threshold; a candidate that loses
+    leaves the row as it was."""
+    from evt_ae_amd.autotuner import tune_workloads as TW
+    from evt_ae_amd.autotuner.gemm_tuner import MMTuner
+    from evt_ae_amd.codegen import TileConfig
+    cache = tmp_path / "tuner_cache.db"
+    monkeypatch.setenv("EVT_TUNER_CACHE", str(cache))
+    inputs = W.make_inputs(1, W.GOLDEN_SHAPES[1])
+    (n,) = fused_nodes(W.fuse(W.CONFIGS[1].module(), [t.to("meta") for t in inputs]))
+    first = MMTuner((4096, 1024, 1024, 1), True, True, False, True, n.target.ir)
+    second = MMTuner((4096, 4096, 1024, 1), True, True, False, True, n.target.ir)
+    a, b, c = (TileConfig(128, 128, 64, 2, 2, 2, True, 4, 0), TileConfig(128, 128, 64, 2, 2, 3, True, 4, 12),
+               TileConfig(256, 128, 64, 4, 2, 3, True, 4, 5))
+    first.store(a, 14.7)            # the sweep's winners
+    second.store(c, 40.0)
+    in_step = {(first.key(), a): 19.5, (first.key(), b): 15.6, (first.key(), c): 17.0,      # us inside the step
+               (second.key(), c): 41.0, (second.key(), a): 40.8, (second.key(), b): 47.0}
+
+    class FakeTimer:
+        def build(self, cache_file):
+            assert str(cache_file) == str(cache)
+            return {t.key(): t.fetch_cached() for t in (first, second)}     # a "step" is the rows it was traced with
+
+        def compare(self, kept, trial):
+            (key,) = [k for k in kept if kept[k] != trial[k]]               # one row differs per trial
+            x, y = in_step[key, kept[key]], in_step[key, trial[key]]
+            return x, y, 700.0 + x, 700.0 + y
+    ranked = [("first", first, [(14.7, a), (17.4, b), (18.0, c)]), ("second", second, [(40.0, c), (40.5, a), (46.0, b)])]
+    TW._in_step_stage({}, ranked, top=3, timer=FakeTimer())
+    assert first.fetch_cached() == b        # 15.6 us in the step against 19.5: taken; c (17.0) then loses against b
+    assert second.fetch_cached() == c       # 40.8 against 41.0 is inside the threshold: the sweep's row stays
