@@ -185,6 +185,7 @@ class FusedOpBase:
         self.slot_sources = epilogue_visitor.slot_sources      # slot -> ('input', idx) | ('output', store name)
         self.store_meta = epilogue_visitor.store_meta          # store name -> (shape, dtype)
         self._workspace = {}
+        self._spare_workspace = None     # cleared at the first eager call, for the first graph capture (workspace_for)
         # rand_like stream: 64-bit seed (torch's global seed at the time of the call unless `rand_seed` is set), a
         # 32-bit offset that advances by one per launch, so successive calls draw different numbers, and a stream
         # id of the op's own (rand_stream_id: from the anchor node's name) that goes into the generator's counter
@@ -303,8 +304,26 @@ class FusedOpBase:
         key = stream if isinstance(stream, int) else stream.cuda_stream      # a raw stream handle or a torch stream
         ws = self._workspace.get(key)
         if ws is None or ws.numel() < ws_bytes:
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
-            self.module.workspace_init(ws.data_ptr(), ws_bytes, key)
+            # what torch says about "the current stream" holds for this launch only if it goes to that stream
+            index = torch.device(device).index
+            current = key == _raw_current_stream(torch.cuda.current_device() if index is None else index)
+            capturing = current and torch.cuda.is_current_stream_capturing()
+            spare = self._spare_workspace
+            if capturing and spare is not None and spare.numel() >= ws_bytes and spare.device == torch.device(device):
+                # A fill recorded into the graph would run at every replay, although launches leave the workspace
+                # clean (measured on an encoder layer's training step: eight fills, 63 of 840 us per replay), and
+                # nothing outside the graph may be waited for while a capture is open.  The capture takes the spare
+                # that the op's first eager call cleared; without one (no eager call before the capture, or a
+                # second capture) the fill is recorded, which is correct and only slower.
+                ws, self._spare_workspace = spare, None
+            else:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
+                self.module.workspace_init(ws.data_ptr(), ws_bytes, key)
+                if current and not capturing and (spare is None or spare.numel() < ws_bytes):
+                    # cleared now and waited for once, so that it is clean whenever a capture takes it
+                    spare = self._spare_workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
+                    self.module.workspace_init(spare.data_ptr(), ws_bytes, key)
+                    torch.cuda.synchronize(spare.device)
             self._workspace[key] = ws
         return ws.data_ptr(), ws_bytes
 

@@ -323,6 +323,40 @@ def test_launch_is_graph_capturable():
             assert torch.equal(outs[name].view(-1), e.contiguous().view(-1)), (rep, name)
 
 
+def test_graph_capture_of_a_fused_call_records_no_workspace_fill():
+    """A fused call made through the op itself under torch.cuda.graph, on the capture's own stream, which the op
+    has never seen: it takes the workspace that the first eager call cleared as a spare, so the graph holds the
+    kernel alone (a recorded fill would run at every replay).  Every replay equals the eager call bit for bit; a
+    second capture finds no spare and records the fill, with the same results."""
+    wl = W.CONFIGS[3]
+    inputs = [t.cuda() for t in W.make_inputs(3, W.SMALL_SHAPES[3])]
+    gm = W.fuse(wl.module(), inputs)
+    (node,) = fused_nodes(gm)
+    op = node.target
+    ph = [n for n in gm.graph.nodes if n.op == "placeholder"]
+    args = [inputs[ph.index(a)] for a in node.args]
+    assert op._spare_workspace is None
+    eager = [o.clone() for o in op(*args)]
+    torch.cuda.synchronize()
+    assert op._spare_workspace is not None and len(op._workspace) == 1
+    spare_ptr = op._spare_workspace.data_ptr()
+    for capture in range(2):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=torch.cuda.Stream()):       # a stream of its own for each capture
+            captured = op(*args)
+        assert op._spare_workspace is None and len(op._workspace) == 2 + capture
+        if capture == 0:
+            assert spare_ptr in {w.data_ptr() for w in op._workspace.values()}
+        for rep in range(3):
+            for t in captured:
+                t.zero_()
+            _ = (inputs[0].float() @ inputs[1].float()).sum().item()   # unrelated eager work + a sync between replays
+            graph.replay()
+            torch.cuda.synchronize()
+            for o, e in zip(captured, eager):
+                assert torch.equal(o, e), (capture, rep)
+
+
 def test_debug_mode_self_check():
     """MODE=DEBUG (evt_fuser.py:98-172): the first call compares the kernel with
     the eager anchor + extracted epilogue module and records the verdict."""
