@@ -576,6 +576,7 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
                                             unsqueeze(ne(target, ignore_index), 1)) [/ batch]   (:294-348;
                                         the reference compares with -1 instead of ignore_index)
       masked_fill(x, mask, v)        -> where(mask, v, x)                        (scalar v; not in the reference)
+      pow(x, 1)                      -> x                                        (not in the reference)
       getitem(unbind(x, d), i)       -> select(x, d, i)                          (not in the reference)
       add of select_backward(g_i, s, d, i) over every i
                                      -> stack([g_0, g_1, ...], d)                (not in the reference)
@@ -624,6 +625,10 @@ def pass_decomposition(module: GraphModule, graph: Graph = None, disabled_ops: S
             elif name == "threshold_backward":
                 g, y, t = node.args
                 new = mk(aten.mul, (g, mk(aten.gt, (y, t))))
+            elif (name == "pow" and len(node.args) == 2 and isinstance(node.args[0], Node)
+                  and type(node.args[1]) in (int, float) and node.args[1] == 1):
+                # autograd writes pow(x, 1) into the backward of every x ** 2, and ATen runs it as a copy of x
+                new = node.args[0]
             elif name == "masked_fill" and len(node.args) == 3 and isinstance(node.args[2], (int, float)):
                 # a fill value under a mask is a select: where(mask, value, x) is in the epilogue vocabulary
                 x, mask, value = node.args

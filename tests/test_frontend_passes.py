@@ -141,6 +141,22 @@ def test_permute_pairs_fold():
     assert torch.equal(out[0], w @ w.t()) and torch.equal(out[1], x.permute(2, 0, 1).permute(0, 2, 1))
 
 
+def test_pow_of_one_is_the_value_itself():
+    """The backward of x ** 2 as autograd writes it holds pow(x, 1), which ATen runs as a copy of x: the
+    decomposition pass takes it out, and only it."""
+    class P(torch.nn.Module):
+        def forward(self, x, g):
+            return aten.mul(aten.mul(aten.pow(x, 1.0), 2.0), g), aten.pow(x, 2), aten.pow(x, 1.5), aten.pow(x, 1)
+
+    gp = W.trace_module(P(), [torch.empty(3, 5), torch.empty(3, 5)])
+    pass_decomposition(gp)
+    assert names_of(gp).count("pow") == 2
+    x, g = torch.randn(3, 5).abs(), torch.randn(3, 5)
+    out = gp(x, g)
+    assert torch.equal(out[0], x * 2.0 * g) and torch.equal(out[1], x ** 2) and torch.equal(out[2], x ** 1.5)
+    assert torch.equal(out[3], x)
+
+
 def test_clean_up_and_loss_elimination():
     class M(torch.nn.Module):
         def forward(self, x, y):
