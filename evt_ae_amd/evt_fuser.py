@@ -306,10 +306,11 @@ class FusedOpBase:
         if ws is None or ws.numel() < ws_bytes:
             # what torch says about "the current stream" holds for this launch only if it goes to that stream
             index = torch.device(device).index
-            current = key == _raw_current_stream(torch.cuda.current_device() if index is None else index)
+            index = torch.cuda.current_device() if index is None else index
+            current = key == _raw_current_stream(index)
             capturing = current and torch.cuda.is_current_stream_capturing()
             spare = self._spare_workspace
-            if capturing and spare is not None and spare.numel() >= ws_bytes and spare.device == torch.device(device):
+            if capturing and spare is not None and spare.numel() >= ws_bytes and spare.device.index == index:
                 # A fill recorded into the graph would run at every replay, although launches leave the workspace
                 # clean (measured on an encoder layer's training step: eight fills, 63 of 840 us per replay), and
                 # nothing outside the graph may be waited for while a capture is open.  The capture takes the spare
