@@ -433,7 +433,7 @@ def bench_reference_keys(torch, steps=30, only=None):
             "rows": rows}
 
 
-def cpu_baseline(torch, W, evt_oracle, cfgs, reps=3):
+def cpu_baseline(torch, W, evt_oracle, cfgs, reps=9):
     """PyTorch fp32 eager evaluation of the same subgraphs on the host cores."""
     torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
     flops, secs = 0, 0.0
@@ -811,10 +811,11 @@ def main():
     dom_tflops = W.CONFIGS[dom].flops / (details[dom]["_ms"] * 1e-3) / 1e12
     cpu = None
     if not args.no_cpu_baseline:
-        v, cores, secs = cpu_baseline(torch, W, evt_oracle, vcfgs)
+        cpu_reps = 9
+        v, cores, secs = cpu_baseline(torch, W, evt_oracle, vcfgs, cpu_reps)
         cpu_model = next((ln.split(":", 1)[1].strip() for ln in open("/proc/cpuinfo") if ln.startswith("model name")), "")
         cpu = {"value": round(v, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port", "cpu": cpu_model,
-               "sample": f"configs {vcfgs} at full size, PyTorch fp32 eager on CPU, median of 3 after 1 warm-up "
+               "sample": f"configs {vcfgs} at full size, PyTorch fp32 eager on CPU, median of {cpu_reps} after 1 warm-up "
                          f"({secs:.2f} s per pass)"}
     # the published peak assumes 2.4 GHz; under this load the part clocks lower, so also relate the kernel to the
     # MFMA rate at the clock it was measured to run at
