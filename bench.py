@@ -547,6 +547,8 @@ def main_loop_traffic(tile):
     mfmas = (tile.bm // 32) * (tile.bn // 32) * (tile.bk // 16)
     dma_kib = (tile.bm + tile.bn) * tile.bk * 2 / 1024.0
     lds_kib = tile.wm * tile.wn * (tile.bm // tile.wm + tile.bn // tile.wn) * tile.bk * 2 / 1024.0
+    if tile.pipe >= 16:      # k-tiles split between the wave groups: wave tiles of twice the rows, half the depth each
+        lds_kib = tile.wm * tile.wn * (2 * tile.bm // tile.wm + tile.bn // tile.wn) * (tile.bk // 2) * 2 / 1024.0
     return mfmas, lds_kib, dma_kib
 
 

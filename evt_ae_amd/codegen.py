@@ -34,7 +34,10 @@ class TileConfig:
     # 3: ping-pong with one barrier per k-tile; 4 + flags: as 3 with 1 = the barrier inside group 0's MFMA phase,
     # 2 = group 0 issues its transfers between its LDS reads, 4 = group 1 as well (stages >= 3);
     # 12: one wave per SIMD (4 waves, stages >= 2): each wave interleaves the MFMAs of a k sub-step with the LDS
-    # reads of the next; 64 x 64 wave tiles on a 128 x 128 tile instead of the 64 x 32 of eight waves
+    # reads of the next; 64 x 64 wave tiles on a 128 x 128 tile instead of the 64 x 32 of eight waves;
+    # 16 + p (p = 2 ... 11): ping-pong loop p with each k-tile's depth split between the two wave groups, which
+    # then share loop wave tiles of twice the rows (a quarter fewer LDS reads per MFMA) and add their accumulators
+    # behind the loop
     pipe: int = 0
     # > 1: a workgroup computes this many consecutive tiles of a row block, the operand ring running on from one
     # into the next, and per-row reductions leave one partial per workgroup (ping-pong pipelines, no per-column
@@ -863,6 +866,13 @@ class Codegen:
         if t.pipe == 12 and (t.wm * t.wn != 4 or not t.dma or t.stages < 2 or t.walk > 1):
             raise NotImplementedError("the one-wave-per-SIMD loop needs four waves, the 16-byte transfers, two or more "
                                       "stages and one tile per workgroup")
+        if t.pipe >= 16:
+            mi, ni = t.bm // t.wm // 32, t.bn // t.wn // 32
+            if (not 18 <= t.pipe <= 27 or t.wm * t.wn != 8 or t.wm % 2 or not t.dma or t.stages < 2 or t.walk > 1 or t.bk % 32
+                    or 2 * mi * ni > 8 or 8 * mi * ni * 4096 > t.lds_bytes()):
+                raise NotImplementedError("split k-tiles need a ping-pong loop of eight waves in an even number of rows, "
+                                          "loop wave tiles of at most eight 32 x 32 blocks, one tile per workgroup and "
+                                          "LDS stages that hold one exchange of the accumulators")
         if t.walk > 1 and (t.pipe < 2 or not t.dma or ir.col_state or not sp.k_exact):
             raise NotImplementedError("a walk over tiles needs a ping-pong pipeline, K a multiple of bk and an epilogue "
                                       "without per-column reduction")

@@ -127,7 +127,7 @@ struct TileCtx {
     // ahead of the tile loop and carried through every main loop (see Mainloop::run)
     if constexpr (Cfg::WALK) asm volatile("" : "+v"(tid));
     lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = Cfg::epi_wave(__builtin_amdgcn_readfirstlane(tid >> 6));
     wm = wave / Cfg::WN; wn = wave % Cfg::WN;
     row_u = m0 + wm * Cfg::TM; row_l = 4 * (lane >> 5);
     col_u = n0 + wn * Cfg::TN;
@@ -1293,6 +1293,51 @@ EVT_DEV void run_epilogue(const GemmArgs& g, const typename Epi::Params& p, int 
   }
 }
 
+// Behind a main loop with split k-tiles (GemmCfg::KSPLIT): wave 4 g + p holds, for the loop's wave tile p, the sums
+// over its half of every k-tile -- 2 MI x NI blocks of accumulators.  It keeps blocks [g MI, (g + 1) MI), hands the
+// others to its partner 4 (1 - g) + p through LDS (64 lanes x 16 bytes per store: no bank conflicts), and adds what
+// the partner hands over: own half + other half, the same sum on whichever side it is formed.
+template <class Cfg, int KEEP>
+EVT_DEV void ksplit_exchange(float4* mine, const float4* theirs, f32x16 (&lacc)[Cfg::LMI][Cfg::LNI],
+                             f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  constexpr int SEND = Cfg::MI - KEEP;     // first block handed over: MI when the first MI are kept, else 0
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x16& x = lacc[SEND + mi][ni];
+        mine[((mi * Cfg::NI + ni) * 4 + q) * 64] = make_float4(x[4 * q], x[4 * q + 1], x[4 * q + 2], x[4 * q + 3]);
+      }
+  __syncthreads();
+#pragma unroll
+  for (int mi = 0; mi < Cfg::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < Cfg::NI; ++ni)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 y = theirs[((mi * Cfg::NI + ni) * 4 + q) * 64];
+        const f32x16& x = lacc[KEEP + mi][ni];
+        acc[mi][ni][4 * q] = x[4 * q] + y.x;
+        acc[mi][ni][4 * q + 1] = x[4 * q + 1] + y.y;
+        acc[mi][ni][4 * q + 2] = x[4 * q + 2] + y.z;
+        acc[mi][ni][4 * q + 3] = x[4 * q + 3] + y.w;
+      }
+}
+template <class Cfg>
+EVT_DEV void ksplit_reduce(char* smem, f32x16 (&lacc)[Cfg::LMI][Cfg::LNI], f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  constexpr int BYTES = Cfg::MI * Cfg::NI * 4096;      // what one wave hands over
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  float4* mine = (float4*)(smem + wave * BYTES) + lane;
+  const float4* theirs = (const float4*)(smem + (wave ^ 4) * BYTES) + lane;
+  __syncthreads();   // every wave has left the operand ring (its transfers were waited for inside the loop)
+  if ((wave >> 2) == 0) ksplit_exchange<Cfg, 0>(mine, theirs, lacc, acc);
+  else ksplit_exchange<Cfg, Cfg::MI>(mine, theirs, lacc, acc);
+  __syncthreads();   // the area is the epilogue's from here on
+}
+
 template <class Cfg, class Epi>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD) evt_gemm_kernel(GemmArgs g, typename Epi::Params p) {
   // a walking workgroup keeps one running state per row behind the operand stages
@@ -1335,7 +1380,13 @@ __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_WAVES_PER_SIMD) evt_gem
 #ifdef EVT_CLOCK_PROBE
     const uint64_t c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
 #endif
-    Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, split, smem, acc);
+    if constexpr (Cfg::KSPLIT) {
+      f32x16 loop_acc[Cfg::LMI][Cfg::LNI];
+      Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, split, smem, loop_acc);
+      ksplit_reduce<Cfg>(smem, loop_acc, acc);
+    } else {
+      Mainloop<Cfg>::run(g, batch, tm * Cfg::BM, tn * Cfg::BN, split, smem, acc);
+    }
     if (g.splits > 1) {
       if (!split_k_exchange<Cfg, Epi>(g, tile_id, split, smem, acc)) return;
     }

@@ -116,14 +116,20 @@ struct GemmCfg {
   //         sub-step with the LDS reads of the next, its transfers spread between them; one barrier per
   //         k-tile.  A 128 x 256 tile then has 64 x 128 wave tiles, a quarter less LDS read traffic per MFMA
   //         than the 64 x 64 wave tiles of eight waves.
-  static constexpr int PIPE = PIPE_;
-  static constexpr bool SOLO = PIPE_ == 12;
-  static constexpr bool PINGPONG = PIPE_ >= 2 && !SOLO;
+  // PIPE 16 + p (p = 2 ... 11): ping-pong loop p with every k-tile split between the two wave groups instead of
+  //         the output tile: waves w and w + 4 compute the same (2 TM) x TN block, one on the first half of each
+  //         k-tile's depth, the other on the second, and add their accumulators through LDS behind the loop, each
+  //         keeping TM of the rows.  A 128 x 256 tile then has 64 x 128 wave tiles in the loop -- three quarters
+  //         of the LDS reads per MFMA of the 64 x 64 ones -- and still two waves per SIMD to alternate.
+  static constexpr bool KSPLIT = PIPE_ >= 16;
+  static constexpr int PIPE = KSPLIT ? PIPE_ - 16 : PIPE_;
+  static constexpr bool SOLO = PIPE == 12;
+  static constexpr bool PINGPONG = PIPE >= 2 && !SOLO;
   static constexpr bool WALK = WALK_;
   // K is a multiple of BK in every launch (the host refuses others): see Operand
   static constexpr bool K_EXACT = K_EXACT_;
   static_assert(!WALK_ || K_EXACT_, "the carried-over operand ring has no code for a partial k-tile");
-  static constexpr int PP_FLAGS = PIPE_ >= 4 ? PIPE_ - 4 : 0;
+  static constexpr int PP_FLAGS = PIPE >= 4 ? PIPE - 4 : 0;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DMA = DMA_, BF16 = BF16_;
   static constexpr int STAGES = STAGES_, GROUP_M = GROUP_M_;
@@ -132,6 +138,19 @@ struct GemmCfg {
   static constexpr int TM = BM / WM, TN = BN / WN;
   static constexpr int MI = TM / 32, NI = TN / 32;
   static constexpr int KS = BK / 16;
+  // the wave tile of the main loop: as the epilogue's, or twice its rows with a split k-tile
+  static constexpr int LTM = KSPLIT ? 2 * TM : TM, LTN = TN;
+  static constexpr int LMI = LTM / 32, LNI = NI;
+  // which of the epilogue's wave tiles a wave owns.  With a split k-tile wave 4 g + p (group g, position p of the
+  // (WM / 2) x WN grid of loop tiles) keeps rows [g TM, (g + 1) TM) of loop tile p.
+  static EVT_DEV int epi_wave(int wave) {
+    if constexpr (KSPLIT) {
+      const int g = wave >> 2, p = wave & 3;
+      return ((p / WN) * 2 + g) * WN + p % WN;
+    } else {
+      return wave;
+    }
+  }
   // Layout of each operand tile in LDS: K-contiguous rows, or k-rows.
   static constexpr bool A_LDS_KC = A_KC || !DMA;
   static constexpr bool B_LDS_KC = B_KC || !DMA;
@@ -156,8 +175,12 @@ struct GemmCfg {
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be 32-aligned");
   static_assert(STAGES >= 1 && STAGES <= 8, "1..8 stages");
   static_assert(PIPE != 1 || (DMA && STAGES >= 3 && (BK / 16) % 2 == 0), "look-ahead needs DMA, >= 3 stages");
+  static_assert(!KSPLIT || (PINGPONG && !WALK_ && WM % 2 == 0 && KS % 2 == 0 && LMI * LNI <= 8 &&
+                            WM * WN * MI * NI * 4096 <= STAGES * (BM + BN) * BK * 2),
+                "split k-tiles: a ping-pong loop, an even number of wave rows, accumulators of 128 registers at most, "
+                "and LDS for one exchange of them");
   static_assert(!PINGPONG || (DMA && STAGES >= 2 && WM * WN == 8), "ping-pong needs DMA, >= 2 stages, 8 waves");
-  static_assert(PIPE >= 0 && PIPE <= 12, "unknown pipeline");
+  static_assert(PIPE >= 0 && PIPE <= 12 && PIPE_ <= 27, "unknown pipeline");
   static_assert(!SOLO || (DMA && STAGES >= 2 && WM * WN == 4 && (BK / 16) % 2 == 0), "one wave per SIMD: DMA, >= 2 stages, 4 waves");
   static_assert(!WALK || PINGPONG, "walking over tiles is built into the ping-pong loops");
   static_assert(!(PP_FLAGS & 4) || STAGES >= 3, "group 1 can only issue in its read phase with three or more stages");
@@ -444,13 +467,16 @@ struct FragReader {
       return r;
     }
   }
-  EVT_DEV void pin(Tile& t) const {
+  EVT_DEV void pin(Tile& t) const { pin_reads<0, NREADS>(t); }
+  // the destinations of reads [LO, HI) (numbered as issue_one numbers them)
+  template <int LO, int HI>
+  EVT_DEV void pin_reads(Tile& t) const {
     if constexpr (LDS_KC) {
 #pragma unroll
-      for (int i = 0; i < KSN * NFRAG; ++i) lds_pin(t.q[i]);
+      for (int i = LO; i < HI; ++i) lds_pin(t.q[i]);
     } else {
 #pragma unroll
-      for (int i = 0; i < 2 * KSN * NFRAG; ++i) lds_pin(t.h[i]);
+      for (int i = LO; i < HI; ++i) lds_pin(t.h[i]);
     }
   }
   EVT_DEV u32x4 frag(const Tile& t, int f, int ks) const {
@@ -543,59 +569,59 @@ template <class Cfg>
 struct Mainloop {
   using OpA = Operand<Cfg::BM, Cfg::BK, Cfg::A_KC, Cfg::DMA, Cfg::THREADS, 0, 0, Cfg::K_EXACT>;
   using OpB = Operand<Cfg::BN, Cfg::BK, Cfg::B_KC, Cfg::DMA, Cfg::THREADS,
-                      Cfg::INTERLEAVE ? Cfg::NI : 0, Cfg::TN, Cfg::K_EXACT>;
-  using RdA = FragReader<Cfg::BM, Cfg::BK, Cfg::A_LDS_KC, Cfg::MI>;
-  using RdB = FragReader<Cfg::BN, Cfg::BK, Cfg::B_LDS_KC, Cfg::NI, Cfg::REGROUP ? Cfg::NI : 0>;
+                      Cfg::INTERLEAVE ? Cfg::LNI : 0, Cfg::LTN, Cfg::K_EXACT>;
+  using RdA = FragReader<Cfg::BM, Cfg::BK, Cfg::A_LDS_KC, Cfg::LMI>;
+  using RdB = FragReader<Cfg::BN, Cfg::BK, Cfg::B_LDS_KC, Cfg::LNI, Cfg::REGROUP ? Cfg::LNI : 0>;
   static constexpr int LPS = OpA::NLOAD + OpB::NLOAD;   // DMA ops per thread per stage
 
   // One k-tile: KS sub-steps of MI x NI MFMAs.  Fragments of sub-step ks+1
   // are fetched from LDS into a second register set while the MFMAs of
   // sub-step ks issue.
   static EVT_DEV void compute(const char* lds, const RdA& ra, const RdB& rb,
-                              f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+                              f32x16 (&acc)[Cfg::LMI][Cfg::LNI]) {
     const char* la = lds;
     const char* lb = lds + Cfg::A_BYTES;
-    u32x4 af[2][Cfg::MI], bf[2][Cfg::NI];
+    u32x4 af[2][Cfg::LMI], bf[2][Cfg::LNI];
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi) af[0][mi] = ra.read(la, mi, 0);
+    for (int mi = 0; mi < Cfg::LMI; ++mi) af[0][mi] = ra.read(la, mi, 0);
 #pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni) bf[0][ni] = rb.read(lb, ni, 0);
+    for (int ni = 0; ni < Cfg::LNI; ++ni) bf[0][ni] = rb.read(lb, ni, 0);
 #pragma unroll
     for (int ks = 0; ks < Cfg::KS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
       if (ks + 1 < Cfg::KS) {
 #pragma unroll
-        for (int mi = 0; mi < Cfg::MI; ++mi) af[nxt][mi] = ra.read(la, mi, ks + 1);
+        for (int mi = 0; mi < Cfg::LMI; ++mi) af[nxt][mi] = ra.read(la, mi, ks + 1);
 #pragma unroll
-        for (int ni = 0; ni < Cfg::NI; ++ni) bf[nxt][ni] = rb.read(lb, ni, ks + 1);
+        for (int ni = 0; ni < Cfg::LNI; ++ni) bf[nxt][ni] = rb.read(lb, ni, ks + 1);
       }
 #pragma unroll
-      for (int mi = 0; mi < Cfg::MI; ++mi)
+      for (int mi = 0; mi < Cfg::LMI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < Cfg::NI; ++ni)
+        for (int ni = 0; ni < Cfg::LNI; ++ni)
           acc[mi][ni] = mfma32<Cfg::BF16>(af[cur][mi], bf[cur][ni], acc[mi][ni]);
     }
   }
 
   // ---- look-ahead pipeline (PIPE == 1) -------------------------------------
   struct Frags {
-    u32x4 a[Cfg::MI];
-    u32x4 b[Cfg::NI];
+    u32x4 a[Cfg::LMI];
+    u32x4 b[Cfg::LNI];
   };
-  static constexpr int NMFMA = Cfg::MI * Cfg::NI;
-  static constexpr int NDSREAD = (Cfg::A_LDS_KC ? Cfg::MI : 2 * Cfg::MI) + (Cfg::B_LDS_KC ? Cfg::NI : 2 * Cfg::NI);
+  static constexpr int NMFMA = Cfg::LMI * Cfg::LNI;
+  static constexpr int NDSREAD = (Cfg::A_LDS_KC ? Cfg::LMI : 2 * Cfg::LMI) + (Cfg::B_LDS_KC ? Cfg::LNI : 2 * Cfg::LNI);
 
   static EVT_DEV void load_frags(Frags& f, const char* lds, const RdA& ra, const RdB& rb, int ks) {
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi) f.a[mi] = ra.read(lds, mi, ks);
+    for (int mi = 0; mi < Cfg::LMI; ++mi) f.a[mi] = ra.read(lds, mi, ks);
 #pragma unroll
-    for (int ni = 0; ni < Cfg::NI; ++ni) f.b[ni] = rb.read(lds + Cfg::A_BYTES, ni, ks);
+    for (int ni = 0; ni < Cfg::LNI; ++ni) f.b[ni] = rb.read(lds + Cfg::A_BYTES, ni, ks);
   }
-  static EVT_DEV void mma(const Frags& f, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+  static EVT_DEV void mma(const Frags& f, f32x16 (&acc)[Cfg::LMI][Cfg::LNI]) {
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi)
+    for (int mi = 0; mi < Cfg::LMI; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < Cfg::NI; ++ni) acc[mi][ni] = mfma32<Cfg::BF16>(f.a[mi], f.b[ni], acc[mi][ni]);
+      for (int ni = 0; ni < Cfg::LNI; ++ni) acc[mi][ni] = mfma32<Cfg::BF16>(f.a[mi], f.b[ni], acc[mi][ni]);
   }
   // Scheduling directive for one sub-step of NMFMA MFMAs: NR LDS reads and NV
   // global->LDS transfers are placed between the MFMAs.  The compiler cannot
@@ -640,7 +666,7 @@ struct Mainloop {
   template <bool STEADY>
   static EVT_DEV void lookahead_iter(int kt, int KT, int& stage, const OpA& a, const OpB& b, const RdA& ra,
                                      const RdB& rb, char* smem, int wave, Frags (&f)[2],
-                                     f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+                                     f32x16 (&acc)[Cfg::LMI][Cfg::LNI]) {
     constexpr int S = Cfg::STAGES, D = S - 1;
     if constexpr (STEADY) {
       wait_tiles<D - 2>();            // tile kt+1 has landed (tiles kt+2.. may be in flight)
@@ -677,7 +703,7 @@ struct Mainloop {
   }
 
   static EVT_DEV void run_lookahead(const OpA& a, const OpB& b, const RdA& ra, const RdB& rb, char* smem,
-                                    int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+                                    int wave, int KT, f32x16 (&acc)[Cfg::LMI][Cfg::LNI]) {
     constexpr int S = Cfg::STAGES, D = S - 1;
 #pragma unroll
     for (int s = 0; s < D; ++s) {
@@ -725,17 +751,23 @@ struct Mainloop {
     typename RdA::Tile a;
     typename RdB::Tile b;
   };
-  static constexpr int PP_NM = Cfg::KS * Cfg::MI * Cfg::NI;   // MFMAs per C phase
+  // With a split k-tile (GemmCfg::KSPLIT) group KH reads and multiplies the k sub-steps [KH KS / 2, (KH + 1) KS / 2)
+  // of every tile (the reads of a tile are numbered k-sub-step major), on a wave tile of twice the rows.
+  static constexpr int PP_DIV = Cfg::KSPLIT ? 2 : 1;
+  static constexpr int PP_KS = Cfg::KS / PP_DIV;
+  static constexpr int PP_NM = PP_KS * Cfg::LMI * Cfg::LNI;   // MFMAs per C phase
+  static constexpr int PP_KH1 = Cfg::KSPLIT ? 1 : 0;          // the half of a k-tile that group 1 takes
   static constexpr bool PP_MIDC = (Cfg::PP_FLAGS & 1) != 0;
   static constexpr bool PP_G0_IN_R = (Cfg::PP_FLAGS & 2) != 0;
   static constexpr bool PP_G1_IN_R = (Cfg::PP_FLAGS & 4) != 0;
   static constexpr bool PP_G0_IN_C = !PP_G0_IN_R && Cfg::STAGES >= 3;
   static constexpr int PP_REST = PP_MIDC ? (PP_NM / 4 > 0 ? PP_NM / 4 : 1) : 0;   // group 0's MFMAs behind the barrier
-  static constexpr int PP_NR = RdA::NREADS + RdB::NREADS;   // LDS reads per R phase
+  static constexpr int PP_NRA = RdA::NREADS / PP_DIV, PP_NRB = RdB::NREADS / PP_DIV;
+  static constexpr int PP_NR = PP_NRA + PP_NRB;             // LDS reads per R phase
   // R phase: all fragments of the tile at `lds` are in registers on return.  With ISSUE the transfers of
   // k-tile `nk` into stage `ds` go between the reads (transfer c behind read number (c * PP_NR) / LPS): a wave
   // that waits for LDS anyway absorbs the pacing of the texture path, and the MFMA phases stay pure.
-  template <bool ISSUE>
+  template <bool ISSUE, int KH = 0>
   static EVT_DEV void pp_read(TileFrags& f, const char* lds, const RdA& ra, const RdB& rb,
                               const OpA& a, const OpB& b, int nk, char* ds, int wave) {
     typename OpA::DmaTile da;
@@ -747,8 +779,8 @@ struct Mainloop {
     const uint32_t la = lds_addr(lds), lb = lds_addr(lds + Cfg::A_BYTES);
 #pragma unroll
     for (int i = 0; i < PP_NR; ++i) {
-      if (i < RdA::NREADS) ra.issue_one(la, f.a, i);
-      else rb.issue_one(lb, f.b, i - RdA::NREADS);
+      if (i < PP_NRA) ra.issue_one(la, f.a, KH * PP_NRA + i);
+      else rb.issue_one(lb, f.b, KH * PP_NRB + i - PP_NRA);
       if constexpr (ISSUE) {
 #pragma unroll
         for (int c = 0; c < LPS; ++c) {
@@ -760,8 +792,8 @@ struct Mainloop {
       }
     }
     lds_wait_all();
-    ra.pin(f.a);
-    rb.pin(f.b);
+    ra.template pin_reads<KH * PP_NRA, (KH + 1) * PP_NRA>(f.a);
+    rb.template pin_reads<KH * PP_NRB, (KH + 1) * PP_NRB>(f.b);
   }
   // MFMAs [M, MEND) of a C phase, transfer c (of LPS) behind MFMA number (c * SPREAD) / LPS
   template <int M, int MEND, int SPREAD>
@@ -775,8 +807,8 @@ struct Mainloop {
   }
   // MFMAs [M0, M1) of the C phase (numbered k-sub-step major); with ISSUE the transfers of k-tile `nk` into
   // stage `ds` are spread between them
-  template <bool ISSUE, int PRIO, int M0, int M1>
-  static EVT_DEV void pp_mma(const TileFrags& f, const RdA& ra, const RdB& rb, f32x16 (&acc)[Cfg::MI][Cfg::NI],
+  template <bool ISSUE, int PRIO, int M0, int M1, int KH = 0>
+  static EVT_DEV void pp_mma(const TileFrags& f, const RdA& ra, const RdB& rb, f32x16 (&acc)[Cfg::LMI][Cfg::LNI],
                              const OpA& a, const OpB& b, int nk, char* ds, int wave) {
     static_assert(!ISSUE || M0 == 0, "transfers are spread from the first MFMA on");
     typename OpA::DmaTile da;
@@ -787,12 +819,13 @@ struct Mainloop {
     }
     __builtin_amdgcn_s_setprio(PRIO);
 #pragma unroll
-    for (int ks = 0; ks < Cfg::KS; ++ks) {
+    for (int kk = 0; kk < PP_KS; ++kk) {
+      const int ks = KH * PP_KS + kk;
 #pragma unroll
-      for (int mi = 0; mi < Cfg::MI; ++mi) {
+      for (int mi = 0; mi < Cfg::LMI; ++mi) {
 #pragma unroll
-        for (int ni = 0; ni < Cfg::NI; ++ni) {
-          const int m = (ks * Cfg::MI + mi) * Cfg::NI + ni;
+        for (int ni = 0; ni < Cfg::LNI; ++ni) {
+          const int m = (kk * Cfg::LMI + mi) * Cfg::LNI + ni;
           if (m < M0 || m >= M1) continue;
           acc[mi][ni] = mfma32<Cfg::BF16>(ra.frag(f.a, mi, ks), rb.frag(f.b, ni, ks), acc[mi][ni]);
           if constexpr (ISSUE) {
@@ -843,7 +876,7 @@ struct Mainloop {
   // make the compiler drain the DMA ring at every phase.
   static EVT_DEV void pp_barrier() { __builtin_amdgcn_s_barrier(); }
   static EVT_DEV void run_pingpong(const OpA& a, OpB& b, const RdA& ra, const RdB& rb, char* smem,
-                                   int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI],
+                                   int wave, int KT, f32x16 (&acc)[Cfg::LMI][Cfg::LNI],
                                    Walk& wk, bool more, int64_t b_step, int tid) {
     constexpr int S = Cfg::STAGES;
     static_assert((S - 1) * LPS < 64, "vmcnt is a 6-bit counter");
@@ -899,14 +932,14 @@ struct Mainloop {
         move_on(T);
         const int nk = fetch_index(T);
         char* ds = pp_refill_stage(stage, smem);
-        if (T > 0) pp_mma<!PP_G1_IN_R, 2, 0, PP_NM>(f, ra, rb, acc, a, b, nk, ds, wave);   // C(T-1)
+        if (T > 0) pp_mma<!PP_G1_IN_R, 2, 0, PP_NM, PP_KH1>(f, ra, rb, acc, a, b, nk, ds, wave);   // C(T-1)
         if constexpr (Cfg::PIPE == 2) pp_barrier();   // ends phase 2T
-        pp_read<PP_G1_IN_R>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, nk, ds, wave);
+        pp_read<PP_G1_IN_R, PP_KH1>(f, smem + stage * Cfg::STAGE_BYTES, ra, rb, a, b, nk, ds, wave);
         wait_tiles<S - 2>();        // my share of tile T+1 has landed
         pp_barrier();               // ends phase 2T+1
         stage = stage + 1 == S ? 0 : stage + 1;
       }
-      if (KT > 0) pp_mma<false, 2, 0, PP_NM>(f, ra, rb, acc, a, b, 0, smem, wave);   // C(KT-1)
+      if (KT > 0) pp_mma<false, 2, 0, PP_NM, PP_KH1>(f, ra, rb, acc, a, b, 0, smem, wave);   // C(KT-1)
     }
     if constexpr (Cfg::WALK) {
       wk.stage = stage;
@@ -933,7 +966,7 @@ struct Mainloop {
     typename RdB::Sub b;
   };
   static constexpr int SO_NR = RdA::SUB_READS + RdB::SUB_READS;   // LDS reads per sub-step
-  static constexpr int SO_NM = Cfg::MI * Cfg::NI;                 // MFMAs per sub-step
+  static constexpr int SO_NM = Cfg::LMI * Cfg::LNI;                 // MFMAs per sub-step
   static EVT_DEV void so_read_all(SubFrags& f, const char* lds, const RdA& ra, const RdB& rb, int ks) {
     const uint32_t la = lds_addr(lds), lb = lds_addr(lds + Cfg::A_BYTES);
 #pragma unroll
@@ -942,7 +975,7 @@ struct Mainloop {
     for (int i = 0; i < RdB::SUB_READS; ++i) rb.issue_sub(lb, f.b, ks, i);
   }
   static EVT_DEV void run_solo(const OpA& a, const OpB& b, const RdA& ra, const RdB& rb, char* smem,
-                               int wave, int KT, f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+                               int wave, int KT, f32x16 (&acc)[Cfg::LMI][Cfg::LNI]) {
     constexpr int S = Cfg::STAGES, KS = Cfg::KS;
     static_assert((S - 1) * LPS < 64, "vmcnt is a 6-bit counter");
     // transfers past the last k-tile read as zeros (or are switched off lane by lane) and land in stages nobody
@@ -982,7 +1015,7 @@ struct Mainloop {
         constexpr int PER = (LPS + KS - 2) / (KS - 1);           // transfers per sub-step
 #pragma unroll
         for (int m = 0; m < SO_NM; ++m) {
-          const int mi = m / Cfg::NI, ni = m % Cfg::NI;
+          const int mi = m / Cfg::LNI, ni = m % Cfg::LNI;
           acc[mi][ni] = mfma32<Cfg::BF16>(ra.frag_sub(now.a, mi), rb.frag_sub(now.b, ni), acc[mi][ni]);
           __builtin_amdgcn_sched_barrier(0);
           if (last && m == SO_BAR - 1) {
@@ -1017,13 +1050,13 @@ struct Mainloop {
   }
 
   static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, int split, char* smem,
-                          f32x16 (&acc)[Cfg::MI][Cfg::NI]) {
+                          f32x16 (&acc)[Cfg::LMI][Cfg::LNI]) {
     Walk wk;
     run(g, batch, m0, n0, split, smem, acc, wk, false);
   }
   // `wk`, `more`: see Walk (WALK kernels call this once per tile of the walk, `more` while another follows)
   static EVT_DEV void run(const GemmArgs& g, int batch, int m0, int n0, int split, char* smem,
-                          f32x16 (&acc)[Cfg::MI][Cfg::NI], Walk& wk, bool more) {
+                          f32x16 (&acc)[Cfg::LMI][Cfg::LNI], Walk& wk, bool more) {
     int tid = threadIdx.x;
     // In a walk this runs once per tile with the epilogue in between.  Everything below that depends only on
     // the thread index (transfer offsets, fragment addresses) would be hoisted out of the tile loop and then
@@ -1032,7 +1065,9 @@ struct Mainloop {
     if constexpr (Cfg::WALK) asm volatile("" : "+v"(tid));
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+    // with a split k-tile the two groups share the loop's wave tiles: position wave & 3 of a (WM / 2) x WN grid
+    const int wpos = Cfg::KSPLIT ? (wave & 3) : wave;
+    const int wm = wpos / Cfg::WN, wn = wpos % Cfg::WN;
 
     OpA a;
     OpB b;
@@ -1050,13 +1085,13 @@ struct Mainloop {
     const int Kw = (g.K - split * g.k_chunk < g.k_chunk) ? g.K - split * g.k_chunk : g.k_chunk;
     RdA ra;
     RdB rb;
-    ra.init(wm * Cfg::TM, lane);
-    rb.init(wn * Cfg::TN, lane);
+    ra.init(wm * Cfg::LTM, lane);
+    rb.init(wn * Cfg::LTN, lane);
 
 #pragma unroll
-    for (int mi = 0; mi < Cfg::MI; ++mi)
+    for (int mi = 0; mi < Cfg::LMI; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < Cfg::NI; ++ni)
+      for (int ni = 0; ni < Cfg::LNI; ++ni)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.f;
 

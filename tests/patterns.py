@@ -76,8 +76,9 @@ NO_ALLOC_TOO_BIG = (5, dict(M=1024, N=131072, K=64), (256, 256, 64, 4, 2, 2, Tru
 
 def pipeline_tiles():
     """Ping-pong main-loop variants (pipe 2: two barriers per k-tile, pipe 3:
-    one) and the one-wave-per-SIMD loop (pipe 12) on every stage count / k-depth /
-    wave grid they are instantiated with."""
+    one), the one-wave-per-SIMD loop (pipe 12) and the ping-pong loops with split
+    k-tiles (pipe 16 + p) on every stage count / k-depth / wave grid they are
+    instantiated with."""
     from evt_ae_amd.codegen import TileConfig
     return [TileConfig(256, 256, 64, 4, 2, 2, True, 4, 2), TileConfig(128, 256, 64, 2, 4, 3, True, 4, 2),
             TileConfig(256, 256, 32, 2, 4, 4, True, 4, 2), TileConfig(256, 128, 64, 4, 2, 3, True, 4, 3),
@@ -88,7 +89,11 @@ def pipeline_tiles():
             TileConfig(256, 256, 64, 2, 4, 2, True, 4, 7),
             # one wave per SIMD: three and four stages, square and oblong wave tiles, two stages
             TileConfig(128, 128, 64, 2, 2, 3, True, 4, 12), TileConfig(128, 128, 64, 2, 2, 4, True, 4, 12),
-            TileConfig(256, 128, 64, 2, 2, 3, True, 4, 12), TileConfig(128, 256, 64, 2, 2, 2, True, 4, 12)]
+            TileConfig(256, 128, 64, 2, 2, 3, True, 4, 12), TileConfig(128, 256, 64, 2, 2, 2, True, 4, 12),
+            # k-tiles split between the wave groups (pipe 16 + p): loop wave tiles 128 x 64 and 64 x 128, epilogue
+            # wave tiles of two row blocks and of one, three stages and two
+            TileConfig(128, 256, 64, 2, 4, 3, True, 4, 21), TileConfig(128, 256, 64, 4, 2, 3, True, 4, 26),
+            TileConfig(256, 128, 64, 4, 2, 3, True, 4, 27), TileConfig(128, 128, 64, 4, 2, 2, True, 4, 19)]
 
 
 # Workgroups that walk over several tiles of a row block (TileConfig.walk): (config, shapes, tile).  K is a
