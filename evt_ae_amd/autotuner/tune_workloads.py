@@ -186,7 +186,7 @@ SHORT_LIST = [(256, 256, 64, 4, 2, 2, 2), (256, 256, 64, 2, 4, 2, 3), (256, 256,
               (128, 128, 64, 2, 2, 3, 12), (128, 128, 64, 2, 2, 4, 12),
               (256, 256, 64, 2, 4, 2, 7), (256, 256, 64, 4, 2, 2, 7), (256, 128, 64, 4, 2, 3, 5), (128, 128, 64, 2, 2, 2, 12),
               (128, 64, 64, 4, 1, 2, 0), (128, 64, 64, 2, 2, 2, 0), (256, 64, 64, 4, 2, 2, 0), (64, 128, 64, 1, 4, 2, 0),
-              (128, 512, 64, 4, 2, 2, 0)]
+              (128, 512, 64, 4, 2, 2, 0), (128, 256, 64, 2, 4, 3, 27), (128, 256, 64, 2, 4, 3, 21), (256, 128, 64, 4, 2, 3, 21)]
 
 
 def main():
